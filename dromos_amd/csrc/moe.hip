@@ -1,0 +1,486 @@
+// Routing and the few-token routed experts: lx_moe_route, lx_moe_experts_decode, lx_moe_experts_decode_bf16
+// (contract: engine/cuda/kernels.h:203-209,495-507,606-611; CPU behaviour: engine/cpu/moe.cpp:163-329,343-397).
+//
+// Decode experts (T <= 8, top_k <= 8, so at most 64 (token, slot) pairs), two launches, no host round trip:
+//   gate/up   every workgroup sorts the pairs by expert in LDS (64 ids: a rank sort), takes one expert
+//             group and a block of intermediate rows, and streams gate row i and up row I + i of that
+//             expert once for all the group's tokens (stream_dot.h): inter[pair, i] = bf16(silu(g) * u).
+//   down      one workgroup per (block of output rows, token): for the token's slots in order it streams
+//             the expert's down rows against inter[pair] and adds w_k * c_k in slot order, so each output
+//             is written once and its bits depend on nothing but the token.
+#include "common.h"
+#include "stream_dot.h"
+
+namespace dro {
+namespace {
+
+constexpr int kThreads = 256;
+constexpr int kWaves = kThreads / kWave;
+constexpr int kMaxPairs = 64;
+
+// ---- routing ---------------------------------------------------------------------------------------------
+
+// One wavefront per token. E <= 4096 (a lane keeps one taken-bit per element it owns).
+__global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
+                                                         int32_t* __restrict__ ids, float* __restrict__ weights,
+                                                         float* __restrict__ entropy, float* __restrict__ confidence, int T,
+                                                         int E, int top_k) {
+  __shared__ float picked_logit[kWaves][64];
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
+  if (t >= T) return;
+  const float* row = logits + t * E;
+  float m = -INFINITY;
+  for (int i = lane; i < E; i += kWave) m = fmaxf(m, row[i]);
+  m = wave_max(m);
+  float z = 0.0f;
+  for (int i = lane; i < E; i += kWave) z += expf(row[i] - m);
+  z = wave_sum(z);
+  float h = 0.0f;
+  for (int i = lane; i < E; i += kWave) {
+    const float p = expf(row[i] - m) / z;
+    h -= p * logf(p > 1e-9f ? p : 1e-9f);
+  }
+  h = wave_sum(h);
+  if (lane == 0) {
+    entropy[t] = h;
+    confidence[t] = 1.0f / z;  // the largest probability is exp(0) / z
+  }
+  // top_k rounds of argmax over logit + bias (one f32 add); ties to the lower index; NaN is never greater.
+  uint64_t taken = 0;
+  for (int r = 0; r < top_k; ++r) {
+    float best = -INFINITY;
+    int best_i = E;
+    for (int i = lane, j = 0; i < E; i += kWave, ++j) {
+      if ((taken >> j) & 1u) continue;
+      const float v = row[i] + (bias ? bias[i] : 0.0f);
+      if (v > best || (v == best && i < best_i)) {
+        best = v;
+        best_i = i;
+      }
+    }
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) {
+      const float ov = __shfl_xor(best, off);
+      const int oi = __shfl_xor(best_i, off);
+      if (ov > best || (ov == best && oi < best_i)) {
+        best = ov;
+        best_i = oi;
+      }
+    }
+    if (best_i < E && (best_i & (kWave - 1)) == lane) taken |= 1ull << (best_i / kWave);
+    if (lane == 0) {
+      ids[t * top_k + r] = best_i;
+      picked_logit[wave][r] = best_i < E ? row[best_i] : NAN;
+    }
+  }
+  __builtin_amdgcn_wave_barrier();
+  __threadfence_block();
+  // Weights: softmax over the picks of their unbiased logits, summed in pick order.
+  float lmax = -INFINITY;
+  for (int r = 0; r < top_k; ++r) lmax = picked_logit[wave][r] > lmax ? picked_logit[wave][r] : lmax;
+  float esum = 0.0f;
+  for (int r = 0; r < top_k; ++r) esum += expf(picked_logit[wave][r] - lmax);
+  if (lane < top_k) weights[t * top_k + lane] = expf(picked_logit[wave][lane] - lmax) / esum;
+}
+
+// ---- decode experts ----------------------------------------------------------------------------------------
+
+struct Stack {
+  const uint8_t* data;
+  const uint8_t* scale;
+  const float* expert_global;
+  float global;
+};
+
+struct DecodeArgs {
+  const uint16_t* latent;  // bf16 [T, L]
+  const int32_t* ids;      // [T, top_k]
+  const float* weights;    // [T, top_k]
+  Stack gu, dn;
+  uint16_t* inter;  // bf16 [T * top_k, I]
+  float* out;       // f32 [T, L]
+  int T, L, I, top_k;
+};
+
+__device__ __forceinline__ float stack_factor(int type, const Stack& s, int e, int64_t row_in_stack) {
+  if (type == LX_W_INT8 || type == LX_W_FP8) return reinterpret_cast<const float*>(s.scale)[row_in_stack];
+  if (type == LX_W_NVFP4) return s.expert_global ? s.expert_global[e] : s.global;
+  return 1.0f;
+}
+
+// Sorts the P pairs by expert (stable) in LDS. order[g] = pair at sorted position g; returns through
+// group_begin / group_end the positions of group `slot` (the slot-th distinct expert in ascending id order),
+// and the number of groups. Run by the whole workgroup.
+__device__ __forceinline__ void group_pairs(const int32_t* ids, int P, int slot, int* s_ids, int* s_order, int* s_info) {
+  if (threadIdx.x < P) s_ids[threadIdx.x] = ids[threadIdx.x];
+  __syncthreads();
+  if (threadIdx.x < P) {
+    const int mine = s_ids[threadIdx.x];
+    int rank = 0;
+    for (int q = 0; q < P; ++q) {
+      const int other = s_ids[q];
+      rank += other < mine || (other == mine && q < static_cast<int>(threadIdx.x));
+    }
+    s_order[rank] = threadIdx.x;
+  }
+  __syncthreads();
+  if (threadIdx.x < kWave) {  // the first wavefront: P <= 64 positions
+    const int g = threadIdx.x;
+    const bool starts = g < P && (g == 0 || s_ids[s_order[g]] != s_ids[s_order[g - 1]]);
+    const uint64_t mask = __ballot(starts);
+    if (g == 0) {
+      const int groups = __popcll(mask);
+      int begin = P, end = P;
+      if (slot < groups) {
+        uint64_t mm = mask;
+        for (int i = 0; i < slot; ++i) mm &= mm - 1;  // drop the lower set bits
+        begin = __ffsll(static_cast<unsigned long long>(mm)) - 1;
+        mm &= mm - 1;
+        end = mm ? __ffsll(static_cast<unsigned long long>(mm)) - 1 : P;
+      }
+      s_info[0] = groups;
+      s_info[1] = begin;
+      s_info[2] = end;
+    }
+  }
+  __syncthreads();
+}
+
+// Intermediate rows [i_begin, i_end) of expert e for the cnt <= MT pairs at sorted positions first..: each
+// wavefront takes rows i = i_begin + wave, + kWaves, ...; the pair (gate row i, up row I + i) is its two
+// streamed rows. MT only sets how many activation rows share a pass; a row's arithmetic is the same for any MT.
+template <int F, int U, int MT>
+__device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, const float* lds, int e, int first, int cnt, const int* s_order,
+                                             int i_begin, int i_end) {
+  const int steps = steps_for<F>(a.L);
+  const int per_row = x_row_floats<F>(steps);
+  const int64_t rb = row_bytes<F>(a.L);
+  const int chunks = static_cast<int>(rb / 16);
+  const int64_t scale_row = F == LX_W_NVFP4 ? a.L / 16 : 0;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int64_t stack_row0 = static_cast<int64_t>(e) * 2 * a.I;
+  for (int i = i_begin + wave; i < i_end; i += kWaves) {
+    const int64_t gate_row = stack_row0 + i, up_row = stack_row0 + a.I + i;
+    const uint8_t* rows[2] = {a.gu.data + gate_row * rb, a.gu.data + up_row * rb};
+    const uint8_t* scales[2] = {a.gu.scale + gate_row * scale_row, a.gu.scale + up_row * scale_row};
+    float acc[MT][2];
+    stream_rows<F, MT, 2, U>(rows, scales, chunks, 0, steps, lds, per_row, acc);
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      acc[m][0] = wave_sum(acc[m][0]);
+      acc[m][1] = wave_sum(acc[m][1]);
+    }
+    if (lane == 0) {
+      const float sg = stack_factor(F, a.gu, e, gate_row), su = stack_factor(F, a.gu, e, up_row);
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        if (m < cnt) {
+          const float g = sg * acc[m][0], u = su * acc[m][1];
+          const int pair = s_order[first + m];
+          a.inter[static_cast<int64_t>(pair) * a.I + i] = f32_to_bf16_bits(silu(g) * u);
+        }
+      }
+    }
+  }
+}
+
+// grid = (row blocks, group slots); mt_cap (a power of two, the LDS image's rows) bounds a pass's pairs.
+template <int F, int U>
+__global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeArgs a, int mt_cap) {
+  extern __shared__ __align__(16) float lds[];
+  __shared__ int s_ids[kMaxPairs], s_order[kMaxPairs], s_info[4], s_rows[8];
+  const int P = a.T * a.top_k;
+  group_pairs(a.ids, P, blockIdx.y, s_ids, s_order, s_info);
+  if (static_cast<int>(blockIdx.y) >= s_info[0]) return;
+  const int begin = s_info[1], end = s_info[2];
+  const int e = s_ids[s_order[begin]];
+  const int steps = steps_for<F>(a.L);
+  const int rows_per_block = (a.I + gridDim.x - 1) / gridDim.x;
+  const int i_begin = blockIdx.x * rows_per_block, i_end = min(a.I, i_begin + rows_per_block);
+  // A group larger than the image (an expert repeated within a token) runs mt_cap pairs at a time.
+  for (int first = begin; first < end; first += mt_cap) {
+    const int cnt = min(mt_cap, end - first);
+    __syncthreads();
+    if (threadIdx.x < 8) s_rows[threadIdx.x] = threadIdx.x < cnt ? s_order[first + threadIdx.x] / a.top_k : 0;
+    __syncthreads();
+    if (cnt <= 1) {
+      stage_x<F, 1>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
+      __syncthreads();
+      gate_up_rows<F, U, 1>(a, lds, e, first, cnt, s_order, i_begin, i_end);
+    } else if (cnt <= 2) {
+      stage_x<F, 2>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
+      __syncthreads();
+      gate_up_rows<F, U, 2>(a, lds, e, first, cnt, s_order, i_begin, i_end);
+    } else if (cnt <= 4) {
+      stage_x<F, 4>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
+      __syncthreads();
+      gate_up_rows<F, U, 4>(a, lds, e, first, cnt, s_order, i_begin, i_end);
+    } else {
+      stage_x<F, 8>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
+      __syncthreads();
+      gate_up_rows<F, U, 8>(a, lds, e, first, cnt, s_order, i_begin, i_end);
+    }
+  }
+}
+
+// grid = (blocks of output rows, T). x = the token's top_k intermediate rows; slot k streams expert
+// ids[t, k]'s down rows. out[t, l] = w0 * c0 + sum_{k >= 1} w_k * c_k in slot order
+// (engine/cpu/moe.cpp:315-327), c_k = rowfactor * dot.
+template <int F, int U>
+__global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs a) {
+  extern __shared__ __align__(16) float lds[];
+  __shared__ int s_rows[8];
+  const int t = blockIdx.y;
+  const int steps = steps_for<F>(a.I);
+  const int per_row = x_row_floats<F>(steps);
+  const int64_t rb = row_bytes<F>(a.I);
+  const int chunks = static_cast<int>(rb / 16);
+  const int64_t scale_row = F == LX_W_NVFP4 ? a.I / 16 : 0;
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  if (threadIdx.x < 8) s_rows[threadIdx.x] = t * a.top_k + min(static_cast<int>(threadIdx.x), a.top_k - 1);
+  __syncthreads();
+  stage_x<F, 8>(lds, a.inter, LX_BF16, a.I, s_rows, a.top_k, a.I, steps);
+  __syncthreads();
+  constexpr int R = 2;
+  const int groups = (a.L + R - 1) / R;
+  const int groups_per_block = (groups + gridDim.x - 1) / gridDim.x;
+  const int g_begin = blockIdx.x * groups_per_block, g_end = min(groups, g_begin + groups_per_block);
+  for (int grp = g_begin + wave; grp < g_end; grp += kWaves) {
+    const int l0 = grp * R;
+    float sums[8][R];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+      if (k < a.top_k) {
+        const int e = a.ids[t * a.top_k + k];
+        const uint8_t* rows[R];
+        const uint8_t* scales[R];
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          const int64_t row = static_cast<int64_t>(e) * a.L + min(l0 + r, a.L - 1);
+          rows[r] = a.dn.data + row * rb;
+          scales[r] = a.dn.scale + row * scale_row;
+        }
+        float acc[1][R];
+        stream_rows<F, 1, R, U>(rows, scales, chunks, 0, steps, lds + k * per_row, per_row, acc);
+#pragma unroll
+        for (int r = 0; r < R; ++r) sums[k][r] = acc[0][r];
+      }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      float o = 0.0f;
+#pragma unroll
+      for (int k = 0; k < 8; ++k) {
+        if (k < a.top_k) {
+          const int e = a.ids[t * a.top_k + k];
+          const float c = stack_factor(F, a.dn, e, static_cast<int64_t>(e) * a.L + min(l0 + r, a.L - 1)) * wave_sum(sums[k][r]);
+          const float wc = a.weights[t * a.top_k + k] * c;
+          o = k == 0 ? wc : o + wc;
+        }
+      }
+      if (lane == 0 && l0 + r < a.L) a.out[static_cast<int64_t>(t) * a.L + l0 + r] = o;
+    }
+  }
+}
+
+// Rows whose bytes cannot be streamed 16 at a time (K not a multiple of the chunk, or a misaligned stack):
+// element-wise kernels with the same sums' structure (lane strides over k, one tree), one wavefront per output.
+__global__ void __launch_bounds__(kThreads) decode_gate_up_plain_kernel(const DecodeArgs a, int type) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * kWaves + threadIdx.x / kWave;  // (pair, i)
+  const int P = a.T * a.top_k;
+  if (item >= static_cast<int64_t>(P) * a.I) return;
+  const int pair = static_cast<int>(item / a.I), i = static_cast<int>(item % a.I);
+  const int e = a.ids[pair], t = pair / a.top_k;
+  const int64_t gate_row = static_cast<int64_t>(e) * 2 * a.I + i, up_row = gate_row + a.I;
+  float g = 0.0f, u = 0.0f;
+  for (int k = lane; k < a.L; k += kWave) {
+    const float x = bf16_bits_to_f32(a.latent[static_cast<int64_t>(t) * a.L + k]);
+    g = __builtin_fmaf(x, weight_element(type, a.gu.data, a.gu.scale, gate_row, k, a.L), g);
+    u = __builtin_fmaf(x, weight_element(type, a.gu.data, a.gu.scale, up_row, k, a.L), u);
+  }
+  g = stack_factor(type, a.gu, e, gate_row) * wave_sum(g);
+  u = stack_factor(type, a.gu, e, up_row) * wave_sum(u);
+  if (lane == 0) a.inter[static_cast<int64_t>(pair) * a.I + i] = f32_to_bf16_bits(silu(g) * u);
+}
+
+__global__ void __launch_bounds__(kThreads) decode_down_plain_kernel(const DecodeArgs a, int type) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * kWaves + threadIdx.x / kWave;  // (t, l)
+  if (item >= static_cast<int64_t>(a.T) * a.L) return;
+  const int t = static_cast<int>(item / a.L), l = static_cast<int>(item % a.L);
+  float o = 0.0f;
+  for (int k = 0; k < a.top_k; ++k) {
+    const int pair = t * a.top_k + k, e = a.ids[pair];
+    const int64_t row = static_cast<int64_t>(e) * a.L + l;
+    float s = 0.0f;
+    for (int j = lane; j < a.I; j += kWave)
+      s = __builtin_fmaf(bf16_bits_to_f32(a.inter[static_cast<int64_t>(pair) * a.I + j]),
+                         weight_element(type, a.dn.data, a.dn.scale, row, j, a.I), s);
+    const float wc = a.weights[pair] * (stack_factor(type, a.dn, e, row) * wave_sum(s));
+    o = k == 0 ? wc : o + wc;
+  }
+  if (lane == 0) a.out[item] = o;
+}
+
+template <int F>
+constexpr int moe_loads_in_flight() {
+  return F == LX_W_NVFP4 ? 2 : 4;
+}
+
+template <int F>
+bool streamable(const Stack& s, int64_t K, int max_rows) {
+  const int64_t rb = row_bytes<F>(K);
+  const int steps = steps_for<F>(K);
+  return rb % 16 == 0 && reinterpret_cast<uintptr_t>(s.data) % 16 == 0 &&
+         (F != LX_W_NVFP4 || reinterpret_cast<uintptr_t>(s.scale) % 2 == 0) &&
+         static_cast<int64_t>(max_rows) * x_row_floats<F>(steps) * 4 <= 128 * 1024;
+}
+
+template <class Kernel>
+void allow_big_lds(Kernel kernel, size_t lds) {
+  if (lds > 48 * 1024)
+    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                            160 * 1024 - 1024) != hipSuccess)
+      (void)hipGetLastError();
+}
+
+template <int F>
+int launch_gate_up(const DecodeArgs& a, hipStream_t s) {
+  const int P = a.T * a.top_k;
+  if (!streamable<F>(a.gu, a.L, 8)) {
+    const int64_t items = static_cast<int64_t>(P) * a.I;
+    hipLaunchKernelGGL(decode_gate_up_plain_kernel, dim3(static_cast<unsigned>((items + kWaves - 1) / kWaves)),
+                       dim3(kThreads), 0, s, a, F);
+    return status_of(hipGetLastError());
+  }
+  constexpr int U = moe_loads_in_flight<F>();
+  // With distinct experts per token a group has at most T pairs; the LDS image holds that many rows.
+  const int mt_cap = a.T <= 1 ? 1 : a.T <= 2 ? 2 : a.T <= 4 ? 4 : 8;
+  const size_t lds = sizeof(float) * mt_cap * x_row_floats<F>(steps_for<F>(a.L));
+  // Enough workgroups for two per compute unit when every slot holds a group; at least a wavefront's row each.
+  int blocks = (2 * compute_units() + P - 1) / P;
+  const int max_blocks = (a.I + kWaves - 1) / kWaves;
+  if (blocks > max_blocks) blocks = max_blocks;
+  if (blocks < 1) blocks = 1;
+  auto kernel = decode_gate_up_kernel<F, U>;
+  allow_big_lds(kernel, lds);
+  hipLaunchKernelGGL(kernel, dim3(blocks, P), dim3(kThreads), lds, s, a, mt_cap);
+  return status_of(hipGetLastError());
+}
+
+template <int F>
+int launch_down(const DecodeArgs& a, hipStream_t s) {
+  if (!streamable<F>(a.dn, a.I, 8)) {
+    const int64_t items = static_cast<int64_t>(a.T) * a.L;
+    hipLaunchKernelGGL(decode_down_plain_kernel, dim3(static_cast<unsigned>((items + kWaves - 1) / kWaves)), dim3(kThreads),
+                       0, s, a, F);
+    return status_of(hipGetLastError());
+  }
+  constexpr int U = moe_loads_in_flight<F>();
+  const size_t lds = sizeof(float) * 8 * x_row_floats<F>(steps_for<F>(a.I));
+  const int groups = (a.L + 1) / 2;
+  int blocks = (2 * compute_units() + a.T - 1) / a.T;
+  const int max_blocks = (groups + kWaves - 1) / kWaves;
+  if (blocks > max_blocks) blocks = max_blocks;
+  if (blocks < 1) blocks = 1;
+  auto kernel = decode_down_kernel<F, U>;
+  allow_big_lds(kernel, lds);
+  hipLaunchKernelGGL(kernel, dim3(blocks, a.T), dim3(kThreads), lds, s, a);
+  return status_of(hipGetLastError());
+}
+
+bool valid_stack(const lx_weight& w, int64_t K) {
+  if (!w.data) return false;
+  switch (w.type) {
+    case LX_W_BF16: return true;
+    case LX_W_INT8:
+    case LX_W_FP8: return w.scale != nullptr;
+    case LX_W_NVFP4: return w.scale != nullptr && K % 16 == 0;
+    default: return false;
+  }
+}
+
+Stack as_stack(const lx_weight& w) {
+  return Stack{static_cast<const uint8_t*>(w.data), static_cast<const uint8_t*>(w.scale), w.expert_global, w.global};
+}
+
+int64_t round256(int64_t b) { return (b + 255) / 256 * 256; }
+
+}  // namespace
+
+// The decode experts on two stacks of any formats; `inter` holds bf16 [T * top_k, I].
+int experts_decode(const void* latent, const int32_t* ids, const float* weights, const lx_weight& gate_up,
+                   const lx_weight& down, float* out, void* inter, int T, int L, int I, int top_k, hipStream_t s) {
+  DecodeArgs a{};
+  a.latent = static_cast<const uint16_t*>(latent);
+  a.ids = ids;
+  a.weights = weights;
+  a.gu = as_stack(gate_up);
+  a.dn = as_stack(down);
+  a.inter = static_cast<uint16_t*>(inter);
+  a.out = out;
+  a.T = T;
+  a.L = L;
+  a.I = I;
+  a.top_k = top_k;
+  int st;
+  switch (gate_up.type) {
+    case LX_W_BF16: st = launch_gate_up<LX_W_BF16>(a, s); break;
+    case LX_W_INT8: st = launch_gate_up<LX_W_INT8>(a, s); break;
+    case LX_W_FP8: st = launch_gate_up<LX_W_FP8>(a, s); break;
+    default: st = launch_gate_up<LX_W_NVFP4>(a, s); break;
+  }
+  if (st) return st;
+  switch (down.type) {
+    case LX_W_BF16: return launch_down<LX_W_BF16>(a, s);
+    case LX_W_INT8: return launch_down<LX_W_INT8>(a, s);
+    case LX_W_FP8: return launch_down<LX_W_FP8>(a, s);
+    default: return launch_down<LX_W_NVFP4>(a, s);
+  }
+}
+
+}  // namespace dro
+
+using namespace dro;
+
+extern "C" {
+
+int lx_moe_route(const float* logits, const float* selection_bias, int32_t* ids, float* weights, float* entropy,
+                 float* confidence, int T, int E, int top_k, void* stream) {
+  if (T <= 0) return kOk;
+  if (top_k < 1 || top_k > 64 || top_k > E || !logits || !ids || !weights || !entropy || !confidence) return fail(kInvalid);
+  if (E > 4096) return fail(kNotSupported);
+  hipLaunchKernelGGL(route_kernel, dim3((T + kWaves - 1) / kWaves), dim3(kThreads), 0, as_stream(stream), logits,
+                     selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  return status_of(hipGetLastError());
+}
+
+int lx_moe_experts_decode(const void* latent, const int32_t* ids, const float* weights, const lx_weight* gate_up,
+                          const lx_weight* down, float* out, void* workspace, int T, int L, int I, int top_k, void* stream) {
+  if (T <= 0) return kOk;
+  if (T > 8 || top_k > 8) return fail(kInvalid);
+  if (!latent || !ids || !weights || !out || L <= 0 || I <= 0 || top_k < 1) return fail(kInvalid);
+  if (!gate_up || !down || !workspace) return fail(kInvalid);
+  if (gate_up->type == LX_W_BF16X || down->type == LX_W_BF16X) return fail(kNotSupported);
+  if (!valid_stack(*gate_up, L) || !valid_stack(*down, I)) return fail(kInvalid);
+  return experts_decode(latent, ids, weights, *gate_up, *down, out, workspace, T, L, I, top_k, as_stream(stream));
+}
+
+int64_t lx_moe_decode_workspace_bytes(int T, int I, int top_k) {
+  if (T <= 0 || I <= 0 || top_k <= 0) return 0;
+  return round256(2 * static_cast<int64_t>(T) * top_k * I);
+}
+
+int64_t lx_moe_bf16x_workspace_bytes(int T, int I, int top_k) { return lx_moe_decode_workspace_bytes(T, I, top_k); }
+
+int lx_moe_experts_decode_bf16(const void* latent, const int32_t* ids, const float* weights, const void* gate_up,
+                               const void* down, float* out, void* workspace, int T, int L, int I, int top_k, void* stream) {
+  if (T <= 0) return kOk;
+  if (top_k > 8 || !workspace) return fail(kInvalid);
+  const lx_weight gu{LX_W_BF16, gate_up, nullptr, 1.0f, nullptr}, dn{LX_W_BF16, down, nullptr, 1.0f, nullptr};
+  return lx_moe_experts_decode(latent, ids, weights, &gu, &dn, out, workspace, T, L, I, top_k, stream);
+}
+
+}  // extern "C"

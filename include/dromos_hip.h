@@ -1,0 +1,191 @@
+/*
+ * libdromos_hip.so: the decode matrix-product path of Dromos on MI355X (gfx950), as a drop-in backend
+ * library. Every symbol below keeps the name, signature, argument meaning and status codes of the
+ * reference's backend ABI, so the engine's dispatch layer (engine/dispatch/dispatch.cpp:43-56,162-235,
+ * which already knows "libdromos_hip.so") binds it with dlsym and calls it unchanged. A symbol of the
+ * reference ABI that is not declared here is simply absent from the library: the dispatch stubs answer
+ * LX_ERR_NOT_SUPPORTED (801) for it (tools/gen_dispatch.py:168-184).
+ *
+ * Conventions (engine/cuda/kernels.h:1-4,27-38,294-302):
+ *   - return value: 0 ok, 1 invalid value, 2 out of memory, 801 not supported; checked before any launch
+ *   - tensor pointers are device pointers to row-major buffers owned by the caller; an lx_weight* is a
+ *     host pointer to a struct whose fields are device pointers
+ *   - `stream` is a hipStream_t (null = the default stream); calls are asynchronous, and the decode
+ *     calls neither allocate nor synchronise, so they can be captured in a graph
+ */
+#ifndef DROMOS_HIP_H_
+#define DROMOS_HIP_H_
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#ifndef LX_API
+#define LX_API __attribute__((visibility("default")))
+#endif
+
+/* engine/cuda/kernels.h:27 */
+typedef enum { LX_F32 = 0, LX_BF16 = 1 } lx_dtype;
+/* engine/cuda/kernels.h:243 (LX_W_BF16X is not on this path: calls with it answer 801) */
+typedef enum { LX_W_BF16 = 0, LX_W_INT8 = 1, LX_W_FP8 = 2, LX_W_NVFP4 = 3, LX_W_BF16X = 4 } lx_wtype;
+/* engine/cuda/kernels.h:431 */
+typedef enum { LX_MATH_BF16 = 0, LX_MATH_INT8 = 1, LX_MATH_FP8 = 2, LX_MATH_FP4 = 3 } lx_math;
+/* engine/cuda/kernels.h:302-306 */
+#define LX_ERR_NOT_SUPPORTED 801
+typedef enum { LX_BACKEND_CUDA = 0, LX_BACKEND_HIP = 1, LX_BACKEND_METAL = 2, LX_BACKEND_CPU = 3 } lx_backend;
+typedef enum { LX_COPY_H2D = 0, LX_COPY_D2H = 1, LX_COPY_D2D = 2, LX_COPY_DEFAULT = 3 } lx_copy_kind;
+/* engine/cuda/tunable.h:27-32 */
+#define LX_ERR_TUNE_REJECTED 802
+#define LX_ERR_TUNE_VARIANT 803
+
+/*
+ * One weight in one format, row-major [N, K], K contiguous (engine/cuda/kernels.h:383-417):
+ *   LX_W_BF16   data bf16 [N, K]
+ *   LX_W_INT8   data int8 [N, K], scale f32 [N]            w = q * scale[n]
+ *   LX_W_FP8    data e4m3fn [N, K], scale f32 [N]          w = fp8 * scale[n]
+ *   LX_W_NVFP4  data u8 [N, K/2] (low nibble = even k), scale e4m3 [N, K/16], global f32
+ *                                                          w = e2m1 * scale[n, k/16] * global
+ * A stack of experts is [E, N, K] laid out expert after expert (scales likewise); an NVFP4 stack may
+ * carry one global per expert in expert_global (f32 [E] on the device, null = `global` for all).
+ */
+typedef struct {
+  lx_wtype type;
+  const void* data;
+  const void* scale;
+  float global;
+  const float* expert_global;
+} lx_weight;
+
+/* ---- decode GEMV, M <= 8 (replaces engine/cuda/kernels.h:235-246, 433-438, 594-596) ---------------
+ *   y[m, n] = alpha * (rowfactor[n] * sum_k x[m, k] * w[n, k] + bias[n]) + beta * y[m, n]
+ * x [M, K] f32 or bf16 (row stride ld_x elements); bias [N] f32 / bf16 or null; y [M, N] f32 / bf16
+ * (row stride ld_y), read only when beta != 0. Weight-only: weights are expanded exactly in registers,
+ * sums are f32, deterministic, and a row's bits do not depend on M or on the other rows.
+ * M > 8 or bad arguments -> 1; M == 0 or N == 0 -> 0 with nothing touched. */
+LX_API int lx_gemv(const void* x, lx_dtype x_dtype, int ld_x, const void* w, lx_wtype w_type, const float* w_scale,
+                   const void* bias, lx_dtype bias_dtype, void* y, lx_dtype y_dtype, int ld_y, int M, int N, int K,
+                   float alpha, float beta, void* stream);
+LX_API int lx_gemv_w(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, const void* bias,
+                     lx_dtype bias_dtype, void* y, lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha,
+                     float beta, void* stream);
+LX_API int lx_gemv_decode_bf16(const void* x, lx_dtype x_dtype, int ld_x, const void* w, const void* bias,
+                               lx_dtype bias_dtype, void* y, lx_dtype y_dtype, int ld_y, int M, int N, int K,
+                               float alpha, float beta, void* stream);
+
+/* ---- batched decode products (replaces engine/cuda/kernels.h:440-451 and 453-477) ----------------
+ * lx_gemm_w: any M, the same product with `math`. This library runs LX_MATH_BF16 (activations rounded
+ * to bf16, weights of any format expanded exactly to bf16, f32 sums on the matrix cores); the
+ * low-precision maths answer 801. The workspace is not used by LX_MATH_BF16 (may be null).
+ * lx_gemm_skinny: bf16 x, up to 64 rows per pass, every format, with the reduction-order contract of
+ * engine/cuda/kernels.h:457-474: the K split depends on (N, K) only, never on M, so a row's bits do not
+ * depend on the batch. With the environment variable LX_BATCH_INVARIANT set (non-empty, not starting
+ * with '0'; read on every call, engine/cuda/common.cuh:66-73) lx_gemv_w with bf16 x and lx_gemm_w run
+ * this same kernel, so a row's bits are the same for every row count from 1 up. */
+LX_API int lx_gemm_w(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, lx_math math, const void* bias,
+                     lx_dtype bias_dtype, void* y, lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha,
+                     float beta, void* workspace, void* stream);
+LX_API int64_t lx_gemm_workspace_bytes(int M, int K, lx_math math);
+LX_API int lx_gemm_skinny(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, const void* bias,
+                          lx_dtype bias_dtype, void* y, lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha,
+                          float beta, void* stream);
+
+/* ---- weight quantisers (replaces engine/cuda/kernels.h:248-251, 513-523) -------------------------
+ * Round-to-nearest-even, IEEE f32 divisions, bytes identical to the reference's CPU quantisers
+ * (engine/cpu/quant.cpp:66-140). NVFP4 writes the tensor's global back to out->global (synchronises
+ * the stream once: load time only). lx_dequantize_weight: out[n, k] = bf16(element * row factor). */
+LX_API int lx_quantize_w8(const void* w, int8_t* q, float* scale, int64_t rows, int cols, void* stream);
+LX_API int lx_quantize_weight(const void* w, lx_weight* out, int64_t rows, int cols, void* stream);
+LX_API int lx_dequantize_weight(const lx_weight* w, void* out, int64_t rows, int cols, void* stream);
+
+/* ---- routing and routed experts (replaces engine/cuda/kernels.h:203-209, 220-225, 495-511, 606-611)
+ * lx_moe_route: per row of f32 logits [T, E]: entropy and confidence of the softmax, ids = top_k by
+ * logit + selection_bias (ties to the lower index), weights = softmax of the picked unbiased logits.
+ * Experts: out[t, :] = sum_k weights[t, k] * down[e] @ bf16(silu(gate[e] @ x) * (up[e] @ x)), e =
+ * ids[t, k]; latent bf16 [T, L]; gate_up [E, 2I, L] (gate rows first); down [E, L, I]; out f32 [T, L],
+ * written once; the k terms are added in slot order. The pairs are grouped by expert on the device
+ * (counting sort + prefix-summed offset table in the workspace): no host round trip.
+ *   lx_moe_experts_decode   T <= 8, top_k <= 8, weight-only f32 math
+ *   lx_moe_experts_grouped  any T, LX_MATH_BF16 on the matrix cores (other maths: 801), E <= 1024
+ *   lx_moe_experts / lx_moe_experts_decode_bf16   the bf16-stack forms of the two */
+LX_API int lx_moe_route(const float* logits, const float* selection_bias, int32_t* ids, float* weights,
+                        float* entropy, float* confidence, int T, int E, int top_k, void* stream);
+LX_API int lx_moe_experts(const void* latent, const int32_t* ids, const float* weights, const void* gate_up,
+                          const void* down, float* out, int T, int L, int I, int top_k, void* stream);
+LX_API int lx_moe_experts_decode(const void* latent, const int32_t* ids, const float* weights,
+                                 const lx_weight* gate_up, const lx_weight* down, float* out, void* workspace, int T,
+                                 int L, int I, int top_k, void* stream);
+LX_API int64_t lx_moe_decode_workspace_bytes(int T, int I, int top_k);
+LX_API int lx_moe_experts_decode_bf16(const void* latent, const int32_t* ids, const float* weights,
+                                      const void* gate_up, const void* down, float* out, void* workspace, int T,
+                                      int L, int I, int top_k, void* stream);
+LX_API int64_t lx_moe_bf16x_workspace_bytes(int T, int I, int top_k);
+LX_API int lx_moe_experts_grouped(const void* latent, const int32_t* ids, const float* weights,
+                                  const lx_weight* gate_up, const lx_weight* down, lx_math math, float* out,
+                                  void* workspace, int T, int L, int I, int E, int top_k, void* stream);
+LX_API int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int top_k, lx_math math);
+
+/* ---- runtime (replaces engine/cuda/kernels.h:308-381 on the HIP runtime) --------------------------- */
+typedef struct {
+  char name[256];
+  int cc_major, cc_minor;
+  int sms;
+  int64_t l2_bytes;
+  int64_t mem_clock_khz;
+  int bus_bits;
+  int driver_version, runtime_version;
+  int64_t l1_bytes, l3_bytes;
+  int64_t read_bandwidth;
+  char isa[192];
+  int native_math;
+} lx_device_props;
+
+LX_API int lx_rt_backend(void); /* LX_BACKEND_HIP */
+LX_API int lx_rt_device_count(void);
+LX_API int lx_rt_set_device(int ordinal);
+LX_API int lx_rt_alloc(void** ptr, int64_t bytes); /* zeroed */
+LX_API int lx_rt_free(void* ptr);
+LX_API int lx_rt_host_alloc(void** ptr, int64_t bytes);
+LX_API int lx_rt_host_free(void* ptr);
+LX_API int lx_rt_memset(void* ptr, int value, int64_t bytes, void* stream);
+LX_API int lx_rt_copy(void* dst, const void* src, int64_t bytes, lx_copy_kind kind, void* stream);
+LX_API int lx_rt_stream_create(void** stream);
+LX_API int lx_rt_stream_destroy(void* stream);
+LX_API int lx_rt_stream_sync(void* stream);
+LX_API int lx_rt_event_create(void** event);
+LX_API int lx_rt_event_create_timed(void** event);
+LX_API int lx_rt_event_destroy(void* event);
+LX_API int lx_rt_event_record(void* event, void* stream);
+LX_API int lx_rt_event_sync(void* event);
+LX_API int lx_rt_event_elapsed(void* start, void* stop, float* ms);
+LX_API int lx_rt_capture_begin(void* stream);
+LX_API int lx_rt_capture_end(void* stream, void** graph);
+LX_API int lx_rt_graph_launch(void* graph, void* stream);
+LX_API int lx_rt_graph_destroy(void* graph);
+LX_API int lx_rt_device_sync(void);
+LX_API int lx_rt_last_error(void); /* and clears it */
+LX_API const char* lx_rt_error_string(int status);
+LX_API int lx_rt_is_host_memory(const void* ptr);
+LX_API int lx_rt_device_props(int ordinal, lx_device_props* props);
+LX_API int lx_rt_mem_info(int64_t* free_bytes, int64_t* total_bytes);
+LX_API int lx_bandwidth_probe(int64_t bytes, int reps, double* read_gbps, double* spec_gbps, void* stream);
+
+/* ---- architecture and kernel variants (replaces engine/cuda/tunable.h:37-55) -----------------------
+ * lx_arch is 95 on gfx950. The GEMV registers its variants under gemv_w_<format>; a variant's name starts
+ * with s<S>, its K split, and lx_tune_set admits a variant for a shape only when its split is the
+ * shape's own (so the rows' bits never depend on the table). */
+LX_API int lx_arch(void);
+LX_API int lx_set_arch_override(int arch);
+LX_API int lx_tune_get(const char* kernel, int M, int N, int K);
+LX_API int lx_tune_set(const char* kernel, int M, int N, int K, int variant);
+LX_API int lx_tune_force(const char* kernel, int M, int N, int K, int variant);
+LX_API void lx_tune_clear(void);
+LX_API int lx_tune_kernels(const char** names, int capacity);
+LX_API int lx_tune_variants(const char* kernel);
+LX_API const char* lx_tune_variant_name(const char* kernel, int variant);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* DROMOS_HIP_H_ */

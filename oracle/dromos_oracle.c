@@ -1,0 +1,691 @@
+/*
+ * CPU oracle for the decode matrix-product path. TEST INFRASTRUCTURE ONLY.
+ *
+ * This file restates, in plain scalar C, the arithmetic of the reference's CPU backend for the
+ * decode products: number formats, weight quantisers, the weight-streaming GEMV / skinny GEMM and the
+ * routed experts. It is the checker that the GPU library's results are compared with. Nothing that
+ * ships may call it: only the tests, the smoke check and the bench's cpu_baseline leg load it.
+ *
+ * It exports the same lx_* C ABI as the GPU library (include/dromos_hip.h), on host pointers, so one
+ * test harness drives the GPU library, this oracle and (where it was built) the reference's own CPU
+ * backend. Every function cites the reference file:line whose behaviour it follows. The code is
+ * single-threaded unless built with -fopenmp (the loops over output rows carry pragmas).
+ *
+ * Parity status of each function (what pins it besides the compiled reference backend):
+ *   bf16 / e4m3 / e2m1 codecs        pinned: exhaustive tables against torch.float8_e4m3fn and closed forms
+ *   lx_quantize_w8 / _weight         pinned: known-answer ties/zero rows + torch IEEE-division references
+ *   lx_dequantize_weight             pinned: closed-form dense values from the stored bytes
+ *   lx_gemv* / lx_gemm_w / _skinny   pinned: float64 x @ W^T on the decoded values
+ *   lx_moe_route                     pinned: stable sort of -(logit + bias) + float64 softmax, tie cases
+ *   lx_moe_experts*                  pinned: float64 experts with the bf16-rounded intermediate
+ */
+#include <math.h>
+#include <stdint.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define ORC_API __attribute__((visibility("default")))
+
+enum { LX_F32 = 0, LX_BF16 = 1 };
+enum { LX_W_BF16 = 0, LX_W_INT8 = 1, LX_W_FP8 = 2, LX_W_NVFP4 = 3 };
+enum { LX_MATH_BF16 = 0, LX_MATH_INT8 = 1, LX_MATH_FP8 = 2, LX_MATH_FP4 = 3 };
+enum { ORC_OK = 0, ORC_INVALID = 1, ORC_NOMEM = 2, ORC_UNSUPPORTED = 801 };
+
+/* The weight descriptor of engine/cuda/kernels.h:411-417. */
+typedef struct {
+  int type;
+  const void* data;
+  const void* scale;
+  float global;
+  const float* expert_global;
+} lx_weight;
+
+static __thread int g_last_error = 0;
+static int fail(int status) {
+  g_last_error = status;
+  return status;
+}
+
+/* ---- number formats -------------------------------------------------------------------------- */
+
+static float bits_to_f32(uint32_t u) {
+  float f;
+  memcpy(&f, &u, 4);
+  return f;
+}
+static uint32_t f32_to_bits(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  return u;
+}
+
+/* bf16 is the top half of an f32 (engine/cpu/cpu.h:44). */
+static float bf16_value(uint16_t h) { return bits_to_f32((uint32_t)h << 16); }
+
+/* f32 -> bf16, nearest even; a NaN keeps its sign and gets a quiet payload bit (engine/cpu/cpu.h:47-52). */
+static uint16_t bf16_round(float f) {
+  uint32_t u = f32_to_bits(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (uint16_t)((u >> 16) | 0x0040u);
+  uint32_t lsb = (u >> 16) & 1u;
+  u += 0x7fffu + lsb;
+  return (uint16_t)(u >> 16);
+}
+
+/* e4m3 "fn": bias 7, no infinities, subnormals m * 2^-9 (engine/cpu/quant.cpp:12-18). The two NaN
+ * codes 0x7f / 0xff decode by the same formula (to +-480), as the reference's table does
+ * (engine/cpu/kern/simd.h:77-85); no valid weight holds them. */
+ORC_API float orc_e4m3_to_f32(uint8_t b) {
+  int e = (b >> 3) & 15, m = b & 7;
+  float v = e == 0 ? ldexpf((float)m, -9) : ldexpf(1.0f + (float)m / 8.0f, e - 7);
+  return (b & 0x80) ? -v : v;
+}
+
+/* f32 -> e4m3, nearest even, saturating at 448, NaN -> 0x7f with the sign (engine/cpu/quant.cpp:20-39). */
+ORC_API uint8_t orc_f32_to_e4m3(float f) {
+  uint32_t u = f32_to_bits(f);
+  uint8_t sign = (uint8_t)((u >> 24) & 0x80u);
+  u &= 0x7fffffffu;
+  if (u > 0x7f800000u) return sign | 0x7f;
+  float a = bits_to_f32(u);
+  if (a >= 448.0f) return sign | 0x7e;
+  if (a < 0.015625f) { /* below 2^-6: the subnormal grid, steps of 2^-9; 8 steps is the first normal */
+    int steps = (int)rintf(a * 512.0f);
+    return sign | (uint8_t)steps;
+  }
+  /* keep 3 mantissa bits: add half of the dropped field, plus the kept lsb for ties to even */
+  u += 0x7ffffu + ((u >> 20) & 1u);
+  int e = (int)(u >> 23) - 127 + 7;
+  int m = (int)((u >> 20) & 7u);
+  if (e > 15 || (e == 15 && m == 7)) return sign | 0x7e;
+  return sign | (uint8_t)(e << 3) | (uint8_t)m;
+}
+
+static const float kE2m1[8] = {0.0f, 0.5f, 1.0f, 1.5f, 2.0f, 3.0f, 4.0f, 6.0f};
+
+/* e2m1 code (bit 3 = sign) -> f32 (engine/cpu/quant.cpp:41-45). */
+ORC_API float orc_e2m1_to_f32(uint32_t code) {
+  float v = kE2m1[code & 7u];
+  return (code & 8u) ? -v : v;
+}
+
+/* Nearest e2m1 code: ties go to the even code, saturates at 6, zero carries no sign
+ * (engine/cpu/quant.cpp:47-56). */
+ORC_API uint32_t orc_f32_to_e2m1(float x) {
+  float mag = fabsf(x);
+  if (mag > 6.0f) mag = 6.0f;
+  uint32_t idx = 0;
+  for (int i = 0; i < 7; ++i) {
+    float mid = 0.5f * (kE2m1[i] + kE2m1[i + 1]);
+    if (mag > mid) idx = (uint32_t)i + 1;
+    else if (mag == mid) { idx = (i & 1) ? (uint32_t)i + 1 : (uint32_t)i; break; }
+    else break;
+  }
+  /* NaN compares false everywhere: idx stays 0, as in the reference */
+  return idx | ((x < 0.0f && idx > 0) ? 8u : 0u);
+}
+
+static float load_f32(const void* p, int dtype, int64_t i) {
+  return dtype == LX_BF16 ? bf16_value(((const uint16_t*)p)[i]) : ((const float*)p)[i];
+}
+static void store_f32(void* p, int dtype, int64_t i, float v) {
+  if (dtype == LX_BF16) ((uint16_t*)p)[i] = bf16_round(v);
+  else ((float*)p)[i] = v;
+}
+static int dtype_ok(int d) { return d == LX_F32 || d == LX_BF16; }
+
+/* ---- weight quantisers (engine/cpu/quant.cpp:66-140, contract engine/cuda/kernels.h:248-251,513-518) ---- */
+
+static float row_amax(const uint16_t* w, int64_t cols) {
+  float m = 0.0f;
+  for (int64_t c = 0; c < cols; ++c) m = fmaxf(m, fabsf(bf16_value(w[c])));
+  return m;
+}
+
+static void quant_int8(const uint16_t* w, int8_t* q, float* scale, int64_t rows, int64_t cols) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const uint16_t* src = w + r * cols;
+    float amax = row_amax(src, cols);
+    float s = amax > 0.0f ? amax / 127.0f : 1.0f; /* IEEE division; a zero row keeps scale 1 */
+    scale[r] = s;
+    for (int64_t c = 0; c < cols; ++c) {
+      float v = rintf(bf16_value(src[c]) / s);
+      v = fminf(fmaxf(v, -127.0f), 127.0f);
+      q[r * cols + c] = (int8_t)(int)v;
+    }
+  }
+}
+
+static void quant_fp8(const uint16_t* w, uint8_t* q, float* scale, int64_t rows, int64_t cols) {
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    const uint16_t* src = w + r * cols;
+    float amax = row_amax(src, cols);
+    float s = amax > 0.0f ? amax / 448.0f : 1.0f;
+    scale[r] = s;
+    for (int64_t c = 0; c < cols; ++c) {
+      float v = bf16_value(src[c]) / s;
+      q[r * cols + c] = orc_f32_to_e4m3(fminf(fmaxf(v, -448.0f), 448.0f));
+    }
+  }
+}
+
+static void quant_nvfp4(const uint16_t* w, uint8_t* q, uint8_t* scale, float* global_out, int64_t rows, int64_t cols) {
+  float amax = 0.0f;
+  for (int64_t r = 0; r < rows; ++r) amax = fmaxf(amax, row_amax(w + r * cols, cols));
+  const float global = amax / 2688.0f; /* 448 * 6 */
+  *global_out = global;
+  const int64_t blocks = cols / 16;
+#pragma omp parallel for schedule(static)
+  for (int64_t r = 0; r < rows; ++r) {
+    for (int64_t b = 0; b < blocks; ++b) {
+      float v[16], bmax = 0.0f;
+      for (int j = 0; j < 16; ++j) {
+        v[j] = bf16_value(w[r * cols + 16 * b + j]);
+        bmax = fmaxf(bmax, fabsf(v[j]));
+      }
+      uint8_t sb = orc_f32_to_e4m3(bmax / (6.0f * global));
+      scale[r * blocks + b] = sb;
+      float eff = orc_e4m3_to_f32(sb) * global;
+      for (int p = 0; p < 8; ++p) {
+        uint32_t lo = 0, hi = 0;
+        if (eff > 0.0f) {
+          lo = orc_f32_to_e2m1(v[2 * p] / eff);
+          hi = orc_f32_to_e2m1(v[2 * p + 1] / eff);
+        }
+        q[r * (cols / 2) + 8 * b + p] = (uint8_t)(lo | (hi << 4)); /* even k in the low nibble */
+      }
+    }
+  }
+}
+
+ORC_API int lx_quantize_w8(const void* w, int8_t* q, float* scale, int64_t rows, int cols, void* stream) {
+  (void)stream;
+  if (rows <= 0) return ORC_OK;
+  if (cols <= 0 || !w || !q || !scale) return fail(ORC_INVALID);
+  quant_int8((const uint16_t*)w, q, scale, rows, cols);
+  return ORC_OK;
+}
+
+ORC_API int lx_quantize_weight(const void* w, lx_weight* out, int64_t rows, int cols, void* stream) {
+  (void)stream;
+  if (!out || !w) return fail(ORC_INVALID);
+  if (rows <= 0) return ORC_OK;
+  if (cols <= 0) return fail(ORC_INVALID);
+  void* data = (void*)out->data;
+  void* scale = (void*)out->scale;
+  switch (out->type) {
+    case LX_W_INT8:
+      if (!data || !scale) return fail(ORC_INVALID);
+      quant_int8((const uint16_t*)w, (int8_t*)data, (float*)scale, rows, cols);
+      return ORC_OK;
+    case LX_W_FP8:
+      if (!data || !scale) return fail(ORC_INVALID);
+      quant_fp8((const uint16_t*)w, (uint8_t*)data, (float*)scale, rows, cols);
+      return ORC_OK;
+    case LX_W_NVFP4:
+      if (!data || !scale || cols % 16 != 0) return fail(ORC_INVALID);
+      quant_nvfp4((const uint16_t*)w, (uint8_t*)data, (uint8_t*)scale, &out->global, rows, cols);
+      return ORC_OK;
+    default: return fail(ORC_INVALID); /* bf16 is its own quantisation */
+  }
+}
+
+/* Element (n, k) of an [N, K] weight, exact, without its row factor (engine/cpu/quant.cpp:143-154). */
+static float weight_element(int type, const void* data, const void* scale, int64_t n, int64_t k, int64_t K) {
+  switch (type) {
+    case LX_W_BF16: return bf16_value(((const uint16_t*)data)[n * K + k]);
+    case LX_W_INT8: return (float)((const int8_t*)data)[n * K + k];
+    case LX_W_FP8: return orc_e4m3_to_f32(((const uint8_t*)data)[n * K + k]);
+    default: {
+      uint8_t byte = ((const uint8_t*)data)[n * (K / 2) + k / 2];
+      uint32_t code = (k & 1) ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 15);
+      return orc_e2m1_to_f32(code) * orc_e4m3_to_f32(((const uint8_t*)scale)[n * (K / 16) + k / 16]);
+    }
+  }
+}
+
+/* out[n, k] = bf16(element * row factor) (engine/cpu/quant.cpp:250-271). */
+ORC_API int lx_dequantize_weight(const lx_weight* w, void* out, int64_t rows, int cols, void* stream) {
+  (void)stream;
+  if (!w || !w->data || !out) return fail(ORC_INVALID);
+  if (rows <= 0) return ORC_OK;
+  if (cols <= 0) return fail(ORC_INVALID);
+  if (w->type < LX_W_BF16 || w->type > LX_W_NVFP4) return fail(ORC_INVALID);
+  if (w->type != LX_W_BF16 && !w->scale) return fail(ORC_INVALID);
+  if (w->type == LX_W_NVFP4 && cols % 16 != 0) return fail(ORC_INVALID);
+  uint16_t* o = (uint16_t*)out;
+  if (w->type == LX_W_BF16) {
+    memcpy(o, w->data, (size_t)(2 * rows * cols));
+    return ORC_OK;
+  }
+#pragma omp parallel for schedule(static)
+  for (int64_t n = 0; n < rows; ++n) {
+    float f = w->type == LX_W_NVFP4 ? w->global : ((const float*)w->scale)[n];
+    for (int64_t k = 0; k < cols; ++k) o[n * cols + k] = bf16_round(weight_element(w->type, w->data, w->scale, n, k, cols) * f);
+  }
+  return ORC_OK;
+}
+
+/* ---- the product ------------------------------------------------------------------------------ */
+
+/* One weight row decoded to f32 without its row factor: what the reference's Row<F> hands the dot
+ * (engine/cpu/kern/isa.cpp:26-91; the NVFP4 block scale is applied per element, :78-90). */
+static void decode_row(int type, const void* data, const void* scale, int64_t n, int64_t K, float* out) {
+  for (int64_t k = 0; k < K; ++k) out[k] = weight_element(type, data, scale, n, k, K);
+}
+
+/* sum_k x[k] * w[k] in f32: four lane accumulators over ascending k (a separate multiply and add per
+ * step), one horizontal sum (0 + 2) + (1 + 3), then a fused scalar tail. This is the reference's tile at
+ * its generic level (vector width 4): engine/cpu/kern/isa.cpp:205-270 with vfma / vhsum of
+ * engine/cpu/kern/simd.h:144-157 and the fused tail of simd.h:467-476. Built with -ffp-contract=off so
+ * the lane step stays two roundings; the sums then equal that level's bit for bit. */
+static float dot_f32(const float* x, const float* w, int64_t K) {
+  float lane[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+  int64_t k = 0;
+  for (; k + 4 <= K; k += 4)
+    for (int j = 0; j < 4; ++j) {
+      float prod = x[k + j] * w[k + j];
+      lane[j] = lane[j] + prod;
+    }
+  float s = (lane[0] + lane[2]) + (lane[1] + lane[3]);
+  for (; k < K; ++k) s = fmaf(x[k], w[k], s);
+  return s;
+}
+
+/* The epilogue's exact operation order (engine/cpu/gemm.cpp:21-34). */
+static void epilogue(float sum, float rf, const void* bias, int bias_dtype, void* y, int y_dtype, int64_t at, int64_t n,
+                     float alpha, float beta) {
+  float t = rf * 1.0f * sum;
+  if (bias) t += load_f32(bias, bias_dtype, n);
+  float v = alpha * t;
+  if (beta != 0.0f) v = beta * load_f32(y, y_dtype, at) + v;
+  store_f32(y, y_dtype, at, v);
+}
+
+static int weight_ok(const lx_weight* w, int64_t K) {
+  if (!w || !w->data) return 0;
+  switch (w->type) {
+    case LX_W_BF16: return 1;
+    case LX_W_INT8:
+    case LX_W_FP8: return w->scale != NULL;
+    case LX_W_NVFP4: return w->scale != NULL && K % 16 == 0;
+    default: return 0;
+  }
+}
+
+/* y = alpha * (rf * (x @ W^T) + bias) + beta * y on f32 activation rows xs [M, K] (already in the
+ * form the math sees them). Shared by the GEMV and the GEMM (engine/cpu/gemm.cpp:74-124). */
+static int product(const float* xs, int64_t M, const lx_weight* w, const void* bias, int bias_dtype, void* y, int y_dtype,
+                   int64_t ld_y, int64_t N, int64_t K, float alpha, float beta) {
+  int err = 0;
+#pragma omp parallel
+  {
+    float* row = (float*)malloc(sizeof(float) * (size_t)K);
+    if (!row) {
+#pragma omp atomic write
+      err = 1;
+    } else {
+#pragma omp for schedule(static)
+      for (int64_t n = 0; n < N; ++n) {
+        decode_row(w->type, w->data, w->scale, n, K, row);
+        float rf = 1.0f;
+        if (w->type == LX_W_INT8 || w->type == LX_W_FP8) rf = ((const float*)w->scale)[n];
+        else if (w->type == LX_W_NVFP4) rf = w->global;
+        for (int64_t m = 0; m < M; ++m)
+          epilogue(dot_f32(xs + m * K, row, K), rf, bias, bias_dtype, y, y_dtype, m * ld_y + n, n, alpha, beta);
+      }
+      free(row);
+    }
+  }
+  return err ? fail(ORC_NOMEM) : ORC_OK;
+}
+
+/* The decode GEMV of every format: weight-only, f32 math on x as given (engine/cpu/gemm.cpp:160-183). */
+static int gemv_any(const void* x, int x_dtype, int ld_x, const lx_weight* w, const void* bias, int bias_dtype, void* y,
+                    int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta) {
+  if (M == 0 || N == 0) return ORC_OK;
+  if (M < 0 || M > 8 || K <= 0 || ld_x < K || ld_y < N) return fail(ORC_INVALID);
+  if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype) || !dtype_ok(bias_dtype)) return fail(ORC_INVALID);
+  if (!x || !y || !weight_ok(w, K)) return fail(ORC_INVALID);
+  float* xs = (float*)malloc(sizeof(float) * (size_t)M * (size_t)K);
+  if (!xs) return fail(ORC_NOMEM);
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t k = 0; k < K; ++k) xs[m * K + k] = load_f32(x, x_dtype, m * (int64_t)ld_x + k);
+  int st = product(xs, M, w, bias, bias_dtype, y, y_dtype, ld_y, N, K, alpha, beta);
+  free(xs);
+  return st;
+}
+
+/* engine/cpu/gemm.cpp:339-348 */
+ORC_API int lx_gemv(const void* x, int x_dtype, int ld_x, const void* w, int w_type, const float* w_scale, const void* bias,
+                    int bias_dtype, void* y, int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta,
+                    void* stream) {
+  (void)stream;
+  if (w_type != LX_W_BF16 && w_type != LX_W_INT8) return fail(ORC_INVALID);
+  if (w_type == LX_W_INT8 && !w_scale && M > 0 && N > 0) return fail(ORC_INVALID);
+  lx_weight wt = {w_type, w, w_scale, 1.0f, NULL};
+  return gemv_any(x, x_dtype, ld_x, &wt, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
+}
+
+/* engine/cpu/gemm.cpp:350-359 */
+ORC_API int lx_gemv_w(const void* x, int x_dtype, int ld_x, const lx_weight* w, const void* bias, int bias_dtype, void* y,
+                      int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
+  (void)stream;
+  if (!w) return fail(ORC_INVALID);
+  return gemv_any(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
+}
+
+/* engine/cpu/gemm.cpp:373-381 */
+ORC_API int lx_gemv_decode_bf16(const void* x, int x_dtype, int ld_x, const void* w, const void* bias, int bias_dtype,
+                                void* y, int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta,
+                                void* stream) {
+  (void)stream;
+  lx_weight wt = {LX_W_BF16, w, NULL, 1.0f, NULL};
+  return gemv_any(x, x_dtype, ld_x, &wt, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
+}
+
+/* Any M, weight-only BF16 math: x is rounded to bf16 (a bf16 x is used as it is) and the weights are
+ * expanded exactly, f32 accumulation (engine/cpu/gemm.cpp:189-296, the LX_MATH_BF16 branch :253-262).
+ * The low-precision maths are outside this build's path and answer 801. */
+static int gemm_bf16_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight* w, const void* bias, int bias_dtype,
+                          void* y, int y_dtype, int64_t ld_y, int64_t M, int64_t N, int64_t K, float alpha, float beta) {
+  if (M == 0 || N == 0) return ORC_OK;
+  if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(ORC_INVALID);
+  if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype) || (bias && !dtype_ok(bias_dtype))) return fail(ORC_INVALID);
+  if (!x || !y || !weight_ok(w, K)) return fail(ORC_INVALID);
+  float* xs = (float*)malloc(sizeof(float) * (size_t)M * (size_t)K);
+  if (!xs) return fail(ORC_NOMEM);
+  for (int64_t m = 0; m < M; ++m)
+    for (int64_t k = 0; k < K; ++k) {
+      uint16_t b = x_dtype == LX_BF16 ? ((const uint16_t*)x)[m * ld_x + k] : bf16_round(((const float*)x)[m * ld_x + k]);
+      xs[m * K + k] = bf16_value(b);
+    }
+  int st = product(xs, M, w, bias, bias_dtype, y, y_dtype, ld_y, N, K, alpha, beta);
+  free(xs);
+  return st;
+}
+
+ORC_API int lx_gemm_w(const void* x, int x_dtype, int ld_x, const lx_weight* w, int math, const void* bias, int bias_dtype,
+                      void* y, int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* workspace,
+                      void* stream) {
+  (void)stream;
+  (void)workspace;
+  if (!w) return fail(ORC_INVALID);
+  if (math < LX_MATH_BF16 || math > LX_MATH_FP4) return fail(ORC_INVALID);
+  if (math != LX_MATH_BF16) return fail(ORC_UNSUPPORTED);
+  return gemm_bf16_math(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
+}
+
+/* engine/cpu/gemm.cpp:290-296 */
+ORC_API int64_t lx_gemm_workspace_bytes(int M, int K, int math) {
+  if (M <= 0 || K <= 0) return 0;
+  int64_t elem = math == LX_MATH_INT8 ? 1 : 4;
+  int64_t bytes = ((int64_t)M * 4 + 63) / 64 * 64 + (int64_t)M * K * elem;
+  return (bytes + 255) / 256 * 256;
+}
+
+/* The skinny decode GEMM's contract (engine/cuda/kernels.h:453-477): bf16 x, exact bf16 products,
+ * f32 sums, f32 epilogue v = alpha * (sum + bias) + beta * y. The reference has it on CUDA only
+ * (bf16 weights); the contract text is what this restates, for every format. */
+ORC_API int lx_gemm_skinny(const void* x, int x_dtype, int ld_x, const lx_weight* w, const void* bias, int bias_dtype,
+                           void* y, int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
+  (void)stream;
+  if (!w) return fail(ORC_INVALID);
+  if (x_dtype != LX_BF16 && M > 0 && N > 0) return fail(ORC_UNSUPPORTED);
+  return gemm_bf16_math(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
+}
+
+/* ---- routing (engine/cpu/moe.cpp:343-397, contract engine/cuda/kernels.h:203-209) ----------------- */
+
+ORC_API int lx_moe_route(const float* logits, const float* selection_bias, int32_t* ids, float* weights, float* entropy,
+                         float* confidence, int T, int E, int top_k, void* stream) {
+  (void)stream;
+  if (T <= 0) return ORC_OK;
+  if (top_k < 1 || top_k > 64 || top_k > E || !logits || !ids || !weights || !entropy || !confidence)
+    return fail(ORC_INVALID);
+  for (int64_t t = 0; t < T; ++t) {
+    const float* row = logits + t * E;
+    float m = -INFINITY;
+    for (int i = 0; i < E; ++i)
+      if (row[i] > m) m = row[i];
+    float z = 0.0f;
+    for (int i = 0; i < E; ++i) z += expf(row[i] - m);
+    float h = 0.0f;
+    for (int i = 0; i < E; ++i) {
+      float p = expf(row[i] - m) / z;
+      h -= p * logf(p > 1e-9f ? p : 1e-9f);
+    }
+    entropy[t] = h;
+    confidence[t] = 1.0f / z; /* the largest probability is exp(0) / z */
+    int picked[64];
+    for (int r = 0; r < top_k; ++r) {
+      float best = -INFINITY;
+      int best_i = E;
+      for (int i = 0; i < E; ++i) {
+        int taken = 0;
+        for (int q = 0; q < r; ++q) taken |= picked[q] == i;
+        if (taken) continue;
+        float v = row[i] + (selection_bias ? selection_bias[i] : 0.0f); /* one f32 add */
+        if (v > best || (v == best && i < best_i)) {
+          best = v;
+          best_i = i;
+        }
+      }
+      picked[r] = best_i;
+    }
+    float lmax = -INFINITY;
+    for (int r = 0; r < top_k; ++r)
+      if (row[picked[r]] > lmax) lmax = row[picked[r]];
+    float e[64], esum = 0.0f;
+    for (int r = 0; r < top_k; ++r) {
+      e[r] = expf(row[picked[r]] - lmax);
+      esum += e[r];
+    }
+    for (int r = 0; r < top_k; ++r) {
+      ids[t * top_k + r] = picked[r];
+      weights[t * top_k + r] = e[r] / esum;
+    }
+  }
+  return ORC_OK;
+}
+
+/* ---- routed experts (engine/cpu/moe.cpp:163-329) -------------------------------------------------- */
+
+static float silu(float v) { return v / (1.0f + expf(-v)); } /* engine/cpu/cpu.h:68 */
+
+/* Expert e of an [E, N, K] stack as a plain [N, K] weight, with the expert's own NVFP4 global when the
+ * stack carries them (engine/cpu/moe.cpp:36-64). */
+static lx_weight expert_slice(const lx_weight* s, int64_t e, int64_t N, int64_t K) {
+  lx_weight o = {s->type, NULL, NULL, 1.0f, NULL};
+  int64_t rows = e * N;
+  switch (s->type) {
+    case LX_W_BF16: o.data = (const uint16_t*)s->data + rows * K; break;
+    case LX_W_INT8:
+    case LX_W_FP8:
+      o.data = (const uint8_t*)s->data + rows * K;
+      o.scale = (const float*)s->scale + rows;
+      break;
+    default:
+      o.data = (const uint8_t*)s->data + rows * (K / 2);
+      o.scale = (const uint8_t*)s->scale + rows * (K / 16);
+      o.global = s->expert_global ? s->expert_global[e] : s->global;
+      break;
+  }
+  return o;
+}
+
+static float row_factor(const lx_weight* w, int64_t n) {
+  if (w->type == LX_W_INT8 || w->type == LX_W_FP8) return ((const float*)w->scale)[n];
+  if (w->type == LX_W_NVFP4) return w->global;
+  return 1.0f;
+}
+
+/* Weight-only experts: for each (token, slot) pair, inter = bf16(silu(s_g * g) * (s_u * u)) with
+ * g = gate_e . x, u = up_e . x (engine/cpu/moe.cpp:241-279, rounding point :267-270), contribution =
+ * s_l * down_e . inter (:292-312), and out[t] = w0 * c0 + sum_{k >= 1} w_k * c_k in slot order
+ * (:315-327). BF16 math on bf16 operands is the same arithmetic (exact products, f32 sums). */
+static int experts(const uint16_t* latent, const int32_t* ids, const float* weights, const lx_weight* gu,
+                   const lx_weight* dn, float* out, int64_t T, int64_t L, int64_t I, int64_t top_k, int64_t E) {
+  const int64_t P = T * top_k;
+  if (E <= 0) {
+    for (int64_t p = 0; p < P; ++p)
+      if (ids[p] + 1 > E) E = ids[p] + 1;
+  }
+  for (int64_t p = 0; p < P; ++p)
+    if (ids[p] < 0 || ids[p] >= E) return fail(ORC_INVALID);
+  float* contrib = (float*)malloc(sizeof(float) * (size_t)P * (size_t)L);
+  float* xf = (float*)malloc(sizeof(float) * (size_t)T * (size_t)L);
+  if (!contrib || !xf) {
+    free(contrib);
+    free(xf);
+    return fail(ORC_NOMEM);
+  }
+  for (int64_t i = 0; i < T * L; ++i) xf[i] = bf16_value(latent[i]);
+  int err = 0;
+  /* Experts in turn; each expert's rows are decoded once for all the pairs that chose it. */
+#pragma omp parallel for schedule(dynamic, 1)
+  for (int64_t e = 0; e < E; ++e) {
+    int64_t cnt = 0;
+    for (int64_t p = 0; p < P; ++p) cnt += ids[p] == e;
+    if (!cnt) continue;
+    lx_weight g = expert_slice(gu, e, 2 * I, L), d = expert_slice(dn, e, L, I);
+    float* wrow = (float*)malloc(sizeof(float) * (size_t)(L > I ? L : I));
+    float* gate = (float*)malloc(sizeof(float) * (size_t)cnt * (size_t)I * 2);
+    float* inter = (float*)malloc(sizeof(float) * (size_t)cnt * (size_t)I);
+    int64_t* pair = (int64_t*)malloc(sizeof(int64_t) * (size_t)cnt);
+    if (!wrow || !gate || !inter || !pair) {
+#pragma omp atomic write
+      err = 1;
+    } else {
+      int64_t c = 0;
+      for (int64_t p = 0; p < P; ++p)
+        if (ids[p] == e) pair[c++] = p;
+      float* up = gate + cnt * I;
+      for (int64_t i = 0; i < 2 * I; ++i) {
+        decode_row(g.type, g.data, g.scale, i, L, wrow);
+        float rf = row_factor(&g, i);
+        for (int64_t r = 0; r < cnt; ++r) {
+          float s = rf * (1.0f * dot_f32(xf + (pair[r] / top_k) * L, wrow, L));
+          if (i < I) gate[r * I + i] = s;
+          else up[r * I + (i - I)] = s;
+        }
+      }
+      for (int64_t r = 0; r < cnt; ++r)
+        for (int64_t i = 0; i < I; ++i) inter[r * I + i] = bf16_value(bf16_round(silu(gate[r * I + i]) * up[r * I + i]));
+      for (int64_t l = 0; l < L; ++l) {
+        decode_row(d.type, d.data, d.scale, l, I, wrow);
+        float rf = row_factor(&d, l);
+        for (int64_t r = 0; r < cnt; ++r) contrib[pair[r] * L + l] = rf * (1.0f * dot_f32(inter + r * I, wrow, I));
+      }
+    }
+    free(wrow);
+    free(gate);
+    free(inter);
+    free(pair);
+  }
+  if (!err) {
+    for (int64_t t = 0; t < T; ++t) {
+      float* o = out + t * L;
+      const float w0 = weights[t * top_k];
+      for (int64_t l = 0; l < L; ++l) o[l] = w0 * contrib[(t * top_k) * L + l];
+      for (int64_t k = 1; k < top_k; ++k) {
+        const float wk = weights[t * top_k + k];
+        for (int64_t l = 0; l < L; ++l) o[l] += wk * contrib[(t * top_k + k) * L + l];
+      }
+    }
+  }
+  free(contrib);
+  free(xf);
+  return err ? fail(ORC_NOMEM) : ORC_OK;
+}
+
+static int stack_ok(const lx_weight* w, int64_t K) { return weight_ok(w, K); }
+
+static int experts_args(const void* latent, const int32_t* ids, const float* weights, float* out, int L, int I, int top_k) {
+  if (!latent || !ids || !weights || !out || L <= 0 || I <= 0 || top_k < 1) return fail(ORC_INVALID);
+  return ORC_OK;
+}
+
+/* engine/cpu/moe.cpp:444-458 */
+ORC_API int lx_moe_experts(const void* latent, const int32_t* ids, const float* weights, const void* gate_up,
+                           const void* down, float* out, int T, int L, int I, int top_k, void* stream) {
+  (void)stream;
+  if (T <= 0) return ORC_OK;
+  int st = experts_args(latent, ids, weights, out, L, I, top_k);
+  if (st) return st;
+  if (!gate_up || !down) return fail(ORC_INVALID);
+  lx_weight gu = {LX_W_BF16, gate_up, NULL, 1.0f, NULL}, dn = {LX_W_BF16, down, NULL, 1.0f, NULL};
+  return experts((const uint16_t*)latent, ids, weights, &gu, &dn, out, T, L, I, top_k, 0);
+}
+
+/* engine/cpu/moe.cpp:496-503 */
+ORC_API int lx_moe_experts_decode_bf16(const void* latent, const int32_t* ids, const float* weights, const void* gate_up,
+                                       const void* down, float* out, void* workspace, int T, int L, int I, int top_k,
+                                       void* stream) {
+  if (T <= 0) return ORC_OK;
+  if (top_k > 8 || !workspace) return fail(ORC_INVALID);
+  return lx_moe_experts(latent, ids, weights, gate_up, down, out, T, L, I, top_k, stream);
+}
+
+/* engine/cpu/moe.cpp:519-538 */
+ORC_API int lx_moe_experts_decode(const void* latent, const int32_t* ids, const float* weights, const lx_weight* gate_up,
+                                  const lx_weight* down, float* out, void* workspace, int T, int L, int I, int top_k,
+                                  void* stream) {
+  (void)stream;
+  (void)workspace;
+  if (T <= 0) return ORC_OK;
+  if (T > 8 || top_k > 8) return fail(ORC_INVALID);
+  int st = experts_args(latent, ids, weights, out, L, I, top_k);
+  if (st) return st;
+  if (!gate_up || !down) return fail(ORC_INVALID);
+  if (!stack_ok(gate_up, L) || !stack_ok(down, I)) return fail(ORC_INVALID);
+  return experts((const uint16_t*)latent, ids, weights, gate_up, down, out, T, L, I, top_k, 0);
+}
+
+/* engine/cpu/moe.cpp:546-572; only the weight-only BF16 math is on this build's path. */
+ORC_API int lx_moe_experts_grouped(const void* latent, const int32_t* ids, const float* weights, const lx_weight* gate_up,
+                                   const lx_weight* down, int math, float* out, void* workspace, int T, int L, int I, int E,
+                                   int top_k, void* stream) {
+  (void)stream;
+  (void)workspace;
+  if (T <= 0) return ORC_OK;
+  int st = experts_args(latent, ids, weights, out, L, I, top_k);
+  if (st) return st;
+  if (E <= 0 || !gate_up || !down || !stack_ok(gate_up, L) || !stack_ok(down, I)) return fail(ORC_INVALID);
+  if (math < LX_MATH_BF16 || math > LX_MATH_FP4) return fail(ORC_INVALID);
+  if (math != LX_MATH_BF16) return fail(ORC_UNSUPPORTED);
+  return experts((const uint16_t*)latent, ids, weights, gate_up, down, out, T, L, I, top_k, E);
+}
+
+static int64_t round256(int64_t b) { return (b + 255) / 256 * 256; }
+
+/* engine/cpu/moe.cpp:540-544 */
+ORC_API int64_t lx_moe_decode_workspace_bytes(int T, int I, int top_k) {
+  if (T <= 0 || I <= 0 || top_k <= 0) return 0;
+  return round256(2 * (int64_t)T * top_k * I);
+}
+/* engine/cpu/moe.cpp:506-509 */
+ORC_API int64_t lx_moe_bf16x_workspace_bytes(int T, int I, int top_k) { return lx_moe_decode_workspace_bytes(T, I, top_k); }
+/* engine/cpu/moe.cpp:574-581 */
+ORC_API int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int top_k, int math) {
+  (void)E;
+  (void)math;
+  if (T <= 0 || L <= 0 || I <= 0 || top_k <= 0) return 0;
+  return round256(2 * (int64_t)T * top_k * I);
+}
+
+/* ---- the few runtime calls a host-memory harness needs (engine/cuda/kernels.h:308-339) ------------- */
+
+ORC_API int lx_rt_backend(void) { return 3; /* LX_BACKEND_CPU */ }
+ORC_API int lx_rt_device_count(void) { return 1; }
+ORC_API int lx_rt_stream_sync(void* stream) {
+  (void)stream;
+  return ORC_OK;
+}
+ORC_API int lx_rt_device_sync(void) { return ORC_OK; }
+ORC_API int lx_rt_last_error(void) {
+  int e = g_last_error;
+  g_last_error = 0;
+  return e;
+}

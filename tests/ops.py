@@ -1,0 +1,159 @@
+"""Calls into a backend library (an abi.Kernels), shared by the CPU and GPU tests: each function allocates
+the outputs on the library's device, calls one lx_* entry point and returns the result."""
+
+import ctypes
+
+import torch
+
+from dromos_amd.abi import DTYPE, F32, MATH_BF16
+from dromos_amd.formats import Weight
+
+
+def gemv_w(lx, x, w, bias=None, y=None, alpha=1.0, beta=0.0, M=None, N=None, K=None, ld_x=None, ld_y=None,
+           y_dtype=torch.float32, entry="gemv_w", status=False):
+    M = x.shape[0] if M is None else M
+    K = x.shape[1] if K is None else K
+    N = w.data.shape[-2] if N is None else N
+    if y is None:
+        y = torch.full((M, N), float("nan"), dtype=y_dtype, device=lx.device)
+    lw = w.lx()
+    args = (x, DTYPE[x.dtype], ld_x if ld_x is not None else x.shape[1], ctypes.pointer(lw), bias,
+            DTYPE[bias.dtype] if bias is not None else F32, y, DTYPE[y.dtype], ld_y if ld_y is not None else y.shape[1],
+            M, N, K, float(alpha), float(beta))
+    if status:
+        return lx.status(entry, *args)
+    lx(entry, *args)
+    return y
+
+
+def gemm_w(lx, x, w, math=MATH_BF16, bias=None, y=None, alpha=1.0, beta=0.0, y_dtype=torch.float32, status=False,
+           ld_x=None, ld_y=None, N=None):
+    M, K = x.shape[0], w_cols(w)
+    N = w.data.shape[-2] if N is None else N
+    if y is None:
+        y = torch.full((M, N), float("nan"), dtype=y_dtype, device=lx.device)
+    nbytes = max(int(lx.size("gemm_workspace_bytes", M, K, math)), 256)
+    ws = torch.full((nbytes,), 0xFF, dtype=torch.uint8, device=lx.device)
+    lw = w.lx()
+    args = (x, DTYPE[x.dtype], ld_x if ld_x is not None else x.shape[1], ctypes.pointer(lw), math, bias,
+            DTYPE[bias.dtype] if bias is not None else F32, y, DTYPE[y.dtype], ld_y if ld_y is not None else y.shape[1],
+            M, N, K, float(alpha), float(beta), ws)
+    if status:
+        return lx.status("gemm_w", *args)
+    lx("gemm_w", *args)
+    return y
+
+
+def w_cols(w):
+    from dromos_amd.abi import W_NVFP4
+
+    return w.data.shape[-1] * 2 if w.fmt == W_NVFP4 else w.data.shape[-1]
+
+
+def gemm_skinny(lx, x, w, bias=None, y=None, alpha=1.0, beta=0.0, y_dtype=torch.float32, status=False):
+    M, K = x.shape
+    N = w.data.shape[-2]
+    if y is None:
+        y = torch.full((M, N), float("nan"), dtype=y_dtype, device=lx.device)
+    lw = w.lx()
+    args = (x, DTYPE[x.dtype], K, ctypes.pointer(lw), bias, DTYPE[bias.dtype] if bias is not None else F32, y,
+            DTYPE[y.dtype], N, M, N, K, float(alpha), float(beta))
+    if status:
+        return lx.status("gemm_skinny", *args)
+    lx("gemm_skinny", *args)
+    return y
+
+
+def dequantize(lx, w, N, K):
+    out = torch.empty(N, K, dtype=torch.bfloat16, device=lx.device)
+    lw = w.lx()
+    lx("dequantize_weight", ctypes.pointer(lw), out, ctypes.c_int64(N), K)
+    return out
+
+
+def route(lx, logits, bias, top_k):
+    T, E = logits.shape
+    ids = torch.full((T, top_k), -1, dtype=torch.int32, device=lx.device)
+    weights = torch.full((T, top_k), float("nan"), dtype=torch.float32, device=lx.device)
+    entropy = torch.full((T,), float("nan"), dtype=torch.float32, device=lx.device)
+    confidence = torch.full((T,), float("nan"), dtype=torch.float32, device=lx.device)
+    lx("moe_route", logits, bias, ids, weights, entropy, confidence, T, E, top_k)
+    return ids, weights, entropy, confidence
+
+
+def experts_decode(lx, latent, ids, weights, gu, dn, I, top_k, status=False):
+    T, L = latent.shape
+    nbytes = int(lx.size("moe_decode_workspace_bytes", T, I, top_k))
+    assert nbytes >= 2 * T * top_k * I
+    ws = torch.full((max(nbytes, 1),), 0xFF, dtype=torch.uint8, device=lx.device)  # garbage: NaN bf16
+    out = torch.full((T, L), float("nan"), device=lx.device)
+    g, d = gu.lx(), dn.lx()
+    args = (latent, ids, weights, ctypes.pointer(g), ctypes.pointer(d), out, ws, T, L, I, top_k)
+    if status:
+        return lx.status("moe_experts_decode", *args)
+    lx("moe_experts_decode", *args)
+    return out
+
+
+def experts_grouped(lx, latent, ids, weights, gu, dn, I, E, top_k, math=MATH_BF16, status=False):
+    T, L = latent.shape
+    fn = lx.lib.lx_moe_grouped_workspace_bytes
+    fn.restype = ctypes.c_int64
+    nbytes = int(fn(T, L, I, E, top_k, math))
+    ws = torch.full((max(nbytes, 1),), 0xFF, dtype=torch.uint8, device=lx.device)
+    out = torch.full((T, L), float("nan"), device=lx.device)
+    g, d = gu.lx(), dn.lx()
+    args = (latent, ids, weights, ctypes.pointer(g), ctypes.pointer(d), math, out, ws, T, L, I, E, top_k)
+    if status:
+        return lx.status("moe_experts_grouped", *args)
+    lx("moe_experts_grouped", *args)
+    return out
+
+
+def experts_bf16(lx, latent, ids, weights, gate_up, down, I, top_k):
+    T, L = latent.shape
+    out = torch.full((T, L), float("nan"), device=lx.device)
+    lx("moe_experts", latent, ids, weights, gate_up, down, out, T, L, I, top_k)
+    return out
+
+
+# ---- float64 statements of what the ops compute, from closed forms only ----------------------------------
+
+
+def gemv_reference(x, dense, bias, alpha, beta, y0):
+    out = x.double().cpu() @ dense.double().T
+    if bias is not None:
+        out = out + bias.double().cpu()
+    out = alpha * out
+    if beta != 0.0:
+        out = out + beta * y0.double().cpu()
+    return out
+
+
+def route_reference(logits, bias, top_k):
+    """Selection on f32 biased logits (one IEEE add), stable descending order; weights and statistics in float64."""
+    logits = logits.cpu()
+    biased = logits.float() if bias is None else logits.float() + bias.cpu().float()
+    ids = torch.sort(-biased, dim=-1, stable=True).indices[:, :top_k]
+    wide = logits.double()
+    weights = torch.softmax(torch.gather(wide, -1, ids), dim=-1)
+    p = torch.softmax(wide, dim=-1)
+    entropy = -(p * torch.log(p.clamp_min(1e-9))).sum(-1)
+    return ids, weights, entropy, p.max(-1).values
+
+
+def experts_reference(latent, ids, weights, gu_dense, dn_dense):
+    """float64 experts on dense stacks gu [E, 2I, L], dn [E, L, I]; the intermediate is rounded to bf16."""
+    import torch.nn.functional as F
+
+    I = gu_dense.shape[1] // 2
+    x = latent.double().cpu()
+    ids, weights = ids.cpu(), weights.cpu()
+    out = torch.zeros(x.shape[0], x.shape[1], dtype=torch.float64)
+    for t in range(ids.shape[0]):
+        for k in range(ids.shape[1]):
+            e = int(ids[t, k])
+            g, u = gu_dense[e, :I] @ x[t], gu_dense[e, I:] @ x[t]
+            mid = (F.silu(g) * u).to(torch.bfloat16).double()
+            out[t] += weights[t, k].double() * (dn_dense[e] @ mid)
+    return out

@@ -1,0 +1,81 @@
+"""Pins the oracle's routing and routed experts: routing against a stable sort of the f32 biased logits and
+float64 softmax statistics (ids exact), tie cases from the reference's tests, the experts against float64 with the
+bf16-rounded intermediate, and both against the reference's CPU backend where it was built."""
+
+import pytest
+import torch
+
+import checks
+import ops
+from conftest import rel_l2
+from dromos_amd.abi import FORMATS
+from dromos_amd.formats import random_stack
+
+FMT = checks.FMT_NAMES
+
+
+@pytest.mark.parametrize("E,T,top_k", [(128, 1, 4), (128, 7, 4), (192, 300, 4), (64, 8, 8), (5, 3, 2), (37, 7, 3), (7, 2, 7), (64, 1, 1)])
+def test_route(oracle, E, T, top_k):
+    checks.route_case(oracle, T, E, top_k, seed=E * 1000 + T)
+
+
+def test_route_without_bias_and_ties(oracle):
+    checks.route_case(oracle, 33, 128, 4, seed=7, with_bias=False)
+    checks.route_ties(oracle)
+
+
+def test_route_equals_the_reference_backend(oracle, ref):
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn(64, 128, generator=g) * 2
+    bias = torch.randn(128, generator=g) * 0.5
+    a, b = ops.route(oracle, logits, bias, 8), ops.route(ref, logits, bias, 8)
+    for u, v in zip(a, b):
+        assert torch.equal(u, v)  # same libm, same order: bit for bit
+
+
+@pytest.mark.parametrize("fmt", FMT)
+@pytest.mark.parametrize("T", [1, 4, 8])
+def test_decode_experts(oracle, fmt, T):
+    checks.decode_case(oracle, fmt, fmt, T, 16, 256, 128, 4, seed=T * 13)
+
+
+@pytest.mark.parametrize("T,E,L,I,top_k", [(1, 1, 16, 16, 1), (3, 5, 48, 32, 2), (5, 9, 64, 48, 3), (8, 8, 32, 64, 8)])
+@pytest.mark.parametrize("fmt", FMT)
+def test_decode_experts_odd_shapes(oracle, fmt, T, E, L, I, top_k):
+    checks.decode_case(oracle, fmt, fmt, T, E, L, I, top_k, seed=T + E)
+
+
+def test_decode_experts_mixed_formats_and_repeats(oracle):
+    checks.decode_case(oracle, "nvfp4", "fp8", 4, 16, 256, 128, 4, seed=23)
+    checks.decode_case(oracle, "int8", "bf16", 4, 16, 256, 128, 4, seed=24)
+    pool = torch.tensor([3, 9, 17, 21, 40, 55])
+    checks.decode_case(oracle, "nvfp4", "nvfp4", 8, 64, 256, 128, 4, seed=33, pool=pool)
+
+
+def test_decode_rejects_more_than_eight_tokens(oracle):
+    gu, dn = random_stack(0, 8, 64, 32, 1), random_stack(0, 8, 32, 32, 2)
+    latent, ids, weights = checks.make_routing(9, 8, 32, 2, 3)
+    assert ops.experts_decode(oracle, latent, ids, weights, gu, dn, 32, 2, status=True) != 0
+
+
+@pytest.mark.parametrize("fmt", FMT)
+def test_grouped_experts(oracle, fmt):
+    checks.grouped_case(oracle, fmt, 37, 128, 64, 16, 3, seed=31)
+
+
+@pytest.mark.parametrize("fmt", FMT)
+def test_experts_equal_the_reference_generic_level(oracle, ref, fmt):
+    # Same grouping, same f32 sums (generic level), same libm exp in silu: every output bit agrees.
+    ref.lib.lx_set_arch_override(1)
+    try:
+        T, E, L, I, top_k = 6, 12, 256, 128, 4
+        gu, dn = random_stack(FORMATS[fmt], E, 2 * I, L, 71), random_stack(FORMATS[fmt], E, L, I, 72)
+        latent, ids, weights = checks.make_routing(T, E, L, top_k, 73)
+        a = ops.experts_decode(oracle, latent, ids, weights, gu, dn, I, top_k)
+        b = ops.experts_decode(ref, latent, ids, weights, gu, dn, I, top_k)
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+        a = ops.experts_grouped(oracle, latent, ids, weights, gu, dn, I, E, top_k)
+        b = ops.experts_grouped(ref, latent, ids, weights, gu, dn, I, E, top_k)
+        assert rel_l2(a, b) < 1e-5  # the reference's BF16 math may take its bf16 dot instructions
+    finally:
+        ref.lib.lx_set_arch_override(0)

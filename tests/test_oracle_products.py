@@ -1,0 +1,117 @@
+"""Pins the oracle's GEMV / GEMM: float64 x @ W^T on the decoded values (a dropped scale, a swapped nibble, a
+transposed operand or a wrong epilogue order fails it), the contract's edge cases, and bit-for-bit agreement
+of the f32 sums with the reference's CPU backend at its generic level."""
+
+import pytest
+import torch
+
+import checks
+import ops
+from conftest import rel_l2
+from dromos_amd.abi import FORMATS, MATH_BF16, MATH_INT8, W_BF16, W_INT8
+from dromos_amd.formats import random_weight
+
+FMT = checks.FMT_NAMES
+
+
+@pytest.mark.parametrize("K", [48, 528, 2048])
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (-1.5, 1.0)])
+@pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("bias_dtype", [None, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("fmt", FMT)
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M", [1, 8])
+def test_gemv_dtype_matrix(oracle, M, x_dtype, fmt, bias_dtype, y_dtype, alpha, beta, K):
+    checks.gemv_case(oracle, fmt, M, 37, K, seed=M * 101 + K, x_dtype=x_dtype, bias_dtype=bias_dtype, y_dtype=y_dtype,
+                     alpha=alpha, beta=beta)
+
+
+@pytest.mark.parametrize("pad", [0, 3, 8])
+@pytest.mark.parametrize("fmt", FMT)
+def test_gemv_strided(oracle, fmt, pad):
+    checks.gemv_case(oracle, fmt, 5, 300, 1024, seed=pad + 9, bias_dtype=torch.bfloat16, alpha=2.0, beta=0.5, pad=pad)
+
+
+@pytest.mark.parametrize("fmt", FMT)
+def test_gemv_rows_do_not_depend_on_batch(oracle, fmt):
+    checks.gemv_rows_do_not_depend_on_batch(oracle, fmt, 256, 2048, seed=5)
+
+
+def test_gemv_nvfp4_global_is_linear(oracle):
+    checks.gemv_nvfp4_global_is_linear(oracle)
+
+
+def test_gemv_argument_errors(oracle):
+    w = random_weight(W_BF16, 8, 64, 1)
+    x = torch.zeros(9, 64)
+    assert ops.gemv_w(oracle, x, w, status=True) == 1  # M > 8
+    assert ops.gemv_w(oracle, x[:0], w, M=0, status=True) == 0
+    assert ops.gemv_w(oracle, x[:2], w, ld_x=32, status=True) == 1  # ld_x < K
+    w3 = random_weight(FORMATS["nvfp4"], 8, 64, 1)
+    assert ops.gemv_w(oracle, torch.zeros(1, 40), w3, K=40, N=8, status=True) == 1  # K % 16 != 0
+
+
+def test_gemv_wrapper_entry_points(oracle):
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(4, 1024, generator=g)
+    for fmt in (W_BF16, W_INT8):
+        w = random_weight(fmt, 300, 1024, fmt + 1)
+        a = torch.empty(4, 300)
+        oracle("gemv", x, 0, 1024, w.data, fmt, w.scale, None, 0, a, 0, 300, 4, 300, 1024, 1.0, 0.0)
+        assert torch.equal(a, ops.gemv_w(oracle, x, w))
+    w = random_weight(W_BF16, 300, 1024, 1)
+    a = torch.empty(4, 300)
+    oracle("gemv_decode_bf16", x, 0, 1024, w.data, None, 0, a, 0, 300, 4, 300, 1024, 1.0, 0.0)
+    assert torch.equal(a, ops.gemv_w(oracle, x, w))
+
+
+@pytest.mark.parametrize("fmt", FMT)
+@pytest.mark.parametrize("M", [1, 16, 64, 70])
+def test_gemm_w_bf16_math(oracle, fmt, M):
+    # Weight-only BF16 math: x is rounded to bf16 first, so the reference uses the rounded activations.
+    N, K = 96, 512
+    g = torch.Generator().manual_seed(M)
+    x = torch.randn(M, K, generator=g)
+    w = random_weight(FORMATS[fmt], N, K, M + 3)
+    bias = torch.randn(N, generator=g).to(torch.bfloat16)
+    y = ops.gemm_w(oracle, x, w, MATH_BF16, bias=bias, alpha=0.5)
+    want = ops.gemv_reference(x.to(torch.bfloat16), w.dense(), bias, 0.5, 0.0, None)
+    checks.check_product(y, want)
+    assert ops.gemm_w(oracle, x, w, MATH_INT8, status=True) == 801  # outside this path
+    ys = ops.gemm_skinny(oracle, x.to(torch.bfloat16), w, bias=bias, alpha=0.5)
+    assert torch.equal(ys, y)
+
+
+@pytest.mark.parametrize("fmt", FMT)
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+def test_f32_sums_equal_the_reference_generic_level(oracle, ref, fmt, x_dtype):
+    # The reference at level 1 sums four lanes with unfused steps, a fixed horizontal order and a fused tail;
+    # the oracle restates exactly that, so the f32 outputs agree to the last bit (K = 1030 leaves a tail).
+    real = ref.lib.lx_set_arch_override(0)
+    try:
+        assert ref.lib.lx_set_arch_override(1) == 1
+        for M, N, K in [(1, 64, 1024), (8, 37, 1030 if fmt != "nvfp4" else 1040), (3, 300, 528)]:
+            g = torch.Generator().manual_seed(K + M)
+            x = torch.randn(M, K, generator=g).to(x_dtype)
+            w = random_weight(FORMATS[fmt], N, K, K)
+            bias = torch.randn(N, generator=g)
+            y0 = torch.randn(M, N, generator=g)
+            a = ops.gemv_w(oracle, x, w, bias, y0.clone(), alpha=1.25, beta=-0.5)
+            b = ops.gemv_w(ref, x, w, bias, y0.clone(), alpha=1.25, beta=-0.5)
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32)), (M, N, K)
+    finally:
+        ref.lib.lx_set_arch_override(0)
+    assert real >= 1
+
+
+@pytest.mark.parametrize("fmt", FMT)
+def test_agrees_with_the_reference_best_level(oracle, ref, fmt):
+    # Whatever vector width the reference picks on this CPU, the two agree far inside the path's tolerance.
+    g = torch.Generator().manual_seed(7)
+    x = torch.randn(4, 4096, generator=g).to(torch.bfloat16)
+    w = random_weight(FORMATS[fmt], 512, 4096, 11)
+    a, b = ops.gemv_w(oracle, x, w), ops.gemv_w(ref, x, w)
+    assert rel_l2(a, b) < 1e-5
+    x64 = torch.randn(40, 4096, generator=g).to(torch.bfloat16)
+    a, b = ops.gemm_w(oracle, x64, w), ops.gemm_w(ref, x64, w)
+    assert rel_l2(a, b) < 1e-5
