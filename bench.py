@@ -1,0 +1,336 @@
+#!/usr/bin/env python3
+"""Measures the decode matrix-product path on one MI355X: weight-stream GB/s and fraction of the 8 TB/s HBM peak.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cases headline|all] [--no-cpu]
+
+A step is one pass of the hot path over one batch: one lx_gemv_w call (the headline), one skinny GEMM, or one
+routed-experts step, always on a weight copy that was not touched recently (the copies rotate through more
+than 512 MB, past the 256 MB Infinity Cache, so every step streams from HBM). The K timed steps are recorded
+once into a HIP graph through the library's own lx_rt_capture_* entry points (as the engine runs its decode
+steps) and the graph is launched between two HIP events on its stream; W untimed steps run first.
+
+Prints one JSON line. `value` is the headline case (INT8 weight-only GEMV, W 14336 x 4096, M = 1, bf16 x);
+`cases` lists every measured case with its own time, GB/s and fraction of peak. Bytes per step are the
+algorithmic bytes: weights + scales + x + y (bench/bench_gemv.py:51-56 of the reference uses the same count).
+"""
+
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+sys.path.insert(0, str(ROOT))
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def algorithmic_bytes_gemv(fmt, M, N, K, y_bytes=4):
+    w = {"bf16": 2 * N * K, "int8": N * K, "fp8": N * K, "nvfp4": N * K // 2}[fmt]
+    s = {"bf16": 0, "int8": 4 * N, "fp8": 4 * N, "nvfp4": N * K // 16 + 4}[fmt]
+    return w + s + M * K * 2 + M * N * y_bytes
+
+
+class Timer:
+    """K steps captured into one graph, launched between two timed HIP events on the capture stream."""
+
+    def __init__(self, lx, torch):
+        self.lx, self.torch = lx, torch
+        self.stream = torch.cuda.Stream()
+        lib = lx.lib
+        self.ev = []
+        for _ in range(2):
+            e = ctypes.c_void_p()
+            assert lib.lx_rt_event_create_timed(ctypes.byref(e)) == 0
+            self.ev.append(e)
+
+    def run(self, step, steps, warmup, repeats=5):
+        """step(i) issues step i on the current stream. Returns the median microseconds per step."""
+        torch, lib = self.torch, self.lx.lib
+        with torch.cuda.stream(self.stream):
+            s = ctypes.c_void_p(self.stream.cuda_stream)
+            for i in range(warmup):
+                step(i)
+            torch.cuda.synchronize()
+            assert lib.lx_rt_capture_begin(s) == 0
+            for i in range(steps):
+                step(warmup + i)
+            graph = ctypes.c_void_p()
+            assert lib.lx_rt_capture_end(s, ctypes.byref(graph)) == 0
+            assert lib.lx_rt_graph_launch(graph, s) == 0  # untimed: uploads the graph
+            torch.cuda.synchronize()
+            times = []
+            for _ in range(repeats):
+                torch.cuda.synchronize()
+                assert lib.lx_rt_event_record(self.ev[0], s) == 0
+                assert lib.lx_rt_graph_launch(graph, s) == 0
+                assert lib.lx_rt_event_record(self.ev[1], s) == 0
+                torch.cuda.synchronize()
+                ms = ctypes.c_float()
+                assert lib.lx_rt_event_elapsed(self.ev[0], self.ev[1], ctypes.byref(ms)) == 0
+                times.append(ms.value * 1e3 / steps)
+            assert lib.lx_rt_graph_destroy(graph) == 0
+        times.sort()
+        return times[len(times) // 2]
+
+
+def make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, invariant=False):
+    """Returns (step, bytes_per_step, cleanup-free holder). Weight copies: one quantised master, cloned."""
+    from dromos_amd.abi import DTYPE, F32, FORMATS
+    from dromos_amd.formats import Weight, master_weight, quantize_with
+
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    master = master_weight(N, K, g).cuda()
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    w0 = quantize_with(lx, master, FORMATS[fmt])
+    del master
+    per_copy = w0.nbytes()
+    copies = max(3, -(-(640 << 20) // per_copy))
+    ws = [w0] + [Weight(w0.fmt, w0.data.clone(), None if w0.scale is None else w0.scale.clone(), w0.glob) for _ in range(copies - 1)]
+    structs = [w.lx() for w in ws]
+    ptrs = [ctypes.pointer(s) for s in structs]
+    y = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    nbytes = algorithmic_bytes_gemv(fmt, M, N, K)
+    ws_buf = torch.empty(max(int(lx.size("gemm_workspace_bytes", M, K, 0)), 256), dtype=torch.uint8, device="cuda")
+
+    def step(i):
+        p = ptrs[i % copies]
+        if entry == "gemv_w":
+            st = lx.status("gemv_w", x, DTYPE[x.dtype], K, p, None, F32, y, F32, N, M, N, K, 1.0, 0.0)
+        elif entry == "gemm_skinny":
+            st = lx.status("gemm_skinny", x, DTYPE[x.dtype], K, p, None, F32, y, F32, N, M, N, K, 1.0, 0.0)
+        else:
+            st = lx.status("gemm_w", x, DTYPE[x.dtype], K, p, 0, None, F32, y, F32, N, M, N, K, 1.0, 0.0, ws_buf)
+        assert st == 0, st
+
+    return step, nbytes, (ws, structs, ptrs, x, y, ws_buf)
+
+
+def make_moe_case(lx, torch, fmt, T, E, L, I, top_k, seed, steps_total):
+    """A routed-experts step (route + experts) on bf16 / quantised stacks. Bytes: distinct experts x per-expert
+    bytes, averaged over the steps' seeded routings, + latent + out + routing."""
+    from dromos_amd.abi import FORMATS
+    from dromos_amd.formats import Weight
+
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    copies = 2 if fmt == "bf16" else 3
+    stacks = []
+    for _ in range(copies):
+        gu = (torch.randn(E, 2 * I, L, generator=g) * 0.02).to(torch.bfloat16).cuda()
+        dn = (torch.randn(E, L, I, generator=g) * 0.02).to(torch.bfloat16).cuda()
+        if fmt == "bf16":
+            stacks.append((Weight(0, gu), Weight(0, dn)))
+        else:
+            from dromos_amd.formats import alloc_quantized
+
+            pair = []
+            for w, n, k in ((gu, 2 * I, L), (dn, L, I)):
+                out = alloc_quantized(FORMATS[fmt], E * n, k, "cuda")
+                s = out.lx()
+                lx("quantize_weight", w.view(E * n, k), ctypes.pointer(s), ctypes.c_int64(E * n), k)
+                pair.append(out)
+            stacks.append(tuple(pair))
+    per_expert = (stacks[0][0].nbytes() + stacks[0][1].nbytes()) // E
+    n_routings = max(8, steps_total)
+    logits = torch.randn(n_routings, T, E, generator=g).cuda()
+    latent = torch.randn(T, L, generator=g).to(torch.bfloat16).cuda()
+    ids = torch.empty(n_routings, T, top_k, dtype=torch.int32, device="cuda")
+    weights = torch.empty(n_routings, T, top_k, dtype=torch.float32, device="cuda")
+    ent = torch.empty(T, device="cuda")
+    conf = torch.empty(T, device="cuda")
+    for r in range(n_routings):
+        lx("moe_route", logits[r], None, ids[r], weights[r], ent, conf, T, E, top_k)
+    distinct = sum(len(set(ids[r].flatten().tolist())) for r in range(n_routings)) / n_routings
+    out = torch.empty(T, L, dtype=torch.float32, device="cuda")
+    decode = T <= 8
+    if decode:
+        nws = int(lx.size("moe_decode_workspace_bytes", T, I, top_k))
+    else:
+        fn = lx.lib.lx_moe_grouped_workspace_bytes
+        fn.restype = ctypes.c_int64
+        nws = int(fn(T, L, I, E, top_k, 0))
+    ws = torch.empty(max(nws, 256), dtype=torch.uint8, device="cuda")
+    structs = [(a.lx(), b.lx()) for a, b in stacks]
+    ptrs = [(ctypes.pointer(a), ctypes.pointer(b)) for a, b in structs]
+    nbytes = distinct * per_expert + T * L * 2 + T * L * 4 + T * E * 4 + T * top_k * 8
+
+    def step(i):
+        r = i % n_routings
+        gu, dn = ptrs[i % copies]
+        st = lx.status("moe_route", logits[r], None, ids[r], weights[r], ent, conf, T, E, top_k)
+        assert st == 0, st
+        if decode:
+            st = lx.status("moe_experts_decode", latent, ids[r], weights[r], gu, dn, out, ws, T, L, I, top_k)
+        else:
+            st = lx.status("moe_experts_grouped", latent, ids[r], weights[r], gu, dn, 0, out, ws, T, L, I, E, top_k)
+        assert st == 0, st
+
+    return step, nbytes, (stacks, structs, ptrs, logits, latent, ids, weights, out, ws), distinct
+
+
+def cpu_baseline(torch, fmt, M, N, K, seed, seconds=12.0):
+    """The same GEMV on the host cores: the reference's own CPU backend when oracle/_ref holds it (kind
+    "reference"), else this repository's plain-C restatement (kind "port"). A bounded sample: calls are
+    repeated on rotated weight copies (> 256 MiB, past the last-level cache) for about `seconds`."""
+    from dromos_amd.abi import DTYPE, F32, FORMATS, Kernels
+    from dromos_amd.formats import Weight, master_weight, quantize_with
+
+    threads = min(16, os.cpu_count() or 1)
+    os.environ.setdefault("LX_THREADS", str(threads))
+    os.environ.setdefault("OMP_NUM_THREADS", str(threads))
+    ref = ROOT / "oracle" / "_ref" / "libdromos_cpu.so"
+    port = ROOT / "oracle" / "liboracle.so"
+    if ref.exists():
+        lib, kind = Kernels(ref, "cpu"), "reference"
+    elif port.exists():
+        lib, kind = Kernels(port, "cpu"), "port"
+    else:
+        return None
+    threads = int(os.environ["LX_THREADS"]) if kind == "reference" else int(os.environ["OMP_NUM_THREADS"])
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    master = master_weight(N, K, g)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w0 = quantize_with(lib, master, FORMATS[fmt])
+    copies = max(2, -(-(288 << 20) // w0.nbytes()))
+    ws = [w0] + [Weight(w0.fmt, w0.data.clone(), None if w0.scale is None else w0.scale.clone(), w0.glob) for _ in range(copies - 1)]
+    structs = [w.lx() for w in ws]
+    y = torch.empty(M, N, dtype=torch.float32)
+    nbytes = algorithmic_bytes_gemv(fmt, M, N, K)
+
+    def call(i):
+        st = lib.status("gemv_w", x, DTYPE[x.dtype], K, ctypes.pointer(structs[i % copies]), None, F32, y, F32, N, M, N, K, 1.0, 0.0)
+        assert st == 0
+
+    for i in range(3):
+        call(i)
+    times, i, t_end = [], 3, time.perf_counter() + seconds
+    while time.perf_counter() < t_end and len(times) < 2000:
+        t0 = time.perf_counter()
+        call(i)
+        times.append(time.perf_counter() - t0)
+        i += 1
+    times.sort()
+    med = times[len(times) // 2]
+    return {
+        "value": round(nbytes / med / 1e9, 2),
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": kind,
+        "sample": f"{len(times)} calls of lx_gemv_w {fmt} {N}x{K} M={M} on {copies} rotated weight copies, median {med * 1e6:.0f} us/call, "
+                  f"host has {os.cpu_count()} logical cpus",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--cases", default="headline", choices=["headline", "gemv", "all"])
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported (one MI355X per box)")
+
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no GPU visible")
+    from dromos_amd.abi import load_hip
+
+    lx = load_hip()  # raises when the library is not built: there is no fallback
+    timer = Timer(lx, torch)
+    K_STEPS, W = args.steps, args.warmup
+
+    cases = []
+
+    def run_gemv(name, fmt, M, N, K, seed, entry="gemv_w", invariant=False):
+        if invariant:
+            os.environ["LX_BATCH_INVARIANT"] = "1"
+        else:
+            os.environ.pop("LX_BATCH_INVARIANT", None)
+        step, nbytes, keep = make_gemv_case(lx, torch, fmt, M, N, K, seed, entry)
+        us = timer.run(step, K_STEPS, W)
+        os.environ.pop("LX_BATCH_INVARIANT", None)
+        gbps = nbytes / us / 1e3
+        case = {"case": name, "entry": "lx_" + entry, "format": fmt, "M": M, "N": N, "K": K, "batch_invariant": invariant,
+                "us_per_step": round(us, 3), "bytes_per_step": int(nbytes), "GBps": round(gbps, 1),
+                "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)}
+        cases.append(case)
+        del keep
+        torch.cuda.empty_cache()
+        return case
+
+    def run_moe(name, fmt, T, E, L, I, top_k, seed):
+        step, nbytes, keep, distinct = make_moe_case(lx, torch, fmt, T, E, L, I, top_k, seed, min(K_STEPS + W, 64))
+        us = timer.run(step, K_STEPS, W)
+        gbps = nbytes / us / 1e3
+        case = {"case": name, "entry": "lx_moe_route + lx_moe_experts_" + ("decode" if T <= 8 else "grouped"), "format": fmt,
+                "T": T, "E": E, "L": L, "I": I, "top_k": top_k, "distinct_experts": round(distinct, 2),
+                "us_per_step": round(us, 3), "bytes_per_step": int(nbytes), "GBps": round(gbps, 1),
+                "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)}
+        cases.append(case)
+        del keep
+        torch.cuda.empty_cache()
+        return case
+
+    head = run_gemv("C2 int8 M=1", "int8", 1, 14336, 4096, 1001)
+    if args.cases in ("gemv", "all"):
+        run_gemv("C1 bf16 M=1", "bf16", 1, 4096, 4096, 0)
+        run_gemv("C2 fp8 M=1", "fp8", 1, 14336, 4096, 1001)
+        run_gemv("C3 nvfp4 M=1", "nvfp4", 1, 4096, 14336, 2001)
+        run_gemv("C2 int8 M=4", "int8", 4, 14336, 4096, 1004)
+        run_gemv("C2 fp8 M=4", "fp8", 4, 14336, 4096, 1004)
+        run_gemv("C3 nvfp4 M=8", "nvfp4", 8, 4096, 14336, 2008)
+    if args.cases == "all":
+        for fmt in ("int8", "fp8"):
+            for M in (16, 64):
+                for inv in (False, True):
+                    run_gemv(f"C2 {fmt} M={M}" + (" invariant" if inv else ""), fmt, M, 14336, 4096, 1000 + M, entry="gemm_w", invariant=inv)
+            for M in (1, 4):
+                run_gemv(f"C2 {fmt} M={M} invariant", fmt, M, 14336, 4096, 1000 + M, invariant=True)
+        for T in (1, 8, 32, 64):
+            run_moe(f"C4 moe bf16 T={T}", "bf16", T, 64, 2048, 1024, 8, 3000 + T)
+    elif args.cases == "headline":
+        run_moe("C4 moe bf16 T=1", "bf16", 1, 64, 2048, 1024, 8, 3001)
+
+    result = {
+        "metric": "weight-stream GB/s and % of HBM peak: M=1 GEMV and top-8 MoE decode",
+        "value": head["GBps"],
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": K_STEPS,
+        "warmup": W,
+        "ms_per_step": round(head["us_per_step"] / 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "int8 weights, bf16 activations, f32 accumulate",
+        "data": "synthetic: N(0, 0.02) bf16 masters quantised by lx_quantize_weight, x ~ N(0, 1) bf16, seeded",
+        "config": {"workload": "C2: INT8 weight-only GEMV, W 14336x4096 (per-channel f32 scale), M=1 bf16 x, f32 y, "
+                               "lx_gemv_w on rotated weight copies (> 512 MB)"},
+        "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(head["GBps"] / HBM_PEAK_GBPS, 4), "traffic": load_traffic()},
+        "cases": cases,
+    }
+    if not args.no_cpu:
+        result["cpu_baseline"] = cpu_baseline(torch, "int8", 1, 14336, 4096, 1001)
+    print(json.dumps(result))
+
+
+def load_traffic():
+    """HBM bytes per launch of the headline kernel from the committed rocprofv3 --pmc summary, or None."""
+    p = ROOT / "profiles" / "gemv_w_int8_14336x4096_m1_traffic.json"
+    if not p.exists():
+        return None
+    try:
+        return json.loads(p.read_text()).get("hbm_bytes_per_launch")
+    except (ValueError, OSError):
+        return None
+
+
+if __name__ == "__main__":
+    main()

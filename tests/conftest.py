@@ -58,7 +58,7 @@ def hip():
 
 
 def rel_l2(got, want):
-    got, want = got.double().flatten(), want.double().flatten()
+    got, want = got.double().cpu().flatten(), want.double().cpu().flatten()
     denom = want.norm().item()
     return (got - want).norm().item() / (denom if denom > 0 else 1.0)
 
