@@ -9,14 +9,17 @@
 // workgroup in LDS as f32. When N is too small to give every compute unit rows, S wavefronts of a
 // workgroup share a row's steps (interleaved) and their partial sums are added in wavefront order through
 // LDS. S depends on (format, N, K) only, never on M, so a row's bits are the same for every M.
+#include <stdlib.h>
+
 #include "common.h"
 #include "stream_dot.h"
 
 namespace dro {
 namespace {
 
-constexpr int kThreads = 256;
-constexpr int kWaves = kThreads / kWave;
+constexpr int kThreads = 256;  // the plain kernel's workgroup
+constexpr int kMaxThreads = 1024;  // the streaming kernel's workgroup is chosen per launch, up to this
+constexpr int kMaxWaves = kMaxThreads / kWave;
 constexpr int kLdsFloats = 32 * 1024;  // 128 KB of x at most: one workgroup per compute unit then
 
 struct GemvArgs {
@@ -34,7 +37,14 @@ struct GemvArgs {
   int M, N;
   int64_t K;
   float alpha, beta;
-  int split;  // S: wavefronts sharing a row
+  int split;  // S: wavefronts sharing a row (1, 2 or 4)
+  // Launch geometry, computed once on the host so a wavefront's first load is a few instructions away.
+  int split_log2;
+  int steps;           // wave steps covering K
+  int steps_per_part;  // ceil(steps / S)
+  int chunks;          // 16-byte chunks in a row
+  int64_t row_bytes;
+  int64_t scale_row_bytes;  // NVFP4: bytes of block scales per row
 };
 
 // The epilogue's operation order (engine/cpu/gemm.cpp:21-34).
@@ -47,47 +57,36 @@ __device__ __forceinline__ void write_out(const GemvArgs& a, int wtype, int m, i
   store_from_f32(a.y, a.y_dtype, at, v);
 }
 
-// Row sets are handed to workgroups round-robin; a set is kWaves / S groups of R rows.
+// One workgroup takes blockDim / 64 / S groups of R rows, one group per wavefront (S wavefronts share a
+// group's steps when S > 1), and every wavefront asks for its whole share of the weights (up to two batches of
+// U steps) before anything else: many short-lived wavefronts, each with all its loads in flight, keep the
+// memory system busier than a few long-lived ones.
 template <int F, int MT, int R, int U>
-__global__ void __launch_bounds__(kThreads) gemv_stream_kernel(const GemvArgs a) {
+__global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs a) {
   extern __shared__ __align__(16) float lds[];
-  const int steps = steps_for<F>(a.K);
+  const int steps = a.steps;
   const int per_row = x_row_floats<F>(steps);
   float* xs = lds;
-  float* partial = lds + MT * per_row;  // [kWaves][MT * R] when S > 1
-  stage_x<F, MT>(xs, a.x, a.x_dtype, a.ld_x, nullptr, a.M, a.K, steps);
-  __syncthreads();
+  float* partial = lds + MT * per_row;  // [waves][MT * R] when S > 1
 
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int S = a.split;
-  const int groups_per_set = kWaves / S;
-  const int part = wave % S;  // which share of the steps
-  const int group_in_set = wave / S;
-  const int64_t rb = row_bytes<F>(a.K);
-  const int chunks = static_cast<int>(rb / 16);
-  const int64_t n_groups = (a.N + R - 1) / R;
-  const int64_t n_sets = (n_groups + groups_per_set - 1) / groups_per_set;
-  const int64_t scale_row = F == LX_W_NVFP4 ? a.K / 16 : 0;
+  const int part = wave & (S - 1);  // which share of the steps
+  const int group = blockIdx.x * ((blockDim.x / kWave) >> a.split_log2) + (wave >> a.split_log2);
+  const int64_t rb = a.row_bytes;
+  // Part p of S takes the contiguous steps [p * per, (p + 1) * per).
+  const int s_begin = min(steps, part * a.steps_per_part), s_end = min(steps, s_begin + a.steps_per_part);
 
-  for (int64_t set = blockIdx.x; set < n_sets; set += gridDim.x) {
-    const int64_t group = set * groups_per_set + group_in_set;
-    const int64_t n0 = group * R;
-    const uint8_t* rows[R];
-    const uint8_t* scales[R];
+  auto rows_fn = [&](int g, const uint8_t* (&rows)[R], const uint8_t* (&scales)[R], const float*& x_image) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      int64_t n = n0 + r;
-      if (n > a.N - 1) n = a.N - 1;  // past the end: stream a valid row, write nothing
+      const int64_t n = min(g * R + r, a.N - 1);  // past the end: stream a valid row, write nothing
       rows[r] = a.w + n * rb;
-      scales[r] = a.scale + n * scale_row;
+      scales[r] = a.scale + n * a.scale_row_bytes;
     }
-    float acc[MT][R];
-    {
-      // Part p of S takes the contiguous steps [p * per, (p + 1) * per).
-      const int per = (steps + S - 1) / S;
-      const int s_begin = min(steps, part * per), s_end = min(steps, s_begin + per);
-      stream_rows<F, MT, R, U>(rows, scales, chunks, s_begin, s_end, xs, per_row, acc);
-    }
+    x_image = xs;
+  };
+  auto done_fn = [&](int g, float (&acc)[MT][R]) {
 #pragma unroll
     for (int m = 0; m < MT; ++m)
 #pragma unroll
@@ -110,16 +109,30 @@ __global__ void __launch_bounds__(kThreads) gemv_stream_kernel(const GemvArgs a)
             acc[m][r] = s;
           }
       }
-      __syncthreads();
     }
     if (lane == 0 && part == 0) {
 #pragma unroll
       for (int m = 0; m < MT; ++m)
 #pragma unroll
         for (int r = 0; r < R; ++r)
-          if (m < a.M && n0 + r < a.N) write_out(a, F, m, n0 + r, acc[m][r]);
+          if (m < a.M && g * R + r < a.N) write_out(a, F, m, static_cast<int64_t>(g) * R + r, acc[m][r]);
     }
+  };
+
+  RowStreamer<F, MT, R, U> st(a.chunks, s_begin, s_end, per_row);
+  if constexpr (MT == 1) {
+    // Ask for x, then for the weights, and only then wait for x: loads return in order.
+    XRegs xr;
+    stage_x_load<F>(xr, a.x, a.x_dtype, a.ld_x, a.K, steps);
+    st.prefetch(rows_fn, group, 0, 1);
+    if (xr.ready) stage_x_store<F>(xr, xs, a.x_dtype, steps);
+    else stage_x<F, MT>(xs, a.x, a.x_dtype, a.ld_x, nullptr, a.M, a.K, steps);
+  } else {
+    st.prefetch(rows_fn, group, 0, 1);
+    stage_x<F, MT>(xs, a.x, a.x_dtype, a.ld_x, nullptr, a.M, a.K, steps);
   }
+  __syncthreads();
+  st.run(rows_fn, done_fn, group, 0, 1);
 }
 
 // Any K, any alignment, x read where it lies: one wavefront per output row, lanes striding over k, the
@@ -127,7 +140,7 @@ __global__ void __launch_bounds__(kThreads) gemv_stream_kernel(const GemvArgs a)
 // (the choice depends on K and the weight's address only, never on M).
 __global__ void __launch_bounds__(kThreads) gemv_plain_kernel(const GemvArgs a, int wtype) {
   const int lane = threadIdx.x & (kWave - 1);
-  const int64_t n = static_cast<int64_t>(blockIdx.x) * kWaves + threadIdx.x / kWave;
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * (kThreads / kWave) + threadIdx.x / kWave;
   if (n >= a.N) return;
   float acc[8];
 #pragma unroll
@@ -152,30 +165,36 @@ int order_class(int N, int64_t K, int R) {
   const int cus = compute_units();
   int S = 1;
   // Fewer row groups than wavefront slots the device wants busy: let wavefronts share rows.
-  while (S < kWaves && (static_cast<int64_t>(N) + R - 1) / R * S < 2LL * cus && steps >= 2 * S) S *= 2;
+  while (S < 4 && (static_cast<int64_t>(N) + R - 1) / R * S < 2LL * cus && steps >= 2 * S) S *= 2;
   return S;
 }
 
-template <int F>
-constexpr int rows_per_wave() {
-  return 2;
-}
-template <int F>
-constexpr int loads_in_flight() {
-  return F == LX_W_NVFP4 ? 2 : 4;
+// How a launch is shaped. None of it changes an output's bits (only S does).
+struct Shape {
+  int threads;  // workgroup size
+  int ru;       // which (R, U) instance
+};
+
+Shape shape_for(int wtype, int M) {
+  // Measured on MI355X at the decode shapes: a wavefront should own about 8 KB of weights, all requested at once.
+  Shape s{256, 1};
+  if (M == 1) {
+    if (wtype == LX_W_BF16) s = Shape{256, 2};        // one row, eight steps in flight
+    else if (wtype == LX_W_NVFP4) s = Shape{512, 2};  // long rows of few bytes: more wavefronts per x image
+    else s = Shape{256, 1};                           // two rows, four steps each
+  }
+  if (const char* e = getenv("DRO_GEMV_THREADS")) s.threads = atoi(e);
+  if (const char* e = getenv("DRO_GEMV_RU")) s.ru = atoi(e);
+  return s;
 }
 
-template <int F, int MT>
-int launch_stream(const GemvArgs& a, hipStream_t stream) {
-  constexpr int R = rows_per_wave<F>(), U = loads_in_flight<F>();
-  const int steps = steps_for<F>(a.K);
-  const size_t lds = sizeof(float) * (static_cast<size_t>(MT) * x_row_floats<F>(steps) + kWaves * MT * R);
-  const int groups_per_set = kWaves / a.split;
+template <int F, int MT, int R, int U>
+int launch_stream(GemvArgs a, const Shape& shape, hipStream_t stream) {
+  const int waves = shape.threads / kWave;
+  const size_t lds = sizeof(float) * (static_cast<size_t>(MT) * x_row_floats<F>(a.steps) + waves * MT * R);
+  const int groups_per_wg = waves / a.split;
   const int64_t n_groups = (a.N + R - 1) / R;
-  const int64_t n_sets = (n_groups + groups_per_set - 1) / groups_per_set;
-  const int per_cu = lds <= 64 * 1024 ? 2 : 1;
-  const int64_t cap = static_cast<int64_t>(compute_units()) * per_cu;
-  const unsigned grid = static_cast<unsigned>(n_sets < cap ? n_sets : cap);
+  const int64_t grid = (n_groups + groups_per_wg - 1) / groups_per_wg;
   auto kernel = gemv_stream_kernel<F, MT, R, U>;
   if (lds > 48 * 1024) {
     static thread_local bool raised = false;
@@ -186,13 +205,29 @@ int launch_stream(const GemvArgs& a, hipStream_t stream) {
       raised = true;
     }
   }
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(kThreads), lds, stream, a);
+  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(shape.threads), lds, stream, a);
   return status_of(hipGetLastError());
+}
+
+template <int F, int MT>
+int launch_rows(const GemvArgs& a, const Shape& shape, hipStream_t stream) {
+  if constexpr (MT == 1) {
+    switch (shape.ru) {
+      case 0: return launch_stream<F, 1, 1, 4>(a, shape, stream);
+      case 2: return launch_stream<F, 1, 1, 8>(a, shape, stream);
+      case 3: return launch_stream<F, 1, 2, 2>(a, shape, stream);
+      case 4: return launch_stream<F, 1, 4, 2>(a, shape, stream);
+      case 5: return launch_stream<F, 1, 2, 8>(a, shape, stream);
+      default: return launch_stream<F, 1, 2, 4>(a, shape, stream);
+    }
+  } else {
+    return launch_stream<F, MT, 2, (F == LX_W_NVFP4 ? 2 : 4)>(a, shape, stream);
+  }
 }
 
 template <int F>
 int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
-  constexpr int R = rows_per_wave<F>();
+  constexpr int R = 2;  // the order class counts row groups of two
   const int64_t rb = row_bytes<F>(a.K);
   const int steps = steps_for<F>(a.K);
   const bool vector_rows = rb % 16 == 0 && reinterpret_cast<uintptr_t>(a.w) % 16 == 0 &&
@@ -200,15 +235,22 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
   // Activation rows a pass can hold in LDS: a function of K only. More rows than that run as several
   // passes over the weights; each row's arithmetic is the same in any pass, so its bits do not change.
   int fit = 8;
-  while (fit >= 1 && static_cast<int64_t>(fit) * x_row_floats<F>(steps) + kWaves * fit * R > kLdsFloats) fit /= 2;
+  while (fit >= 1 && static_cast<int64_t>(fit) * x_row_floats<F>(steps) + kMaxWaves * fit * 4 > kLdsFloats) fit /= 2;
   if (!vector_rows || fit < 1) {
-    const unsigned grid = static_cast<unsigned>((a.N + kWaves - 1) / kWaves);
+    const int waves = kThreads / kWave;
+    const unsigned grid = static_cast<unsigned>((a.N + waves - 1) / waves);
     hipLaunchKernelGGL(gemv_plain_kernel, dim3(grid), dim3(kThreads), 0, stream, a, F);
     return status_of(hipGetLastError());
   }
   a.split = order_class<F>(a.N, a.K, R);
   const int tuned = tuned_variant(kernel_name, a.M, a.N, static_cast<int>(a.K));
   if (tuned >= 0 && tuned <= 2) a.split = 1 << tuned;
+  a.split_log2 = a.split == 4 ? 2 : a.split == 2 ? 1 : 0;
+  a.steps = steps;
+  a.steps_per_part = (steps + a.split - 1) / a.split;
+  a.chunks = static_cast<int>(rb / 16);
+  a.row_bytes = rb;
+  a.scale_row_bytes = F == LX_W_NVFP4 ? a.K / 16 : 0;
   const int M = a.M;
   const char* x0 = static_cast<const char*>(a.x);
   char* y0 = static_cast<char*>(a.y);
@@ -218,12 +260,13 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
     a.x = x0 + m0 * x_row;
     a.y = y0 + m0 * y_row;
     const int mt = a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : 8;
+    const Shape shape = shape_for(F, a.M);
     int st;
     switch (mt) {
-      case 1: st = launch_stream<F, 1>(a, stream); break;
-      case 2: st = launch_stream<F, 2>(a, stream); break;
-      case 4: st = launch_stream<F, 4>(a, stream); break;
-      default: st = launch_stream<F, 8>(a, stream); break;
+      case 1: st = launch_rows<F, 1>(a, shape, stream); break;
+      case 2: st = launch_rows<F, 2>(a, shape, stream); break;
+      case 4: st = launch_rows<F, 4>(a, shape, stream); break;
+      default: st = launch_rows<F, 8>(a, shape, stream); break;
     }
     if (st) return st;
   }
@@ -238,10 +281,10 @@ bool valid_dtype(int d) { return d == LX_F32 || d == LX_BF16; }
 bool gemv_admits(int wtype, int variant, int N, int K) {
   int S = 1;
   switch (wtype) {
-    case LX_W_BF16: S = order_class<LX_W_BF16>(N, K, rows_per_wave<LX_W_BF16>()); break;
-    case LX_W_INT8: S = order_class<LX_W_INT8>(N, K, rows_per_wave<LX_W_INT8>()); break;
-    case LX_W_FP8: S = order_class<LX_W_FP8>(N, K, rows_per_wave<LX_W_FP8>()); break;
-    default: S = order_class<LX_W_NVFP4>(N, K, rows_per_wave<LX_W_NVFP4>()); break;
+    case LX_W_BF16: S = order_class<LX_W_BF16>(N, K, 2); break;
+    case LX_W_INT8: S = order_class<LX_W_INT8>(N, K, 2); break;
+    case LX_W_FP8: S = order_class<LX_W_FP8>(N, K, 2); break;
+    default: S = order_class<LX_W_NVFP4>(N, K, 2); break;
   }
   return (1 << variant) == S;
 }

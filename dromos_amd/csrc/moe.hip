@@ -26,7 +26,7 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
                                                          float* __restrict__ entropy, float* __restrict__ confidence, int T,
                                                          int E, int top_k) {
   __shared__ float picked_logit[kWaves][64];
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int64_t t = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
   if (t >= T) return;
   const float* row = logits + t * E;
@@ -150,28 +150,33 @@ __device__ __forceinline__ void group_pairs(const int32_t* ids, int P, int slot,
 // Intermediate rows [i_begin, i_end) of expert e for the cnt <= MT pairs at sorted positions first..: each
 // wavefront takes rows i = i_begin + wave, + kWaves, ...; the pair (gate row i, up row I + i) is its two
 // streamed rows. MT only sets how many activation rows share a pass; a row's arithmetic is the same for any MT.
+// Stages the pairs' latent rows itself (after asking for the first weights), so the whole workgroup calls it.
 template <int F, int U, int MT>
-__device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, const float* lds, int e, int first, int cnt, const int* s_order,
-                                             int i_begin, int i_end) {
+__device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, int e, int first, int cnt, const int* s_order,
+                                             const int* s_rows, int i_begin, int i_end) {
   const int steps = steps_for<F>(a.L);
   const int per_row = x_row_floats<F>(steps);
   const int64_t rb = row_bytes<F>(a.L);
   const int chunks = static_cast<int>(rb / 16);
   const int64_t scale_row = F == LX_W_NVFP4 ? a.L / 16 : 0;
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int64_t stack_row0 = static_cast<int64_t>(e) * 2 * a.I;
-  for (int i = i_begin + wave; i < i_end; i += kWaves) {
-    const int64_t gate_row = stack_row0 + i, up_row = stack_row0 + a.I + i;
-    const uint8_t* rows[2] = {a.gu.data + gate_row * rb, a.gu.data + up_row * rb};
-    const uint8_t* scales[2] = {a.gu.scale + gate_row * scale_row, a.gu.scale + up_row * scale_row};
-    float acc[MT][2];
-    stream_rows<F, MT, 2, U>(rows, scales, chunks, 0, steps, lds, per_row, acc);
+  auto rows_fn = [&](int i, const uint8_t* (&rows)[2], const uint8_t* (&scales)[2], const float*& x_image) {
+    const int64_t gate_row = stack_row0 + min(i, a.I - 1), up_row = gate_row + a.I;
+    rows[0] = a.gu.data + gate_row * rb;
+    rows[1] = a.gu.data + up_row * rb;
+    scales[0] = a.gu.scale + gate_row * scale_row;
+    scales[1] = a.gu.scale + up_row * scale_row;
+    x_image = lds;
+  };
+  auto done_fn = [&](int i, float (&acc)[MT][2]) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       acc[m][0] = wave_sum(acc[m][0]);
       acc[m][1] = wave_sum(acc[m][1]);
     }
     if (lane == 0) {
+      const int64_t gate_row = stack_row0 + i, up_row = gate_row + a.I;
       const float sg = stack_factor(F, a.gu, e, gate_row), su = stack_factor(F, a.gu, e, up_row);
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
@@ -182,7 +187,14 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, const float* l
         }
       }
     }
-  }
+  };
+  RowStreamer<F, MT, 2, U> st(chunks, 0, steps, per_row);
+  const int first_i = i_begin + wave;
+  const int n = first_i < i_end ? (i_end - first_i + kWaves - 1) / kWaves : 0;
+  if (n > 0) st.prefetch(rows_fn, first_i, kWaves, n);
+  stage_x<F, MT>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
+  __syncthreads();
+  st.run(rows_fn, done_fn, first_i, kWaves, n);
 }
 
 // grid = (row blocks, group slots); mt_cap (a power of two, the LDS image's rows) bounds a pass's pairs.
@@ -195,93 +207,78 @@ __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeAr
   if (static_cast<int>(blockIdx.y) >= s_info[0]) return;
   const int begin = s_info[1], end = s_info[2];
   const int e = s_ids[s_order[begin]];
-  const int steps = steps_for<F>(a.L);
   const int rows_per_block = (a.I + gridDim.x - 1) / gridDim.x;
   const int i_begin = blockIdx.x * rows_per_block, i_end = min(a.I, i_begin + rows_per_block);
   // A group larger than the image (an expert repeated within a token) runs mt_cap pairs at a time.
   for (int first = begin; first < end; first += mt_cap) {
     const int cnt = min(mt_cap, end - first);
     __syncthreads();
-    if (threadIdx.x < 8) s_rows[threadIdx.x] = threadIdx.x < cnt ? s_order[first + threadIdx.x] / a.top_k : 0;
+    if (threadIdx.x < 8) s_rows[threadIdx.x] = static_cast<int>(threadIdx.x) < cnt ? s_order[first + threadIdx.x] / a.top_k : 0;
     __syncthreads();
-    if (cnt <= 1) {
-      stage_x<F, 1>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
-      __syncthreads();
-      gate_up_rows<F, U, 1>(a, lds, e, first, cnt, s_order, i_begin, i_end);
-    } else if (cnt <= 2) {
-      stage_x<F, 2>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
-      __syncthreads();
-      gate_up_rows<F, U, 2>(a, lds, e, first, cnt, s_order, i_begin, i_end);
-    } else if (cnt <= 4) {
-      stage_x<F, 4>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
-      __syncthreads();
-      gate_up_rows<F, U, 4>(a, lds, e, first, cnt, s_order, i_begin, i_end);
-    } else {
-      stage_x<F, 8>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
-      __syncthreads();
-      gate_up_rows<F, U, 8>(a, lds, e, first, cnt, s_order, i_begin, i_end);
-    }
+    if (cnt <= 1) gate_up_rows<F, U, 1>(a, lds, e, first, cnt, s_order, s_rows, i_begin, i_end);
+    else if (cnt <= 2) gate_up_rows<F, U, 2>(a, lds, e, first, cnt, s_order, s_rows, i_begin, i_end);
+    else if (cnt <= 4) gate_up_rows<F, U, 4>(a, lds, e, first, cnt, s_order, s_rows, i_begin, i_end);
+    else gate_up_rows<F, U, 8>(a, lds, e, first, cnt, s_order, s_rows, i_begin, i_end);
   }
 }
 
 // grid = (blocks of output rows, T). x = the token's top_k intermediate rows; slot k streams expert
 // ids[t, k]'s down rows. out[t, l] = w0 * c0 + sum_{k >= 1} w_k * c_k in slot order
-// (engine/cpu/moe.cpp:315-327), c_k = rowfactor * dot.
+// (engine/cpu/moe.cpp:315-327), c_k = rowfactor * dot. A wavefront's stream is, for each of its pairs of
+// output rows in turn, the top_k experts' copies of those two rows.
 template <int F, int U>
 __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs a) {
   extern __shared__ __align__(16) float lds[];
   __shared__ int s_rows[8];
+  constexpr int R = 2;
   const int t = blockIdx.y;
   const int steps = steps_for<F>(a.I);
   const int per_row = x_row_floats<F>(steps);
   const int64_t rb = row_bytes<F>(a.I);
   const int chunks = static_cast<int>(rb / 16);
   const int64_t scale_row = F == LX_W_NVFP4 ? a.I / 16 : 0;
-  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
-  if (threadIdx.x < 8) s_rows[threadIdx.x] = t * a.top_k + min(static_cast<int>(threadIdx.x), a.top_k - 1);
-  __syncthreads();
-  stage_x<F, 8>(lds, a.inter, LX_BF16, a.I, s_rows, a.top_k, a.I, steps);
-  __syncthreads();
-  constexpr int R = 2;
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int top_k = a.top_k;
   const int groups = (a.L + R - 1) / R;
   const int groups_per_block = (groups + gridDim.x - 1) / gridDim.x;
   const int g_begin = blockIdx.x * groups_per_block, g_end = min(groups, g_begin + groups_per_block);
-  for (int grp = g_begin + wave; grp < g_end; grp += kWaves) {
-    const int l0 = grp * R;
-    float sums[8][R];
-#pragma unroll
-    for (int k = 0; k < 8; ++k) {
-      if (k < a.top_k) {
-        const int e = a.ids[t * a.top_k + k];
-        const uint8_t* rows[R];
-        const uint8_t* scales[R];
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          const int64_t row = static_cast<int64_t>(e) * a.L + min(l0 + r, a.L - 1);
-          rows[r] = a.dn.data + row * rb;
-          scales[r] = a.dn.scale + row * scale_row;
-        }
-        float acc[1][R];
-        stream_rows<F, 1, R, U>(rows, scales, chunks, 0, steps, lds + k * per_row, per_row, acc);
-#pragma unroll
-        for (int r = 0; r < R; ++r) sums[k][r] = acc[0][r];
-      }
-    }
+  const int first_g = g_begin + wave;
+  const int n_mine = first_g < g_end ? (g_end - first_g + kWaves - 1) / kWaves : 0;
+
+  // Stream position c = (j-th pair of rows of this wavefront, slot k).
+  auto rows_fn = [&](int c, const uint8_t* (&rows)[R], const uint8_t* (&scales)[R], const float*& x_image) {
+    const int j = c / top_k, k = c - j * top_k;
+    const int l0 = (first_g + j * kWaves) * R;
+    const int e = a.ids[t * top_k + k];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      float o = 0.0f;
-#pragma unroll
-      for (int k = 0; k < 8; ++k) {
-        if (k < a.top_k) {
-          const int e = a.ids[t * a.top_k + k];
-          const float c = stack_factor(F, a.dn, e, static_cast<int64_t>(e) * a.L + min(l0 + r, a.L - 1)) * wave_sum(sums[k][r]);
-          const float wc = a.weights[t * a.top_k + k] * c;
-          o = k == 0 ? wc : o + wc;
-        }
-      }
-      if (lane == 0 && l0 + r < a.L) a.out[static_cast<int64_t>(t) * a.L + l0 + r] = o;
+      const int64_t row = static_cast<int64_t>(e) * a.L + min(l0 + r, a.L - 1);
+      rows[r] = a.dn.data + row * rb;
+      scales[r] = a.dn.scale + row * scale_row;
     }
-  }
+    x_image = lds + k * per_row;
+  };
+  float o[R] = {0.0f, 0.0f};
+  auto done_fn = [&](int c, float (&acc)[1][R]) {
+    const int j = c / top_k, k = c - j * top_k;
+    const int l0 = (first_g + j * kWaves) * R;
+    const int e = a.ids[t * top_k + k];
+    const float w = a.weights[t * top_k + k];
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const float contrib = stack_factor(F, a.dn, e, static_cast<int64_t>(e) * a.L + min(l0 + r, a.L - 1)) * wave_sum(acc[0][r]);
+      const float wc = w * contrib;
+      o[r] = k == 0 ? wc : o[r] + wc;
+      if (k == top_k - 1 && lane == 0 && l0 + r < a.L) a.out[static_cast<int64_t>(t) * a.L + l0 + r] = o[r];
+    }
+  };
+  RowStreamer<F, 1, R, U> st(chunks, 0, steps, per_row);
+  if (n_mine > 0) st.prefetch(rows_fn, 0, 1, n_mine * top_k);
+  if (threadIdx.x < 8) s_rows[threadIdx.x] = t * top_k + min(static_cast<int>(threadIdx.x), top_k - 1);
+  __syncthreads();
+  stage_x<F, 8>(lds, a.inter, LX_BF16, a.I, s_rows, top_k, a.I, steps);
+  __syncthreads();
+  st.run(rows_fn, done_fn, 0, 1, n_mine * top_k);
 }
 
 // Rows whose bytes cannot be streamed 16 at a time (K not a multiple of the chunk, or a misaligned stack):

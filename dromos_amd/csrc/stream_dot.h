@@ -1,15 +1,20 @@
 // The weight-streaming dot product shared by the decode GEMV and the decode experts.
 //
-// A wavefront owns R weight rows at a time and streams them whole: at step s, lane l reads the 16 bytes
-// at chunk s * 64 + l of each row (one 128-bit non-temporal load, 1 KB contiguous per row per wave), so a
-// row's bytes are read exactly once, in order. The activations sit in LDS as f32, laid out so that the
-// 16 bytes a lane reads next are always 16 bytes after its neighbour's (no bank conflicts): the k values
-// of chunk (s, l) are stored as kElems / 4 groups of four, group q at float index
-//   s * 64 * kElems + q * 256 + l * 4.
-// Every (activation row, weight row) pair keeps one f32 accumulator per lane, fed in ascending step
-// order, and the 64 lane sums are combined by one fixed tree (wave_sum). The order never depends on how
-// many activation rows share the pass (MT) or how many weight rows the wave holds (R), so an output's
-// bits depend only on its own x row, its weight row and the K split.
+// A wavefront owns R weight rows at a time (a "group") and streams them whole: at step s, lane l reads the
+// 16 bytes at chunk s * 64 + l of each row (one 128-bit non-temporal load, 1 KB contiguous per row per
+// wave), so a row's bytes are read exactly once, in order. Loads run one batch (U steps of R rows) ahead of
+// the arithmetic in a second register buffer, across group boundaries too, so a wavefront always has a
+// batch in flight while it multiplies the previous one.
+//
+// The activations sit in LDS as f32, laid out so that the 16 bytes a lane reads next are always 16 bytes
+// after its neighbour's (no bank conflicts): the k values of chunk (s, l) are stored as kElems / 4 groups of
+// four, group q at float index  s * 64 * kElems + q * 256 + l * 4.  The image is zero past K, so a lane
+// whose chunk lies past the end of the row (its load is clamped to the row's last chunk) adds exact zeros.
+//
+// Every (activation row, weight row) pair keeps one f32 accumulator per lane, fed in ascending step order,
+// and the 64 lane sums are combined by one fixed tree (wave_sum). The order never depends on how many
+// activation rows share the pass (MT), how many weight rows the wave holds (R) or the batch depth (U), so an
+// output's bits depend only on its own x row, its weight row and the K split.
 #pragma once
 
 #include "common.h"
@@ -38,23 +43,134 @@ __host__ __device__ inline int steps_for(int64_t K) {
 
 // Stages rows [0, M) of x (f32 or bf16, row stride ld_x, optionally gathered through row_of[m]) into the
 // LDS image `xs` for MT rows of `steps` steps each; everything past K, and rows M .. MT - 1, are zero.
-// Called by the whole workgroup; the caller synchronises afterwards.
+// Called by the whole workgroup; the caller synchronises afterwards. Rows whose address and stride allow it
+// are read 16 bytes at a time, several loads in flight per thread (K is a multiple of 8 whenever the weight
+// rows are streamed, so a vector never straddles the end of a row).
 template <int F, int MT>
 __device__ __forceinline__ void stage_x(float* xs, const void* x, int x_dtype, int64_t ld_x, const int* row_of, int M,
                                         int64_t K, int steps) {
   constexpr int E = Fmt<F>::kElems;
   const int per_row = steps * kWave * E;
+  const int esize = x_dtype == LX_BF16 ? 2 : 4;
+  const bool vec = reinterpret_cast<uintptr_t>(x) % 16 == 0 && (ld_x * esize) % 16 == 0 && K % 8 == 0;
   for (int m = 0; m < MT; ++m) {
     float* dst = xs + m * per_row;
     if (m >= M) {
-      for (int i = threadIdx.x; i < per_row; i += blockDim.x) dst[i] = 0.0f;
+      for (int i = threadIdx.x * 4; i < per_row; i += blockDim.x * 4) *reinterpret_cast<f32x4*>(dst + i) = f32x4{0.f, 0.f, 0.f, 0.f};
       continue;
     }
     const int64_t base = static_cast<int64_t>(row_of ? row_of[m] : m) * ld_x;
-    for (int k = threadIdx.x; k < per_row; k += blockDim.x) {
-      const float v = k < K ? load_as_f32(x, x_dtype, base + k) : 0.0f;
-      const int s = k / (kWave * E), within = k % (kWave * E);
-      dst[x_slot<F>(s, within / E, within % E)] = v;
+    if (vec && x_dtype == LX_BF16) {
+      const u32x4* src = reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(x) + base);
+      const int n_vec = per_row / 8, k_vec = static_cast<int>(K / 8);
+      for (int v0 = threadIdx.x; v0 < n_vec; v0 += blockDim.x * 4) {
+        u32x4 r[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int v = v0 + u * blockDim.x;
+          r[u] = v < k_vec ? src[v] : u32x4{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int v = v0 + u * blockDim.x;
+          if (v < n_vec) {
+            const int k = v * 8, s = k / (kWave * E), within = k % (kWave * E);
+            float* at = dst + x_slot<F>(s, within / E, within % E);
+            *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(r[u].x << 16), __uint_as_float(r[u].x & 0xffff0000u),
+                                                  __uint_as_float(r[u].y << 16), __uint_as_float(r[u].y & 0xffff0000u)};
+            *reinterpret_cast<f32x4*>(at + 256) = f32x4{__uint_as_float(r[u].z << 16), __uint_as_float(r[u].z & 0xffff0000u),
+                                                        __uint_as_float(r[u].w << 16), __uint_as_float(r[u].w & 0xffff0000u)};
+          }
+        }
+      }
+    } else if (vec) {
+      const f32x4* src = reinterpret_cast<const f32x4*>(static_cast<const float*>(x) + base);
+      const int n_vec = per_row / 4, k_vec = static_cast<int>(K / 4);
+      for (int v0 = threadIdx.x; v0 < n_vec; v0 += blockDim.x * 4) {
+        f32x4 r[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int v = v0 + u * blockDim.x;
+          r[u] = v < k_vec ? src[v] : f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int v = v0 + u * blockDim.x;
+          if (v < n_vec) {
+            const int k = v * 4, s = k / (kWave * E), within = k % (kWave * E);
+            *reinterpret_cast<f32x4*>(dst + x_slot<F>(s, within / E, within % E)) = r[u];
+          }
+        }
+      }
+    } else {
+      for (int k0 = threadIdx.x; k0 < per_row; k0 += blockDim.x * 8) {
+        float r[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int k = k0 + u * blockDim.x;
+          r[u] = k < K ? load_as_f32(x, x_dtype, base + k) : 0.0f;
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+          const int k = k0 + u * blockDim.x;
+          if (k < per_row) {
+            const int s = k / (kWave * E), within = k % (kWave * E);
+            dst[x_slot<F>(s, within / E, within % E)] = r[u];
+          }
+        }
+      }
+    }
+  }
+}
+
+// The same staging in two phases for one activation row, so a kernel can ask for x, then for its first
+// weights, and only then wait for x: XRegs holds a thread's share of the row between the two calls. Usable
+// when the row can be read 16 bytes at a time and a thread's share is at most kVecs vectors; otherwise
+// `ready` is false and the caller falls back to stage_x.
+struct XRegs {
+  static constexpr int kVecs = 4;
+  u32x4 v[kVecs];
+  bool ready;
+};
+
+template <int F>
+__device__ __forceinline__ void stage_x_load(XRegs& r, const void* x, int x_dtype, int64_t ld_x, int64_t K, int steps) {
+  constexpr int E = Fmt<F>::kElems;
+  const int per_row = steps * kWave * E;
+  const int vec_shift = x_dtype == LX_BF16 ? 3 : 2;  // elements per 16-byte vector: 8 or 4
+  const int n_vec = per_row >> vec_shift, k_vec = static_cast<int>(K) >> vec_shift;
+  r.ready = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && ((ld_x << (4 - vec_shift)) & 15) == 0 && (K & 7) == 0 &&
+            n_vec <= XRegs::kVecs * static_cast<int>(blockDim.x);
+  if (!r.ready) return;
+  const u32x4* src = static_cast<const u32x4*>(x);
+#pragma unroll
+  for (int u = 0; u < XRegs::kVecs; ++u) {
+    const int v = threadIdx.x + u * blockDim.x;
+    r.v[u] = v < k_vec ? src[v] : u32x4{0u, 0u, 0u, 0u};
+  }
+}
+
+template <int F>
+__device__ __forceinline__ void stage_x_store(const XRegs& r, float* xs, int x_dtype, int steps) {
+  constexpr int E = Fmt<F>::kElems;
+  const int per_row = steps * kWave * E;
+  const int vec_shift = x_dtype == LX_BF16 ? 3 : 2;
+  const int n_vec = per_row >> vec_shift;
+#pragma unroll
+  for (int u = 0; u < XRegs::kVecs; ++u) {
+    const int v = threadIdx.x + u * blockDim.x;
+    if (v < n_vec) {
+      const int k = v << vec_shift, s = k / (kWave * E), within = k % (kWave * E);
+      float* at = xs + x_slot<F>(s, within / E, within % E);
+      if (x_dtype == LX_BF16) {
+        *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(r.v[u].x << 16), __uint_as_float(r.v[u].x & 0xffff0000u),
+                                              __uint_as_float(r.v[u].y << 16), __uint_as_float(r.v[u].y & 0xffff0000u)};
+        *reinterpret_cast<f32x4*>(at + 256) = f32x4{__uint_as_float(r.v[u].z << 16), __uint_as_float(r.v[u].z & 0xffff0000u),
+                                                    __uint_as_float(r.v[u].w << 16), __uint_as_float(r.v[u].w & 0xffff0000u)};
+      } else {
+        *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(r.v[u].x), __uint_as_float(r.v[u].y), __uint_as_float(r.v[u].z),
+                                              __uint_as_float(r.v[u].w)};
+      }
     }
   }
 }
@@ -67,16 +183,10 @@ struct Chunk {
 };
 
 template <int F>
-__device__ __forceinline__ Chunk<F> load_chunk(const uint8_t* row, const uint8_t* row_scales, int chunk, bool valid) {
-  Chunk<F> c;
-  c.w = u32x4{0u, 0u, 0u, 0u};
-  c.scales = 0u;
-  if (valid) {
-    c.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row) + chunk);
-    if constexpr (F == LX_W_NVFP4)
-      c.scales = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(row_scales) + chunk);
-  }
-  return c;
+__device__ __forceinline__ void load_chunk(Chunk<F>& c, const uint8_t* row, const uint8_t* row_scales, int chunk) {
+  c.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row) + chunk);
+  if constexpr (F == LX_W_NVFP4)
+    c.scales = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(row_scales) + chunk);
 }
 
 // acc[m] += sum over the chunk's k of x[m, k] * w[k], for MT activation rows; xs points at the LDS image of
@@ -140,43 +250,112 @@ __device__ __forceinline__ void chunk_fma(const Chunk<F>& c, const float* xs, in
   }
 }
 
-// acc[m][r] = sum_k x[m, k] * row_r[k] over steps [s_begin, s_end) of R rows, U steps of loads in flight.
-// rows[r] / scales[r] point at the rows' first bytes; a row has `chunks` 16-byte chunks. Lane sums only:
-// the caller reduces across the wave.
+// Streams a sequence of groups of R rows through a wavefront.
+//
+//   RowStreamer<F, MT, R, U> st(chunks, s_begin, s_end, per_row);
+//   st.prefetch(rows_fn, first_group, group_stride, n_groups);   // weights do not depend on x: ask first
+//   ... stage x in LDS, __syncthreads() ...
+//   st.run(rows_fn, done_fn, first_group, group_stride, n_groups);
+//
+// rows_fn(group, rows, scales, xs) fills the R row pointers (and NVFP4 scale rows) of group `group` and the
+// LDS image its products read; done_fn(group, acc) receives the lane sums acc[MT][R] of a finished group (the
+// caller reduces them across the wave). Steps [s_begin, s_end) of every row are taken, in batches of U.
 template <int F, int MT, int R, int U>
-__device__ __forceinline__ void stream_rows(const uint8_t* const (&rows)[R], const uint8_t* const (&scales)[R],
-                                            int chunks, int s_begin, int s_end, const float* xs, int per_row,
-                                            float (&acc)[MT][R]) {
-  const int lane = threadIdx.x & (kWave - 1);
-#pragma unroll
-  for (int m = 0; m < MT; ++m)
-#pragma unroll
-    for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
-  for (int s0 = s_begin; s0 < s_end; s0 += U) {
-    Chunk<F> c[U][R];
+struct RowStreamer {
+  Chunk<F> buf_a[U][R], buf_b[U][R];
+  int chunks, s_begin, s_end, per_row, batches, lane;
+
+  __device__ __forceinline__ RowStreamer(int chunks_, int s_begin_, int s_end_, int per_row_)
+      : chunks(chunks_), s_begin(s_begin_), s_end(s_end_), per_row(per_row_) {
+    const int n = s_end - s_begin;
+    batches = n > 0 ? (n + U - 1) / U : 1;
+    lane = threadIdx.x & (kWave - 1);
+  }
+
+  template <class RowsFn>
+  __device__ __forceinline__ void issue(Chunk<F> (&buf)[U][R], RowsFn& rows_fn, int group, int batch) {
+    const uint8_t* rows[R];
+    const uint8_t* scales[R];
+    const float* xs;
+    rows_fn(group, rows, scales, xs);
+    const int last_step = s_end > s_begin ? s_end - 1 : s_begin;
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      const int chunk = (s0 + u) * kWave + lane;
-      const bool valid = s0 + u < s_end && chunk < chunks;
+      // A step past the range, or a chunk past the row's end, re-reads a valid chunk; it is never multiplied
+      // (the step is skipped) or multiplies zeros (the x image is zero there).
+      const int s = min(s_begin + batch * U + u, last_step);
+      const int chunk = min(s * kWave + lane, chunks - 1);
 #pragma unroll
-      for (int r = 0; r < R; ++r) c[u][r] = load_chunk<F>(rows[r], scales[r], chunk, valid);
+      for (int r = 0; r < R; ++r) load_chunk<F>(buf[u][r], rows[r], scales[r], chunk);
     }
+  }
+
+  __device__ __forceinline__ void consume(const Chunk<F> (&buf)[U][R], const float* xs, int batch, float (&acc)[MT][R]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
-      if (s0 + u < s_end) {
-        const float* xl = xs + x_slot<F>(s0 + u, lane, 0);
+      const int s = s_begin + batch * U + u;
+      if (s < s_end) {
+        const float* xl = xs + x_slot<F>(s, lane, 0);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           float a[MT];
 #pragma unroll
           for (int m = 0; m < MT; ++m) a[m] = acc[m][r];
-          chunk_fma<F, MT>(c[u][r], xl, per_row, a);
+          chunk_fma<F, MT>(buf[u][r], xl, per_row, a);
 #pragma unroll
           for (int m = 0; m < MT; ++m) acc[m][r] = a[m];
         }
       }
     }
   }
-}
+
+  // Asks for the first two batches of a stream of n_groups groups (the second one only if there is one).
+  template <class RowsFn>
+  __device__ __forceinline__ void prefetch(RowsFn& rows_fn, int first_group, int stride, int n_groups) {
+    issue(buf_a, rows_fn, first_group, 0);
+    if (batches > 1) issue(buf_b, rows_fn, first_group, 1);
+    else if (n_groups > 1) issue(buf_b, rows_fn, first_group + stride, 0);
+  }
+
+  // Groups first_group, first_group + stride, ... (n_groups of them); prefetch() has asked for the first two
+  // batches.
+  template <class RowsFn, class DoneFn>
+  __device__ __forceinline__ void run(RowsFn& rows_fn, DoneFn& done_fn, int first_group, int stride, int n_groups) {
+    float acc[MT][R];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+    int group = first_group, batch = 0, left = n_groups;
+    bool first = true;  // the first half-iteration's next batch is already on its way
+    // One half-iteration: ask for the batch after (group, batch) into `next`, multiply `cur`.
+    auto half = [&](const Chunk<F>(&cur)[U][R], Chunk<F>(&next)[U][R]) {
+      const bool last_batch = batch + 1 == batches;
+      const int ng = last_batch ? group + stride : group, nb = last_batch ? 0 : batch + 1;
+      if (!(last_batch && left == 1) && !first) issue(next, rows_fn, ng, nb);
+      first = false;
+      const uint8_t* rows[R];
+      const uint8_t* scales[R];
+      const float* xs;
+      rows_fn(group, rows, scales, xs);
+      consume(cur, xs, batch, acc);
+      if (last_batch) {
+        done_fn(group, acc);
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+          for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+        --left;
+      }
+      group = ng;
+      batch = nb;
+    };
+    while (left > 0) {
+      half(buf_a, buf_b);
+      if (left == 0) break;
+      half(buf_b, buf_a);
+    }
+  }
+};
 
 }  // namespace dro
