@@ -1,11 +1,202 @@
-// Batched decode products on the matrix cores: lx_gemm_w, lx_gemm_skinny, and lx_gemv_w's entry (which
-// routes to the streaming GEMV, or to the skinny kernel in batch-invariant mode).
+// Batched decode products on the matrix cores: lx_gemm_skinny, lx_gemm_w (LX_MATH_BF16), and lx_gemv_w's entry
+// (contracts: engine/cuda/kernels.h:433-477; CPU behaviour of the BF16 math: engine/cpu/gemm.cpp:189-296).
+//
+//   y[m, n] = alpha * (rowfactor[n] * sum_k bf16(x[m, k]) * w[n, k] + bias[n]) + beta * y[m, n]
+//
+// One workgroup per tile of 16 weight rows; its S wavefronts split K (tile_mfma.h) and each asks for its whole
+// slice of the weights at once. Up to 64 activation rows ride along in one pass (more rows are further passes).
+// Neither S nor anything else that shapes a sum depends on M, so a row's bits are the same in any batch: the
+// reduction-order contract of the skinny GEMM, for every weight format.
+#include <stdlib.h>
+
 #include "common.h"
+#include "tile_mfma.h"
 
 namespace dro {
+
 int gemv_any(const void* x, int x_dtype, int ld_x, const lx_weight& w, const void* bias, int bias_dtype, void* y,
              int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream);
+
+namespace {
+
+struct GemmArgs {
+  XSource xs;
+  const uint8_t* w;
+  const uint8_t* scale;
+  float global;
+  const void* bias;
+  int bias_dtype;
+  void* y;
+  int y_dtype;
+  int64_t ld_y;
+  int M, N, K;
+  float alpha, beta;
+  int chunks, steps, steps_per_wave;
+  int64_t row_bytes, scale_row_bytes;
+};
+
+// The epilogue's operation order (engine/cpu/gemm.cpp:21-34).
+__device__ __forceinline__ void write_out(const GemmArgs& a, int wtype, int m, int n, float sum) {
+  float t = row_factor(wtype, a.scale, a.global, n) * sum;
+  if (a.bias) t += load_as_f32(a.bias, a.bias_dtype, n);
+  float v = a.alpha * t;
+  const int64_t at = m * a.ld_y + n;
+  if (a.beta != 0.0f) v = a.beta * load_as_f32(a.y, a.y_dtype, at) + v;
+  store_from_f32(a.y, a.y_dtype, at, v);
 }
+
+template <int F, int MT>
+__global__ void __launch_bounds__(kMaxSplit* kWave) skinny_kernel(const GemmArgs a) {
+  extern __shared__ __align__(16) f32x4 lds4[];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int n0 = blockIdx.x * kTileRows;
+  const int64_t n = min(n0 + (lane & 15), a.N - 1);  // past the end: read a valid row, write nothing
+  const uint8_t* rows[1] = {a.w + n * a.row_bytes};
+  const uint8_t* scales[1] = {a.scale + n * a.scale_row_bytes};
+  mfma_tile<F, 1, MT>(rows, scales, a.chunks, a.steps, a.steps_per_wave, a.xs, lds4, [&](int mt, int q, f32x4(&sums)[1]) {
+    const int m = mt * 16 + (q & 15), nq = n0 + 4 * (q >> 4);
+    if (m < a.M) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (nq + r < a.N) write_out(a, F, m, nq + r, sums[0][r]);
+    }
+  });
+}
+
+// Any shape and alignment: one wavefront per output column, lanes striding over k, activation rows eight at a
+// time. x is rounded to bf16 first when `round_x` (the BF16 math on f32 activations).
+__global__ void __launch_bounds__(256) gemm_plain_kernel(const GemmArgs a, int wtype, int round_x) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  if (n >= a.N) return;
+  for (int m0 = 0; m0 < a.M; m0 += 8) {
+    float acc[8];
+#pragma unroll
+    for (int m = 0; m < 8; ++m) acc[m] = 0.0f;
+    for (int k = lane; k < a.K; k += kWave) {
+      const float w = weight_element(wtype, a.w, a.scale, n, k, a.K);
+#pragma unroll
+      for (int m = 0; m < 8; ++m) {
+        if (m0 + m < a.M) {
+          float xv = load_as_f32(a.xs.x, a.xs.dtype, (m0 + m) * a.xs.ld + k);
+          if (round_x) xv = bf16_bits_to_f32(f32_to_bf16_bits(xv));
+          acc[m] = __builtin_fmaf(xv, w, acc[m]);
+        }
+      }
+    }
+#pragma unroll
+    for (int m = 0; m < 8; ++m) {
+      const float s = wave_sum(acc[m]);
+      if (lane == 0 && m0 + m < a.M) write_out(a, wtype, m0 + m, static_cast<int>(n), s);
+    }
+  }
+}
+
+template <int F, int MT>
+int launch_skinny(const GemmArgs& a, int S, hipStream_t stream) {
+  const size_t lds = S > 1 ? sizeof(f32x4) * S * MT * kWave : 0;
+  auto kernel = skinny_kernel<F, MT>;
+  if (lds > 48 * 1024) {
+    static thread_local bool raised = false;
+    if (!raised) {
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) !=
+          hipSuccess)
+        (void)hipGetLastError();
+      raised = true;
+    }
+  }
+  const unsigned grid = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(S * kWave), lds, stream, a);
+  return status_of(hipGetLastError());
+}
+
+template <int F>
+int launch_format(GemmArgs a, const char* x0, char* y0, int M, int x_esize, int y_esize, hipStream_t stream) {
+  const int64_t rb = row_bytes<F>(a.K);
+  const bool aligned = rb % 16 == 0 && reinterpret_cast<uintptr_t>(a.w) % 16 == 0 &&
+                       (F != LX_W_NVFP4 || reinterpret_cast<uintptr_t>(a.scale) % 2 == 0) &&
+                       reinterpret_cast<uintptr_t>(x0) % 16 == 0 && (a.xs.ld * x_esize) % 16 == 0 && a.K % 8 == 0;
+  if (!aligned) {
+    a.M = M;
+    hipLaunchKernelGGL(gemm_plain_kernel, dim3(static_cast<unsigned>((a.N + 3) / 4)), dim3(256), 0, stream, a, F,
+                       a.xs.dtype == LX_F32 ? 1 : 0);
+    return status_of(hipGetLastError());
+  }
+  a.row_bytes = rb;
+  a.scale_row_bytes = F == LX_W_NVFP4 ? a.K / 16 : 0;
+  a.chunks = static_cast<int>(rb / 16);
+  a.steps = load_steps_for<F>(a.K);
+  int S = split_for<F>(a.K, 1);
+  if (const char* e = getenv("DRO_SKINNY_SPLIT")) S = atoi(e);
+  a.steps_per_wave = (a.steps + S - 1) / S;
+  // Up to 64 activation rows a pass; every pass is the same arithmetic per row.
+  for (int m0 = 0; m0 < M; m0 += 64) {
+    a.M = M - m0 < 64 ? M - m0 : 64;
+    a.xs.M = a.M;
+    a.xs.x = x0 + static_cast<int64_t>(m0) * a.xs.ld * x_esize;
+    a.y = y0 + static_cast<int64_t>(m0) * a.ld_y * y_esize;
+    int st;
+    switch ((a.M + 15) / 16) {
+      case 1: st = launch_skinny<F, 1>(a, S, stream); break;
+      case 2: st = launch_skinny<F, 2>(a, S, stream); break;
+      case 3: st = launch_skinny<F, 3>(a, S, stream); break;
+      default: st = launch_skinny<F, 4>(a, S, stream); break;
+    }
+    if (st) return st;
+  }
+  return kOk;
+}
+
+bool valid_dtype(int d) { return d == LX_F32 || d == LX_BF16; }
+
+bool valid_weight(const lx_weight* w, int64_t K) {
+  if (!w || !w->data) return false;
+  switch (w->type) {
+    case LX_W_BF16: return true;
+    case LX_W_INT8:
+    case LX_W_FP8: return w->scale != nullptr;
+    case LX_W_NVFP4: return w->scale != nullptr && K % 16 == 0;
+    default: return false;
+  }
+}
+
+}  // namespace
+
+// The matrix-core product of any format: BF16 math (x rounded to bf16), any M. Validation follows
+// engine/cpu/gemm.cpp:189-197.
+int gemm_bf16_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w, const void* bias, int bias_dtype, void* y,
+                   int y_dtype, int64_t ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
+  if (M == 0 || N == 0) return kOk;
+  if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(kInvalid);
+  if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype) || (bias && !valid_dtype(bias_dtype))) return fail(kInvalid);
+  if (w.type == LX_W_BF16X) return fail(kNotSupported);
+  if (!x || !y || !valid_weight(&w, K)) return fail(kInvalid);
+  GemmArgs a{};
+  a.xs = XSource{x, x_dtype, ld_x, nullptr, 1, M, K};
+  a.w = static_cast<const uint8_t*>(w.data);
+  a.scale = static_cast<const uint8_t*>(w.scale);
+  a.global = w.type == LX_W_NVFP4 ? w.global : 1.0f;
+  a.bias = bias;
+  a.bias_dtype = bias_dtype;
+  a.y = y;
+  a.y_dtype = y_dtype;
+  a.ld_y = ld_y;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.alpha = alpha;
+  a.beta = beta;
+  const int xe = x_dtype == LX_BF16 ? 2 : 4, ye = y_dtype == LX_BF16 ? 2 : 4;
+  hipStream_t s = as_stream(stream);
+  switch (w.type) {
+    case LX_W_BF16: return launch_format<LX_W_BF16>(a, static_cast<const char*>(x), static_cast<char*>(y), M, xe, ye, s);
+    case LX_W_INT8: return launch_format<LX_W_INT8>(a, static_cast<const char*>(x), static_cast<char*>(y), M, xe, ye, s);
+    case LX_W_FP8: return launch_format<LX_W_FP8>(a, static_cast<const char*>(x), static_cast<char*>(y), M, xe, ye, s);
+    default: return launch_format<LX_W_NVFP4>(a, static_cast<const char*>(x), static_cast<char*>(y), M, xe, ye, s);
+  }
+}
+
+}  // namespace dro
 
 using namespace dro;
 
@@ -14,7 +205,20 @@ extern "C" {
 int lx_gemv_w(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, const void* bias, lx_dtype bias_dtype, void* y,
               lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
   if (!w) return fail(kInvalid);
+  // Batch-invariant mode: bf16 activations take the matrix-core kernel, whose sums are the same for every row
+  // count from 1 up (lx_gemm_w runs the same kernel). f32 activations keep the exact f32 product.
+  if (batch_invariant() && x_dtype == LX_BF16 && M >= 1 && M <= 8 && N > 0)
+    return gemm_bf16_math(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
   return gemv_any(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
+}
+
+int lx_gemm_w(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, lx_math math, const void* bias, lx_dtype bias_dtype,
+              void* y, lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* workspace, void* stream) {
+  (void)workspace;  // the BF16 math needs none
+  if (!w) return fail(kInvalid);
+  if (math != LX_MATH_BF16 && math != LX_MATH_INT8 && math != LX_MATH_FP8 && math != LX_MATH_FP4) return fail(kInvalid);
+  if (math != LX_MATH_BF16) return fail(kNotSupported);
+  return gemm_bf16_math(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
 }
 
 int64_t lx_gemm_workspace_bytes(int M, int K, lx_math math) {
@@ -24,18 +228,14 @@ int64_t lx_gemm_workspace_bytes(int M, int K, lx_math math) {
   return (bytes + 255) / 256 * 256;
 }
 
-}  // extern "C"
+int lx_gemm_skinny(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, const void* bias, lx_dtype bias_dtype, void* y,
+                   lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
+  if (!w) return fail(kInvalid);
+  if (x_dtype != LX_BF16 && M > 0 && N > 0) return fail(kNotSupported);  // bf16 activations only, as the reference
+  return gemm_bf16_math(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
+}
 
-// TEMPORARY until the matrix-core kernels land.
-extern "C" {
-int lx_gemm_w(const void*, lx_dtype, int, const lx_weight*, lx_math, const void*, lx_dtype, void*, lx_dtype, int, int, int, int,
-              float, float, void*, void*) {
-  return fail(kNotSupported);
-}
-int lx_gemm_skinny(const void*, lx_dtype, int, const lx_weight*, const void*, lx_dtype, void*, lx_dtype, int, int, int, int,
-                   float, float, void*) {
-  return fail(kNotSupported);
-}
+// TEMPORARY until the grouped experts land.
 int lx_moe_experts(const void*, const int32_t*, const float*, const void*, const void*, float*, int, int, int, int, void*) {
   return fail(kNotSupported);
 }
@@ -44,4 +244,5 @@ int lx_moe_experts_grouped(const void*, const int32_t*, const float*, const lx_w
   return fail(kNotSupported);
 }
 int64_t lx_moe_grouped_workspace_bytes(int, int, int, int, int, lx_math) { return 0; }
-}
+
+}  // extern "C"

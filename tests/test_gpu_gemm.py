@@ -1,0 +1,145 @@
+"""GPU parity: the matrix-core products lx_gemm_w (BF16 math) and lx_gemm_skinny through the C ABI, against
+float64 on the decoded values with bf16-rounded activations, against the CPU oracle at the BASELINE shapes, and the
+bitwise invariants: a row's bits do not depend on the batch, and in batch-invariant mode lx_gemv_w and lx_gemm_w
+give the same bits for every row count from 1 up."""
+
+import os
+
+import pytest
+import torch
+
+import checks
+import ops
+from conftest import rel_l2
+from dromos_amd.abi import FORMATS, MATH_BF16, MATH_FP4, MATH_FP8, MATH_INT8
+from dromos_amd.formats import master_weight, quantize_with, random_weight
+
+pytestmark = pytest.mark.gpu
+FMT = checks.FMT_NAMES
+
+
+def gemm_case(hip, fmt, M, N, K, seed, x_dtype=torch.bfloat16, bias_dtype=None, y_dtype=torch.float32, alpha=1.0, beta=0.0,
+              entry="gemm_w"):
+    g = torch.Generator().manual_seed(seed)
+    w = random_weight(FORMATS[fmt], N, K, seed + 1)
+    x = torch.randn(M, K, generator=g).to(x_dtype)
+    bias = None if bias_dtype is None else torch.randn(N, generator=g).to(bias_dtype)
+    y0 = torch.randn(M, N, generator=g).to(y_dtype)
+    y = y0.clone() if beta != 0.0 else torch.full((M, N), float("nan"), dtype=y_dtype)
+    call = ops.gemm_w if entry == "gemm_w" else ops.gemm_skinny
+    kw = dict(bias=None if bias is None else bias.cuda(), y=y.cuda(), alpha=alpha, beta=beta)
+    got = call(hip, x.cuda(), w.to("cuda"), **kw) if entry != "gemm_w" else call(hip, x.cuda(), w.to("cuda"), MATH_BF16, **kw)
+    want = ops.gemv_reference(x.to(torch.bfloat16), w.dense(), bias, alpha, beta, y0)
+    checks.check_product(got.cpu(), want)
+    return got
+
+
+@pytest.mark.parametrize("M", [1, 5, 9, 16, 17, 33, 64, 70, 130])
+@pytest.mark.parametrize("fmt", FMT)
+def test_gemm_w_every_m(hip, fmt, M):
+    gemm_case(hip, fmt, M, 300, 1024, seed=M, bias_dtype=torch.float32)
+
+
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (0.5, 0.0), (-1.5, 1.0)])
+@pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("bias_dtype", [None, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("fmt", FMT)
+def test_gemm_w_dtype_matrix(hip, fmt, x_dtype, bias_dtype, y_dtype, alpha, beta):
+    gemm_case(hip, fmt, 20, 37, 544, seed=11, x_dtype=x_dtype, bias_dtype=bias_dtype, y_dtype=y_dtype, alpha=alpha, beta=beta)
+
+
+@pytest.mark.parametrize("K", [16, 32, 48, 64, 128, 256, 272, 512, 544, 1024, 1040, 2064, 4096, 14336])
+@pytest.mark.parametrize("fmt", FMT)
+def test_gemm_w_k_boundaries(hip, fmt, K):
+    # K around the load-step sizes (32 / 64 / 128 k per step), rows that end inside a step, and K = 48, whose
+    # rows cannot be read 16 bytes at a time in every format (the plain kernel).
+    gemm_case(hip, fmt, 12, 21, K, seed=K)
+
+
+@pytest.mark.parametrize("N,K", [(10304, 2048), (2048, 4096), (256, 6400), (8, 2048), (1, 512)])
+@pytest.mark.parametrize("fmt", FMT)
+def test_gemm_w_decode_shapes(hip, fmt, N, K):
+    gemm_case(hip, fmt, 32, N, K, seed=N % 89)
+
+
+def test_gemm_w_strided_and_untouched_padding(hip):
+    for fmt in FMT:
+        M, N, K, pad = 19, 300, 1024, 8
+        g = torch.Generator().manual_seed(5)
+        w = random_weight(FORMATS[fmt], N, K, 6)
+        xb = torch.randn(M, K + pad, generator=g).to(torch.bfloat16)
+        y0 = torch.randn(M, N + pad, generator=g)
+        y = y0.clone().cuda()
+        ops.gemm_w(hip, xb.cuda(), w.to("cuda"), MATH_BF16, y=y, alpha=2.0, beta=0.5, ld_x=K + pad, ld_y=N + pad, N=N)
+        want = ops.gemv_reference(xb[:, :K], w.dense(), None, 2.0, 0.5, y0[:, :N])
+        checks.check_product(y.cpu()[:, :N], want)
+        assert torch.equal(y.cpu()[:, N:], y0[:, N:]), "wrote past the N columns of y"
+
+
+def test_other_maths_and_arguments(hip):
+    w = random_weight(FORMATS["int8"], 32, 64, 1).to("cuda")
+    x = torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda")
+    for math in (MATH_INT8, MATH_FP8, MATH_FP4):
+        assert ops.gemm_w(hip, x, w, math, status=True) == 801
+    assert ops.gemm_w(hip, x, w, 7, status=True) == 1
+    assert ops.gemm_w(hip, x[:0], w, MATH_BF16, status=True) == 0
+    assert ops.gemm_skinny(hip, x.float(), w, status=True) == 801  # bf16 activations only
+    assert ops.gemm_skinny(hip, x, w, status=True) == 0
+
+
+@pytest.mark.parametrize("fmt", FMT)
+@pytest.mark.parametrize("N,K", [(1024, 2048), (300, 4096), (2048, 1024)])
+def test_skinny_rows_do_not_depend_on_the_batch(hip, fmt, N, K):
+    # engine/cuda/kernels.h:466-471: M = 1, 2, 8, 16, 32, 64 and across chunks of 64.
+    w = random_weight(FORMATS[fmt], N, K, N + K).to("cuda")
+    g = torch.Generator().manual_seed(N)
+    x = torch.randn(100, K, generator=g).to(torch.bfloat16).cuda()
+    bias = torch.randn(N, generator=g).cuda()
+    full = ops.gemm_skinny(hip, x, w, bias=bias)
+    for M in (1, 2, 8, 16, 32, 64):
+        part = ops.gemm_skinny(hip, x[:M].contiguous(), w, bias=bias)
+        assert torch.equal(part, full[:M]), f"rows of an M={M} call differ from the same rows of an M=100 call"
+    for m in (0, 17, 63, 64, 99):
+        alone = ops.gemm_skinny(hip, x[m : m + 1].contiguous(), w, bias=bias)
+        assert torch.equal(alone[0], full[m]), f"row {m} alone differs from the row in the batch"
+    assert torch.equal(ops.gemm_skinny(hip, x, w, bias=bias), full)  # and from run to run
+    assert torch.equal(ops.gemm_w(hip, x, w, MATH_BF16, bias=bias), full)  # lx_gemm_w is the same kernel
+
+
+@pytest.mark.parametrize("fmt", FMT)
+def test_batch_invariant_mode_spans_gemv_and_gemm(hip, fmt):
+    # With LX_BATCH_INVARIANT set, lx_gemv_w (M <= 8, bf16 x) and lx_gemm_w give a row the same bits whatever the
+    # row count, 1 included; without it lx_gemv_w takes the streaming kernel (its own, also batch-independent, sums).
+    N, K = 512, 4096
+    w = random_weight(FORMATS[fmt], N, K, 3).to("cuda")
+    x = torch.randn(64, K, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16).cuda()
+    os.environ["LX_BATCH_INVARIANT"] = "1"
+    try:
+        ref64 = ops.gemm_w(hip, x, w, MATH_BF16)
+        for M in (1, 4, 8):
+            y = ops.gemv_w(hip, x[:M].contiguous(), w)
+            assert torch.equal(y, ref64[:M]), f"M={M}"
+        assert torch.equal(ops.gemm_w(hip, x[:16].contiguous(), w, MATH_BF16), ref64[:16])
+    finally:
+        del os.environ["LX_BATCH_INVARIANT"]
+    os.environ["LX_BATCH_INVARIANT"] = "0"  # starts with '0': off
+    try:
+        y1 = ops.gemv_w(hip, x[:1].contiguous(), w)
+    finally:
+        del os.environ["LX_BATCH_INVARIANT"]
+    assert torch.equal(y1, ops.gemv_w(hip, x[:1].contiguous(), w))
+    assert rel_l2(y1, ref64[:1]) < 1e-5
+
+
+@pytest.mark.parametrize("fmt,M", [("int8", 16), ("int8", 64), ("fp8", 16), ("fp8", 64)])
+def test_baseline_config_against_the_oracle(hip, oracle, fmt, M):
+    N, K = 14336, 4096
+    g = torch.Generator().manual_seed(1000 + M)
+    master = master_weight(N, K, g)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = quantize_with(hip, master.cuda(), FORMATS[fmt])
+    y = ops.gemm_w(hip, x.cuda(), w, MATH_BF16)
+    want = ops.gemm_w(oracle, x, w.to("cpu"), MATH_BF16)
+    err = rel_l2(y.cpu(), want)
+    assert err <= 1e-2 and err <= 1e-4, err
