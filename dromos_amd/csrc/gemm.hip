@@ -19,8 +19,14 @@ int gemv_any(const void* x, int x_dtype, int ld_x, const lx_weight& w, const voi
 
 namespace {
 
+struct XRows {
+  const void* x;
+  int dtype;
+  int64_t ld;  // elements between rows
+};
+
 struct GemmArgs {
-  XSource xs;
+  XRows xs;
   const uint8_t* w;
   const uint8_t* scale;
   float global;
@@ -45,7 +51,7 @@ __device__ __forceinline__ void write_out(const GemmArgs& a, int wtype, int m, i
   store_from_f32(a.y, a.y_dtype, at, v);
 }
 
-template <int F, int MT>
+template <int F, int MT, bool XF32>
 __global__ void __launch_bounds__(kMaxSplit* kWave) skinny_kernel(const GemmArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
   const int lane = threadIdx.x & (kWave - 1);
@@ -53,7 +59,13 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) skinny_kernel(const GemmArgs
   const int64_t n = min(n0 + (lane & 15), a.N - 1);  // past the end: read a valid row, write nothing
   const uint8_t* rows[1] = {a.w + n * a.row_bytes};
   const uint8_t* scales[1] = {a.scale + n * a.scale_row_bytes};
-  mfma_tile<F, 1, MT>(rows, scales, a.chunks, a.steps, a.steps_per_wave, a.xs, lds4, [&](int mt, int q, f32x4(&sums)[1]) {
+  const void* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int64_t m = min(mt * 16 + (lane & 15), a.M - 1);
+    xrow[mt] = static_cast<const char*>(a.xs.x) + m * a.xs.ld * (XF32 ? 4 : 2);
+  }
+  mfma_tile<F, 1, MT, XF32>(rows, scales, a.chunks, a.steps, a.steps_per_wave, xrow, a.K, lds4, [&](int mt, int q, f32x4(&sums)[1]) {
     const int m = mt * 16 + (q & 15), nq = n0 + 4 * (q >> 4);
     if (m < a.M) {
 #pragma unroll
@@ -92,10 +104,10 @@ __global__ void __launch_bounds__(256) gemm_plain_kernel(const GemmArgs a, int w
   }
 }
 
-template <int F, int MT>
-int launch_skinny(const GemmArgs& a, int S, hipStream_t stream) {
+template <int F, int MT, bool XF32>
+int launch_skinny_x(const GemmArgs& a, int S, hipStream_t stream) {
   const size_t lds = S > 1 ? sizeof(f32x4) * S * MT * kWave : 0;
-  auto kernel = skinny_kernel<F, MT>;
+  auto kernel = skinny_kernel<F, MT, XF32>;
   if (lds > 48 * 1024) {
     static thread_local bool raised = false;
     if (!raised) {
@@ -108,6 +120,11 @@ int launch_skinny(const GemmArgs& a, int S, hipStream_t stream) {
   const unsigned grid = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(S * kWave), lds, stream, a);
   return status_of(hipGetLastError());
+}
+
+template <int F, int MT>
+int launch_skinny(const GemmArgs& a, int S, hipStream_t stream) {
+  return a.xs.dtype == LX_F32 ? launch_skinny_x<F, MT, true>(a, S, stream) : launch_skinny_x<F, MT, false>(a, S, stream);
 }
 
 template <int F>
@@ -132,7 +149,6 @@ int launch_format(GemmArgs a, const char* x0, char* y0, int M, int x_esize, int 
   // Up to 64 activation rows a pass; every pass is the same arithmetic per row.
   for (int m0 = 0; m0 < M; m0 += 64) {
     a.M = M - m0 < 64 ? M - m0 : 64;
-    a.xs.M = a.M;
     a.xs.x = x0 + static_cast<int64_t>(m0) * a.xs.ld * x_esize;
     a.y = y0 + static_cast<int64_t>(m0) * a.ld_y * y_esize;
     int st;
@@ -172,7 +188,7 @@ int gemm_bf16_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w,
   if (w.type == LX_W_BF16X) return fail(kNotSupported);
   if (!x || !y || !valid_weight(&w, K)) return fail(kInvalid);
   GemmArgs a{};
-  a.xs = XSource{x, x_dtype, ld_x, nullptr, 1, M, K};
+  a.xs = XRows{x, x_dtype, ld_x};
   a.w = static_cast<const uint8_t*>(w.data);
   a.scale = static_cast<const uint8_t*>(w.scale);
   a.global = w.type == LX_W_NVFP4 ? w.global : 1.0f;

@@ -90,45 +90,71 @@ __device__ __forceinline__ bf16x8 weight_fragment<LX_W_NVFP4>(const u32x4& w, ui
   return __builtin_bit_cast(bf16x8, p);
 }
 
-// Where a wavefront's activation fragments come from: rows of bf16 or f32 in global memory (16-byte aligned
-// rows), optionally gathered through a row table. fragment(m, k) = x[m, k .. k + 8) as bf16, zero past M or K.
-struct XSource {
-  const void* x;
-  int dtype;
-  int64_t ld;       // elements between rows
-  const int* rows;  // activation m reads row rows[m] / rows_div, or row m when null
-  int rows_div;
-  int M, K;
-
-  __device__ __forceinline__ bf16x8 fragment(int m, int k) const {
-    bf16x8 zero = __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
-    if (m >= M || k >= K) return zero;
-    const int64_t row = rows ? rows[m] / rows_div : m;
-    if (dtype == LX_BF16) {
-      const u32x4 v = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(x) + row * ld + k);
-      return __builtin_bit_cast(bf16x8, v);
-    }
-    const f32x4* p = reinterpret_cast<const f32x4*>(static_cast<const float*>(x) + row * ld + k);
-    const f32x4 a = p[0], b = p[1];
-    bf16x2 q[4] = {pack_bf16(a.x, a.y), pack_bf16(a.z, a.w), pack_bf16(b.x, b.y), pack_bf16(b.z, b.w)};
-    return __builtin_bit_cast(bf16x8, q);
-  }
+// Where a wavefront's activation fragments come from: rows of bf16 or f32 in global memory whose addresses and
+// strides are multiples of 16 bytes. XF32 says which; the caller resolves each lane's row pointers (one per
+// activation tile, clamped into the matrix: the columns of a clamped row are computed and never written).
+template <bool XF32>
+struct XFrag {
+  u32x4 raw[XF32 ? 2 : 1];
 };
+
+// x[row, k .. k + 8) as loaded; k is clamped into the row (a fragment past K is zeroed when it is used).
+template <bool XF32>
+__device__ __forceinline__ void load_x_fragment(XFrag<XF32>& f, const void* row, int k, int K) {
+  const int kc = min(k, K - 8);
+  if constexpr (XF32) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(static_cast<const float*>(row) + kc);
+    f.raw[0] = p[0];
+    f.raw[1] = p[1];
+  } else {
+    f.raw[0] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(row) + kc);
+  }
+}
+
+// The fragment as the B operand: bf16 as it is, f32 rounded to bf16 (nearest even); zero past K.
+template <bool XF32>
+__device__ __forceinline__ bf16x8 x_operand(const XFrag<XF32>& f, int k, int K) {
+  u32x4 v;
+  if constexpr (XF32) {
+    bf16x2 q[4] = {pack_bf16(__uint_as_float(f.raw[0].x), __uint_as_float(f.raw[0].y)),
+                   pack_bf16(__uint_as_float(f.raw[0].z), __uint_as_float(f.raw[0].w)),
+                   pack_bf16(__uint_as_float(f.raw[1].x), __uint_as_float(f.raw[1].y)),
+                   pack_bf16(__uint_as_float(f.raw[1].z), __uint_as_float(f.raw[1].w))};
+    v = __builtin_bit_cast(u32x4, q);
+  } else {
+    v = f.raw[0];
+  }
+  if (k >= K) v = u32x4{0u, 0u, 0u, 0u};
+  return __builtin_bit_cast(bf16x8, v);
+}
+
+// Load steps asked for at once: bounded by the registers the activation fragments of a batch take
+// (steps x instructions per step x activation tiles x 4 or 8 registers), at most kLoadsInFlight / NT.
+template <int F, int NT, int MT, bool XF32>
+constexpr int batch_steps() {
+  constexpr int J = Fmt<F>::kElems / 8;
+  int u = 16 / (J * MT * (XF32 ? 2 : 1));
+  const int cap = kLoadsInFlight / NT;
+  u = u > cap ? cap : u;
+  return u < 1 ? 1 : u;
+}
 
 // acc[t][mt] += tile t's rows times activation tile mt over load steps [t_begin, t_end).
 // rows[t] / scales[t] point at this lane's weight row of tile t (row i = lane % 16 of the tile, clamped into the
-// matrix by the caller). `chunks` is the number of 16-byte chunks in a row.
-template <int F, int NT, int MT>
+// matrix by the caller); xrow[mt] at this lane's activation row of tile mt. `chunks` is the number of 16-byte
+// chunks in a weight row. Every load of a batch, weights and activations, is asked for before the first use.
+template <int F, int NT, int MT, bool XF32>
 __device__ __forceinline__ void mfma_slice(const uint8_t* const (&rows)[NT], const uint8_t* const (&scales)[NT], int chunks,
-                                           int t_begin, int t_end, const XSource& xs, f32x4 (&acc)[NT][MT]) {
+                                           int t_begin, int t_end, const void* const (&xrow)[MT], int K, f32x4 (&acc)[NT][MT]) {
   constexpr int E = Fmt<F>::kElems;
   constexpr int J = E / 8;  // matrix instructions per load step
-  constexpr int U = kLoadsInFlight / NT;
+  constexpr int U = batch_steps<F, NT, MT, XF32>();
   const int lane = threadIdx.x & (kWave - 1);
-  const int g = lane >> 4, i = lane & 15;
+  const int g = lane >> 4;
   for (int tb = t_begin; tb < t_end; tb += U) {
     u32x4 wv[U][NT];
     uint32_t sc[U][NT];
+    XFrag<XF32> xf[U][J][MT];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       // A step past the slice, or a chunk past the row's end, re-reads a valid chunk of the same row; its
@@ -144,18 +170,24 @@ __device__ __forceinline__ void mfma_slice(const uint8_t* const (&rows)[NT], con
     }
 #pragma unroll
     for (int u = 0; u < U; ++u) {
+      const int k0 = (4 * min(tb + u, t_end - 1) + g) * E;
+#pragma unroll
+      for (int j = 0; j < J; ++j)
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) load_x_fragment<XF32>(xf[u][j][mt], xrow[mt], k0 + 8 * j, K);
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
       if (tb + u < t_end) {
         const int k0 = (4 * (tb + u) + g) * E;
 #pragma unroll
         for (int j = 0; j < J; ++j) {
-          bf16x8 xf[MT];
-#pragma unroll
-          for (int mt = 0; mt < MT; ++mt) xf[mt] = xs.fragment(mt * 16 + i, k0 + 8 * j);
 #pragma unroll
           for (int n = 0; n < NT; ++n) {
             const bf16x8 wf = weight_fragment<F>(wv[u][n], sc[u][n], j);
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) acc[n][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, xf[mt], acc[n][mt], 0, 0, 0);
+            for (int mt = 0; mt < MT; ++mt)
+              acc[n][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, x_operand<XF32>(xf[u][j][mt], k0 + 8 * j, K), acc[n][mt], 0, 0, 0);
           }
         }
       }
@@ -167,9 +199,10 @@ __device__ __forceinline__ void mfma_slice(const uint8_t* const (&rows)[NT], con
 // in ascending w through `lds` (S * NT * MT * 64 f32x4), and epi(mt, q, sums) is called once for every
 // (activation tile mt, lane slot q) with the NT finished sums: sums[t][r] belongs to weight row 4 * (q / 16) + r
 // of tile t and activation row mt * 16 + q % 16.
-template <int F, int NT, int MT, class Epi>
+template <int F, int NT, int MT, bool XF32, class Epi>
 __device__ __forceinline__ void mfma_tile(const uint8_t* const (&rows)[NT], const uint8_t* const (&scales)[NT], int chunks,
-                                          int steps, int steps_per_wave, const XSource& xs, f32x4* lds, Epi&& epi) {
+                                          int steps, int steps_per_wave, const void* const (&xrow)[MT], int K, f32x4* lds,
+                                          Epi&& epi) {
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int S = blockDim.x / kWave;
   f32x4 acc[NT][MT];
@@ -178,7 +211,7 @@ __device__ __forceinline__ void mfma_tile(const uint8_t* const (&rows)[NT], cons
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[n][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int t_begin = min(steps, wave * steps_per_wave), t_end = min(steps, t_begin + steps_per_wave);
-  mfma_slice<F, NT, MT>(rows, scales, chunks, t_begin, t_end, xs, acc);
+  mfma_slice<F, NT, MT, XF32>(rows, scales, chunks, t_begin, t_end, xrow, K, acc);
   if (S == 1) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
