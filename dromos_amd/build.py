@@ -14,7 +14,7 @@ ROOT = Path(__file__).resolve().parent.parent
 CSRC = ROOT / "dromos_amd" / "csrc"
 LIB_DIR = ROOT / "dromos_amd" / "lib"
 HIP_LIB = LIB_DIR / "libdromos_hip.so"
-SOURCES = ["runtime.hip", "quant.hip", "gemv.hip", "gemm.hip", "moe.hip"]
+SOURCES = ["runtime.hip", "quant.hip", "gemv.hip", "gemm.hip", "moe.hip", "moe_grouped.hip"]
 
 # -ffp-contract=off: the epilogues and the ordered sums are written as separate multiplies and adds, as the
 # CPU reference computes them; fused operations are spelled __builtin_fmaf where they are meant.

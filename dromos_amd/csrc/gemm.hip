@@ -251,14 +251,4 @@ int lx_gemm_skinny(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w
   return gemm_bf16_math(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
 }
 
-// TEMPORARY until the grouped experts land.
-int lx_moe_experts(const void*, const int32_t*, const float*, const void*, const void*, float*, int, int, int, int, void*) {
-  return fail(kNotSupported);
-}
-int lx_moe_experts_grouped(const void*, const int32_t*, const float*, const lx_weight*, const lx_weight*, lx_math, float*, void*,
-                           int, int, int, int, int, void*) {
-  return fail(kNotSupported);
-}
-int64_t lx_moe_grouped_workspace_bytes(int, int, int, int, int, lx_math) { return 0; }
-
 }  // extern "C"

@@ -9,6 +9,7 @@
 //             the expert's down rows against inter[pair] and adds w_k * c_k in slot order, so each output
 //             is written once and its bits depend on nothing but the token.
 #include "common.h"
+#include "moe_common.h"
 #include "stream_dot.h"
 
 namespace dro {
@@ -85,29 +86,6 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
 }
 
 // ---- decode experts ----------------------------------------------------------------------------------------
-
-struct Stack {
-  const uint8_t* data;
-  const uint8_t* scale;
-  const float* expert_global;
-  float global;
-};
-
-struct DecodeArgs {
-  const uint16_t* latent;  // bf16 [T, L]
-  const int32_t* ids;      // [T, top_k]
-  const float* weights;    // [T, top_k]
-  Stack gu, dn;
-  uint16_t* inter;  // bf16 [T * top_k, I]
-  float* out;       // f32 [T, L]
-  int T, L, I, top_k;
-};
-
-__device__ __forceinline__ float stack_factor(int type, const Stack& s, int e, int64_t row_in_stack) {
-  if (type == LX_W_INT8 || type == LX_W_FP8) return reinterpret_cast<const float*>(s.scale)[row_in_stack];
-  if (type == LX_W_NVFP4) return s.expert_global ? s.expert_global[e] : s.global;
-  return 1.0f;
-}
 
 // Sorts the P pairs by expert (stable) in LDS. order[g] = pair at sorted position g; returns through
 // group_begin / group_end the positions of group `slot` (the slot-th distinct expert in ascending id order),
@@ -346,12 +324,6 @@ void allow_big_lds(Kernel kernel, size_t lds) {
 template <int F>
 int launch_gate_up(const DecodeArgs& a, hipStream_t s) {
   const int P = a.T * a.top_k;
-  if (!streamable<F>(a.gu, a.L, 8)) {
-    const int64_t items = static_cast<int64_t>(P) * a.I;
-    hipLaunchKernelGGL(decode_gate_up_plain_kernel, dim3(static_cast<unsigned>((items + kWaves - 1) / kWaves)),
-                       dim3(kThreads), 0, s, a, F);
-    return status_of(hipGetLastError());
-  }
   constexpr int U = moe_loads_in_flight<F>();
   // With distinct experts per token a group has at most T pairs; the LDS image holds that many rows.
   const int mt_cap = a.T <= 1 ? 1 : a.T <= 2 ? 2 : a.T <= 4 ? 4 : 8;
@@ -369,12 +341,6 @@ int launch_gate_up(const DecodeArgs& a, hipStream_t s) {
 
 template <int F>
 int launch_down(const DecodeArgs& a, hipStream_t s) {
-  if (!streamable<F>(a.dn, a.I, 8)) {
-    const int64_t items = static_cast<int64_t>(a.T) * a.L;
-    hipLaunchKernelGGL(decode_down_plain_kernel, dim3(static_cast<unsigned>((items + kWaves - 1) / kWaves)), dim3(kThreads),
-                       0, s, a, F);
-    return status_of(hipGetLastError());
-  }
   constexpr int U = moe_loads_in_flight<F>();
   const size_t lds = sizeof(float) * 8 * x_row_floats<F>(steps_for<F>(a.I));
   const int groups = (a.L + 1) / 2;
@@ -388,22 +354,21 @@ int launch_down(const DecodeArgs& a, hipStream_t s) {
   return status_of(hipGetLastError());
 }
 
-bool valid_stack(const lx_weight& w, int64_t K) {
-  if (!w.data) return false;
-  switch (w.type) {
-    case LX_W_BF16: return true;
-    case LX_W_INT8:
-    case LX_W_FP8: return w.scale != nullptr;
-    case LX_W_NVFP4: return w.scale != nullptr && K % 16 == 0;
-    default: return false;
-  }
-}
-
-Stack as_stack(const lx_weight& w) {
-  return Stack{static_cast<const uint8_t*>(w.data), static_cast<const uint8_t*>(w.scale), w.expert_global, w.global};
-}
-
 int64_t round256(int64_t b) { return (b + 255) / 256 * 256; }
+
+int gate_up_plain(const DecodeArgs& a, int type, hipStream_t s) {
+  const int64_t items = static_cast<int64_t>(a.T) * a.top_k * a.I;
+  hipLaunchKernelGGL(decode_gate_up_plain_kernel, dim3(static_cast<unsigned>((items + kWaves - 1) / kWaves)), dim3(kThreads), 0,
+                     s, a, type);
+  return status_of(hipGetLastError());
+}
+
+int down_plain(const DecodeArgs& a, int type, hipStream_t s) {
+  const int64_t items = static_cast<int64_t>(a.T) * a.L;
+  hipLaunchKernelGGL(decode_down_plain_kernel, dim3(static_cast<unsigned>((items + kWaves - 1) / kWaves)), dim3(kThreads), 0, s,
+                     a, type);
+  return status_of(hipGetLastError());
+}
 
 }  // namespace
 
@@ -422,20 +387,38 @@ int experts_decode(const void* latent, const int32_t* ids, const float* weights,
   a.L = L;
   a.I = I;
   a.top_k = top_k;
+  auto can_stream = [](int type, const Stack& st, int64_t K) {
+    switch (type) {
+      case LX_W_BF16: return streamable<LX_W_BF16>(st, K, 8);
+      case LX_W_INT8: return streamable<LX_W_INT8>(st, K, 8);
+      case LX_W_FP8: return streamable<LX_W_FP8>(st, K, 8);
+      default: return streamable<LX_W_NVFP4>(st, K, 8);
+    }
+  };
   int st;
-  switch (gate_up.type) {
-    case LX_W_BF16: st = launch_gate_up<LX_W_BF16>(a, s); break;
-    case LX_W_INT8: st = launch_gate_up<LX_W_INT8>(a, s); break;
-    case LX_W_FP8: st = launch_gate_up<LX_W_FP8>(a, s); break;
-    default: st = launch_gate_up<LX_W_NVFP4>(a, s); break;
+  if (!can_stream(gate_up.type, a.gu, L)) {
+    st = gate_up_plain(a, gate_up.type, s);
+  } else {
+    switch (gate_up.type) {
+      case LX_W_BF16: st = launch_gate_up<LX_W_BF16>(a, s); break;
+      case LX_W_INT8: st = launch_gate_up<LX_W_INT8>(a, s); break;
+      case LX_W_FP8: st = launch_gate_up<LX_W_FP8>(a, s); break;
+      default: st = launch_gate_up<LX_W_NVFP4>(a, s); break;
+    }
   }
   if (st) return st;
+  if (!can_stream(down.type, a.dn, I)) return down_plain(a, down.type, s);
   switch (down.type) {
     case LX_W_BF16: return launch_down<LX_W_BF16>(a, s);
     case LX_W_INT8: return launch_down<LX_W_INT8>(a, s);
     case LX_W_FP8: return launch_down<LX_W_FP8>(a, s);
     default: return launch_down<LX_W_NVFP4>(a, s);
   }
+}
+
+int experts_plain(const DecodeArgs& a, int gu_type, int dn_type, hipStream_t s) {
+  if (int st = gate_up_plain(a, gu_type, s)) return st;
+  return down_plain(a, dn_type, s);
 }
 
 }  // namespace dro
