@@ -77,14 +77,14 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs
   // Part p of S takes the contiguous steps [p * per, (p + 1) * per).
   const int s_begin = min(steps, part * a.steps_per_part), s_end = min(steps, s_begin + a.steps_per_part);
 
-  auto rows_fn = [&](int g, const uint8_t* (&rows)[R], const uint8_t* (&scales)[R], const float*& x_image) {
+  auto rows_fn = [&](int g, const uint8_t* (&rows)[R], const uint8_t* (&scales)[R], const float* (&x_image)[R]) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int64_t n = min(g * R + r, a.N - 1);  // past the end: stream a valid row, write nothing
       rows[r] = a.w + n * rb;
       scales[r] = a.scale + n * a.scale_row_bytes;
+      x_image[r] = xs;
     }
-    x_image = xs;
   };
   auto done_fn = [&](int g, float (&acc)[MT][R]) {
 #pragma unroll
@@ -172,19 +172,15 @@ int order_class(int N, int64_t K, int R) {
 // How a launch is shaped. None of it changes an output's bits (only S does).
 struct Shape {
   int threads;  // workgroup size
-  int ru;       // which (R, U) instance
+  int depth;    // U: steps asked for at once; a wavefront holds R = 8 / U rows (4 at most)
 };
 
-Shape shape_for(int wtype, int M) {
-  // Measured on MI355X at the decode shapes: a wavefront should own about 8 KB of weights, all requested at once.
-  Shape s{256, 1};
-  if (M == 1) {
-    if (wtype == LX_W_BF16) s = Shape{256, 2};        // one row, eight steps in flight
-    else if (wtype == LX_W_NVFP4) s = Shape{512, 2};  // long rows of few bytes: more wavefronts per x image
-    else s = Shape{256, 1};                           // two rows, four steps each
-  }
+// Measured on MI355X at the decode shapes: a wavefront should own about 8 KB of weights, all requested at once,
+// so rows of few steps are taken several at a time.
+Shape shape_for(int wtype, int steps) {
+  Shape s{wtype == LX_W_NVFP4 ? 512 : 256, batch_depth(steps, 8)};
   if (const char* e = getenv("DRO_GEMV_THREADS")) s.threads = atoi(e);
-  if (const char* e = getenv("DRO_GEMV_RU")) s.ru = atoi(e);
+  if (const char* e = getenv("DRO_GEMV_DEPTH")) s.depth = atoi(e);
   return s;
 }
 
@@ -211,17 +207,11 @@ int launch_stream(GemvArgs a, const Shape& shape, hipStream_t stream) {
 
 template <int F, int MT>
 int launch_rows(const GemvArgs& a, const Shape& shape, hipStream_t stream) {
-  if constexpr (MT == 1) {
-    switch (shape.ru) {
-      case 0: return launch_stream<F, 1, 1, 4>(a, shape, stream);
-      case 2: return launch_stream<F, 1, 1, 8>(a, shape, stream);
-      case 3: return launch_stream<F, 1, 2, 2>(a, shape, stream);
-      case 4: return launch_stream<F, 1, 4, 2>(a, shape, stream);
-      case 5: return launch_stream<F, 1, 2, 8>(a, shape, stream);
-      default: return launch_stream<F, 1, 2, 4>(a, shape, stream);
-    }
-  } else {
-    return launch_stream<F, MT, 2, (F == LX_W_NVFP4 ? 2 : 4)>(a, shape, stream);
+  switch (shape.depth) {
+    case 8: return launch_stream<F, MT, 1, 8>(a, shape, stream);
+    case 4: return launch_stream<F, MT, 2, 4>(a, shape, stream);
+    case 2: return launch_stream<F, MT, 4, 2>(a, shape, stream);
+    default: return launch_stream<F, MT, 4, 1>(a, shape, stream);
   }
 }
 
@@ -260,7 +250,7 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
     a.x = x0 + m0 * x_row;
     a.y = y0 + m0 * y_row;
     const int mt = a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : 8;
-    const Shape shape = shape_for(F, a.M);
+    const Shape shape = shape_for(F, steps);
     int st;
     switch (mt) {
       case 1: st = launch_rows<F, 1>(a, shape, stream); break;

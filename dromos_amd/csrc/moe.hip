@@ -21,42 +21,60 @@ constexpr int kMaxPairs = 64;
 
 // ---- routing ---------------------------------------------------------------------------------------------
 
-// One wavefront per token. E <= 4096 (a lane keeps one taken-bit per element it owns).
+// One wavefront per token; a lane keeps its NPL logits (elements lane, lane + 64, ...) in registers, so the row
+// is read once. E <= 64 * NPL.
+template <int NPL>
 __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
                                                          int32_t* __restrict__ ids, float* __restrict__ weights,
                                                          float* __restrict__ entropy, float* __restrict__ confidence, int T,
                                                          int E, int top_k) {
-  __shared__ float picked_logit[kWaves][64];
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int64_t t = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
   if (t >= T) return;
   const float* row = logits + t * E;
+  float v[NPL], biased[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; ++j) {
+    const int i = lane + j * kWave;
+    v[j] = i < E ? row[i] : -INFINITY;
+    // One f32 add, as the reference selects (a NaN or a missing element is never greater).
+    biased[j] = i < E ? v[j] + (bias ? bias[i] : 0.0f) : -INFINITY;
+  }
   float m = -INFINITY;
-  for (int i = lane; i < E; i += kWave) m = fmaxf(m, row[i]);
+#pragma unroll
+  for (int j = 0; j < NPL; ++j) m = fmaxf(m, v[j]);
   m = wave_max(m);
-  float z = 0.0f;
-  for (int i = lane; i < E; i += kWave) z += expf(row[i] - m);
+  float z = 0.0f, p_num[NPL];
+#pragma unroll
+  for (int j = 0; j < NPL; ++j) {
+    p_num[j] = lane + j * kWave < E ? expf(v[j] - m) : 0.0f;
+    z += p_num[j];
+  }
   z = wave_sum(z);
   float h = 0.0f;
-  for (int i = lane; i < E; i += kWave) {
-    const float p = expf(row[i] - m) / z;
-    h -= p * logf(p > 1e-9f ? p : 1e-9f);
+#pragma unroll
+  for (int j = 0; j < NPL; ++j) {
+    if (lane + j * kWave < E) {
+      const float p = p_num[j] / z;
+      h -= p * logf(p > 1e-9f ? p : 1e-9f);
+    }
   }
   h = wave_sum(h);
   if (lane == 0) {
     entropy[t] = h;
     confidence[t] = 1.0f / z;  // the largest probability is exp(0) / z
   }
-  // top_k rounds of argmax over logit + bias (one f32 add); ties to the lower index; NaN is never greater.
-  uint64_t taken = 0;
+  // top_k rounds of argmax over the biased logits; ties to the lower index. Lane r keeps pick r.
+  int my_id = E;
+  float my_logit = NAN, lmax = -INFINITY;
   for (int r = 0; r < top_k; ++r) {
     float best = -INFINITY;
     int best_i = E;
-    for (int i = lane, j = 0; i < E; i += kWave, ++j) {
-      if ((taken >> j) & 1u) continue;
-      const float v = row[i] + (bias ? bias[i] : 0.0f);
-      if (v > best || (v == best && i < best_i)) {
-        best = v;
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) {
+      const int i = lane + j * kWave;
+      if (biased[j] > best || (biased[j] == best && i < best_i && i < E)) {
+        best = biased[j];
         best_i = i;
       }
     }
@@ -69,23 +87,34 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
         best_i = oi;
       }
     }
-    if (best_i < E && (best_i & (kWave - 1)) == lane) taken |= 1ull << (best_i / kWave);
-    if (lane == 0) {
-      ids[t * top_k + r] = best_i;
-      picked_logit[wave][r] = best_i < E ? row[best_i] : NAN;
+    // The owner of the pick retires it and hands its unbiased logit to every lane.
+    float picked = NAN;
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) {
+      if (lane + j * kWave == best_i) {
+        picked = v[j];
+        biased[j] = -INFINITY;
+        v[j] = -INFINITY;
+      }
     }
+    const int owner = best_i < E ? (best_i & (kWave - 1)) : 0;
+    picked = __shfl(picked, owner);
+    if (best_i >= E) picked = NAN;
+    if (lane == r) {
+      my_id = best_i;
+      my_logit = picked;
+    }
+    lmax = picked > lmax ? picked : lmax;
   }
-  __builtin_amdgcn_wave_barrier();
-  __threadfence_block();
-  // Weights: softmax over the picks of their unbiased logits, summed in pick order.
-  float lmax = -INFINITY;
-  for (int r = 0; r < top_k; ++r) lmax = picked_logit[wave][r] > lmax ? picked_logit[wave][r] : lmax;
+  // Weights: softmax over the picks of their unbiased logits, summed in pick order (lane r holds pick r).
+  const float e_mine = lane < top_k ? expf(my_logit - lmax) : 0.0f;
   float esum = 0.0f;
-  for (int r = 0; r < top_k; ++r) esum += expf(picked_logit[wave][r] - lmax);
-  if (lane < top_k) weights[t * top_k + lane] = expf(picked_logit[wave][lane] - lmax) / esum;
+  for (int r = 0; r < top_k; ++r) esum += __shfl(e_mine, r);
+  if (lane < top_k) {
+    ids[t * top_k + lane] = my_id;
+    weights[t * top_k + lane] = e_mine / esum;
+  }
 }
-
-// ---- decode experts ----------------------------------------------------------------------------------------
 
 // Sorts the P pairs by expert (stable) in LDS. order[g] = pair at sorted position g; returns through
 // group_begin / group_end the positions of group `slot` (the slot-th distinct expert in ascending id order),
@@ -125,13 +154,13 @@ __device__ __forceinline__ void group_pairs(const int32_t* ids, int P, int slot,
   __syncthreads();
 }
 
-// Intermediate rows [i_begin, i_end) of expert e for the cnt <= MT pairs at sorted positions first..: each
-// wavefront takes rows i = i_begin + wave, + kWaves, ...; the pair (gate row i, up row I + i) is its two
-// streamed rows. MT only sets how many activation rows share a pass; a row's arithmetic is the same for any MT.
-// Stages the pairs' latent rows itself (after asking for the first weights), so the whole workgroup calls it.
+// One intermediate row i per wavefront (i = blockIdx.x * waves + wave) of expert e for the cnt <= MT pairs at
+// sorted positions first..: the pair (gate row i, up row I + i) is the wavefront's two streamed rows, all of
+// their loads in flight before the activations are waited for. MT only sets how many activation rows share
+// the pass; a row's arithmetic is the same for any MT. The whole workgroup calls it (it stages x).
 template <int F, int U, int MT>
 __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, int e, int first, int cnt, const int* s_order,
-                                             const int* s_rows, int i_begin, int i_end) {
+                                             const int* s_rows) {
   const int steps = steps_for<F>(a.L);
   const int per_row = x_row_floats<F>(steps);
   const int64_t rb = row_bytes<F>(a.L);
@@ -139,76 +168,91 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
   const int64_t scale_row = F == LX_W_NVFP4 ? a.L / 16 : 0;
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int64_t stack_row0 = static_cast<int64_t>(e) * 2 * a.I;
-  auto rows_fn = [&](int i, const uint8_t* (&rows)[2], const uint8_t* (&scales)[2], const float*& x_image) {
-    const int64_t gate_row = stack_row0 + min(i, a.I - 1), up_row = gate_row + a.I;
+  const int i = blockIdx.x * (blockDim.x / kWave) + wave;
+  auto rows_fn = [&](int ii, const uint8_t* (&rows)[2], const uint8_t* (&scales)[2], const float* (&x_image)[2]) {
+    const int64_t gate_row = stack_row0 + min(ii, a.I - 1), up_row = gate_row + a.I;
     rows[0] = a.gu.data + gate_row * rb;
     rows[1] = a.gu.data + up_row * rb;
     scales[0] = a.gu.scale + gate_row * scale_row;
     scales[1] = a.gu.scale + up_row * scale_row;
-    x_image = lds;
+    x_image[0] = lds;
+    x_image[1] = lds;
   };
-  auto done_fn = [&](int i, float (&acc)[MT][2]) {
+  auto done_fn = [&](int ii, float (&acc)[MT][2]) {
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       acc[m][0] = wave_sum(acc[m][0]);
       acc[m][1] = wave_sum(acc[m][1]);
     }
-    if (lane == 0) {
-      const int64_t gate_row = stack_row0 + i, up_row = gate_row + a.I;
+    if (lane == 0 && ii < a.I) {
+      const int64_t gate_row = stack_row0 + ii, up_row = gate_row + a.I;
       const float sg = stack_factor(F, a.gu, e, gate_row), su = stack_factor(F, a.gu, e, up_row);
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         if (m < cnt) {
           const float g = sg * acc[m][0], u = su * acc[m][1];
-          const int pair = s_order[first + m];
-          a.inter[static_cast<int64_t>(pair) * a.I + i] = f32_to_bf16_bits(silu(g) * u);
+          const int pair = s_order ? s_order[first + m] : first + m;
+          a.inter[static_cast<int64_t>(pair) * a.I + ii] = f32_to_bf16_bits(silu(g) * u);
         }
       }
     }
   };
   RowStreamer<F, MT, 2, U> st(chunks, 0, steps, per_row);
-  const int first_i = i_begin + wave;
-  const int n = first_i < i_end ? (i_end - first_i + kWaves - 1) / kWaves : 0;
-  if (n > 0) st.prefetch(rows_fn, first_i, kWaves, n);
-  stage_x<F, MT>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
+  if constexpr (MT == 1) {
+    // Ask for x, then for the weights, and only then wait for x: loads return in order.
+    const int token = s_rows ? s_rows[0] : first / a.top_k;
+    const uint16_t* xrow = a.latent + static_cast<int64_t>(token) * a.L;
+    XRegs xr;
+    stage_x_load<F>(xr, xrow, LX_BF16, a.L, a.L, steps);
+    st.prefetch(rows_fn, i, 0, 1);
+    if (xr.ready) stage_x_store<F>(xr, lds, LX_BF16, steps);
+    else stage_x<F, 1>(lds, xrow, LX_BF16, a.L, nullptr, 1, a.L, steps);
+  } else {
+    st.prefetch(rows_fn, i, 0, 1);
+    stage_x<F, MT>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
+  }
   __syncthreads();
-  st.run(rows_fn, done_fn, first_i, kWaves, n);
+  st.run(rows_fn, done_fn, i, 0, 1);
 }
 
-// grid = (row blocks, group slots); mt_cap (a power of two, the LDS image's rows) bounds a pass's pairs.
+// grid = (I / wavefronts per workgroup, group slots); mt_cap (a power of two, the LDS image's rows) bounds a
+// pass's pairs. One token: every slot is its own group and nothing is sorted.
 template <int F, int U>
 __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeArgs a, int mt_cap) {
   extern __shared__ __align__(16) float lds[];
   __shared__ int s_ids[kMaxPairs], s_order[kMaxPairs], s_info[4], s_rows[8];
   const int P = a.T * a.top_k;
+  if (a.T == 1) {
+    if (static_cast<int>(blockIdx.y) >= P) return;
+    const int e = __builtin_amdgcn_readfirstlane(a.ids[blockIdx.y]);
+    gate_up_rows<F, U, 1>(a, lds, e, blockIdx.y, 1, nullptr, nullptr);
+    return;
+  }
   group_pairs(a.ids, P, blockIdx.y, s_ids, s_order, s_info);
   if (static_cast<int>(blockIdx.y) >= s_info[0]) return;
   const int begin = s_info[1], end = s_info[2];
   const int e = s_ids[s_order[begin]];
-  const int rows_per_block = (a.I + gridDim.x - 1) / gridDim.x;
-  const int i_begin = blockIdx.x * rows_per_block, i_end = min(a.I, i_begin + rows_per_block);
   // A group larger than the image (an expert repeated within a token) runs mt_cap pairs at a time.
   for (int first = begin; first < end; first += mt_cap) {
     const int cnt = min(mt_cap, end - first);
     __syncthreads();
     if (threadIdx.x < 8) s_rows[threadIdx.x] = static_cast<int>(threadIdx.x) < cnt ? s_order[first + threadIdx.x] / a.top_k : 0;
     __syncthreads();
-    if (cnt <= 1) gate_up_rows<F, U, 1>(a, lds, e, first, cnt, s_order, s_rows, i_begin, i_end);
-    else if (cnt <= 2) gate_up_rows<F, U, 2>(a, lds, e, first, cnt, s_order, s_rows, i_begin, i_end);
-    else if (cnt <= 4) gate_up_rows<F, U, 4>(a, lds, e, first, cnt, s_order, s_rows, i_begin, i_end);
-    else gate_up_rows<F, U, 8>(a, lds, e, first, cnt, s_order, s_rows, i_begin, i_end);
+    if (cnt <= 1) gate_up_rows<F, U, 1>(a, lds, e, first, cnt, s_order, s_rows);
+    else if (cnt <= 2) gate_up_rows<F, U, 2>(a, lds, e, first, cnt, s_order, s_rows);
+    else if (cnt <= 4) gate_up_rows<F, U, 4>(a, lds, e, first, cnt, s_order, s_rows);
+    else gate_up_rows<F, U, 8>(a, lds, e, first, cnt, s_order, s_rows);
   }
 }
 
-// grid = (blocks of output rows, T). x = the token's top_k intermediate rows; slot k streams expert
-// ids[t, k]'s down rows. out[t, l] = w0 * c0 + sum_{k >= 1} w_k * c_k in slot order
-// (engine/cpu/moe.cpp:315-327), c_k = rowfactor * dot. A wavefront's stream is, for each of its pairs of
-// output rows in turn, the top_k experts' copies of those two rows.
+// grid = (L / wavefronts per workgroup, T): one output row l per wavefront. Its stream is the token's top_k
+// experts' copies of row l, four at a time, each against its own slot's intermediate row, and
+// out[t, l] = w0 * c0 + sum_{k >= 1} w_k * c_k in slot order (engine/cpu/moe.cpp:315-327), c_k = rowfactor * dot.
 template <int F, int U>
 __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs a) {
   extern __shared__ __align__(16) float lds[];
   __shared__ int s_rows[8];
-  constexpr int R = 2;
+  constexpr int R = 4;
   const int t = blockIdx.y;
   const int steps = steps_for<F>(a.I);
   const int per_row = x_row_floats<F>(steps);
@@ -217,46 +261,44 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
   const int64_t scale_row = F == LX_W_NVFP4 ? a.I / 16 : 0;
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int top_k = a.top_k;
-  const int groups = (a.L + R - 1) / R;
-  const int groups_per_block = (groups + gridDim.x - 1) / gridDim.x;
-  const int g_begin = blockIdx.x * groups_per_block, g_end = min(groups, g_begin + groups_per_block);
-  const int first_g = g_begin + wave;
-  const int n_mine = first_g < g_end ? (g_end - first_g + kWaves - 1) / kWaves : 0;
+  const int l = blockIdx.x * (blockDim.x / kWave) + wave;
+  const int lc = min(l, a.L - 1);
 
-  // Stream position c = (j-th pair of rows of this wavefront, slot k).
-  auto rows_fn = [&](int c, const uint8_t* (&rows)[R], const uint8_t* (&scales)[R], const float*& x_image) {
-    const int j = c / top_k, k = c - j * top_k;
-    const int l0 = (first_g + j * kWaves) * R;
-    const int e = a.ids[t * top_k + k];
+  // Group c holds slots 4c .. 4c + 3 (a slot past top_k repeats the last one and is not added).
+  auto rows_fn = [&](int c, const uint8_t* (&rows)[R], const uint8_t* (&scales)[R], const float* (&x_image)[R]) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const int64_t row = static_cast<int64_t>(e) * a.L + min(l0 + r, a.L - 1);
+      const int k = min(c * R + r, top_k - 1);
+      const int e = a.ids[t * top_k + k];
+      const int64_t row = static_cast<int64_t>(e) * a.L + lc;
       rows[r] = a.dn.data + row * rb;
       scales[r] = a.dn.scale + row * scale_row;
+      x_image[r] = lds + k * per_row;
     }
-    x_image = lds + k * per_row;
   };
-  float o[R] = {0.0f, 0.0f};
+  float o = 0.0f;
   auto done_fn = [&](int c, float (&acc)[1][R]) {
-    const int j = c / top_k, k = c - j * top_k;
-    const int l0 = (first_g + j * kWaves) * R;
-    const int e = a.ids[t * top_k + k];
-    const float w = a.weights[t * top_k + k];
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const float contrib = stack_factor(F, a.dn, e, static_cast<int64_t>(e) * a.L + min(l0 + r, a.L - 1)) * wave_sum(acc[0][r]);
-      const float wc = w * contrib;
-      o[r] = k == 0 ? wc : o[r] + wc;
-      if (k == top_k - 1 && lane == 0 && l0 + r < a.L) a.out[static_cast<int64_t>(t) * a.L + l0 + r] = o[r];
+      const int k = c * R + r;
+      const float sum = wave_sum(acc[0][r]);
+      if (k < top_k) {
+        const int e = a.ids[t * top_k + k];
+        const float contrib = stack_factor(F, a.dn, e, static_cast<int64_t>(e) * a.L + lc) * sum;
+        const float wc = a.weights[t * top_k + k] * contrib;
+        o = k == 0 ? wc : o + wc;
+      }
     }
   };
+  const int n_groups = (top_k + R - 1) / R;
   RowStreamer<F, 1, R, U> st(chunks, 0, steps, per_row);
-  if (n_mine > 0) st.prefetch(rows_fn, 0, 1, n_mine * top_k);
+  st.prefetch(rows_fn, 0, 1, n_groups);
   if (threadIdx.x < 8) s_rows[threadIdx.x] = t * top_k + min(static_cast<int>(threadIdx.x), top_k - 1);
   __syncthreads();
   stage_x<F, 8>(lds, a.inter, LX_BF16, a.I, s_rows, top_k, a.I, steps);
   __syncthreads();
-  st.run(rows_fn, done_fn, 0, 1, n_mine * top_k);
+  st.run(rows_fn, done_fn, 0, 1, n_groups);
+  if (lane == 0 && l < a.L) a.out[static_cast<int64_t>(t) * a.L + l] = o;
 }
 
 // Rows whose bytes cannot be streamed 16 at a time (K not a multiple of the chunk, or a misaligned stack):
@@ -300,11 +342,6 @@ __global__ void __launch_bounds__(kThreads) decode_down_plain_kernel(const Decod
 }
 
 template <int F>
-constexpr int moe_loads_in_flight() {
-  return F == LX_W_NVFP4 ? 2 : 4;
-}
-
-template <int F>
 bool streamable(const Stack& s, int64_t K, int max_rows) {
   const int64_t rb = row_bytes<F>(K);
   const int steps = steps_for<F>(K);
@@ -321,37 +358,42 @@ void allow_big_lds(Kernel kernel, size_t lds) {
       (void)hipGetLastError();
 }
 
-template <int F>
-int launch_gate_up(const DecodeArgs& a, hipStream_t s) {
+template <int F, int U>
+int launch_gate_up_u(const DecodeArgs& a, hipStream_t s) {
   const int P = a.T * a.top_k;
-  constexpr int U = moe_loads_in_flight<F>();
   // With distinct experts per token a group has at most T pairs; the LDS image holds that many rows.
   const int mt_cap = a.T <= 1 ? 1 : a.T <= 2 ? 2 : a.T <= 4 ? 4 : 8;
   const size_t lds = sizeof(float) * mt_cap * x_row_floats<F>(steps_for<F>(a.L));
-  // Enough workgroups for two per compute unit when every slot holds a group; at least a wavefront's row each.
-  int blocks = (2 * compute_units() + P - 1) / P;
-  const int max_blocks = (a.I + kWaves - 1) / kWaves;
-  if (blocks > max_blocks) blocks = max_blocks;
-  if (blocks < 1) blocks = 1;
   auto kernel = decode_gate_up_kernel<F, U>;
   allow_big_lds(kernel, lds);
-  hipLaunchKernelGGL(kernel, dim3(blocks, P), dim3(kThreads), lds, s, a, mt_cap);
+  hipLaunchKernelGGL(kernel, dim3((a.I + kWaves - 1) / kWaves, P), dim3(kThreads), lds, s, a, mt_cap);
+  return status_of(hipGetLastError());
+}
+
+template <int F>
+int launch_gate_up(const DecodeArgs& a, hipStream_t s) {
+  switch (batch_depth(steps_for<F>(a.L), 4)) {  // two rows a wavefront: four steps each at most
+    case 4: return launch_gate_up_u<F, 4>(a, s);
+    case 2: return launch_gate_up_u<F, 2>(a, s);
+    default: return launch_gate_up_u<F, 1>(a, s);
+  }
+}
+
+template <int F, int U>
+int launch_down_u(const DecodeArgs& a, hipStream_t s) {
+  const size_t lds = sizeof(float) * 8 * x_row_floats<F>(steps_for<F>(a.I));
+  auto kernel = decode_down_kernel<F, U>;
+  allow_big_lds(kernel, lds);
+  hipLaunchKernelGGL(kernel, dim3((a.L + kWaves - 1) / kWaves, a.T), dim3(kThreads), lds, s, a);
   return status_of(hipGetLastError());
 }
 
 template <int F>
 int launch_down(const DecodeArgs& a, hipStream_t s) {
-  constexpr int U = moe_loads_in_flight<F>();
-  const size_t lds = sizeof(float) * 8 * x_row_floats<F>(steps_for<F>(a.I));
-  const int groups = (a.L + 1) / 2;
-  int blocks = (2 * compute_units() + a.T - 1) / a.T;
-  const int max_blocks = (groups + kWaves - 1) / kWaves;
-  if (blocks > max_blocks) blocks = max_blocks;
-  if (blocks < 1) blocks = 1;
-  auto kernel = decode_down_kernel<F, U>;
-  allow_big_lds(kernel, lds);
-  hipLaunchKernelGGL(kernel, dim3(blocks, a.T), dim3(kThreads), lds, s, a);
-  return status_of(hipGetLastError());
+  switch (batch_depth(steps_for<F>(a.I), 2)) {  // four rows a wavefront: two steps each at most
+    case 2: return launch_down_u<F, 2>(a, s);
+    default: return launch_down_u<F, 1>(a, s);
+  }
 }
 
 int64_t round256(int64_t b) { return (b + 255) / 256 * 256; }
@@ -432,8 +474,13 @@ int lx_moe_route(const float* logits, const float* selection_bias, int32_t* ids,
   if (T <= 0) return kOk;
   if (top_k < 1 || top_k > 64 || top_k > E || !logits || !ids || !weights || !entropy || !confidence) return fail(kInvalid);
   if (E > 4096) return fail(kNotSupported);
-  hipLaunchKernelGGL(route_kernel, dim3((T + kWaves - 1) / kWaves), dim3(kThreads), 0, as_stream(stream), logits,
-                     selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  const dim3 grid((T + kWaves - 1) / kWaves), block(kThreads);
+  hipStream_t s = as_stream(stream);
+  if (E <= 64) hipLaunchKernelGGL(route_kernel<1>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  else if (E <= 128) hipLaunchKernelGGL(route_kernel<2>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  else if (E <= 256) hipLaunchKernelGGL(route_kernel<4>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  else if (E <= 1024) hipLaunchKernelGGL(route_kernel<16>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  else hipLaunchKernelGGL(route_kernel<64>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
   return status_of(hipGetLastError());
 }
 

@@ -41,6 +41,16 @@ __host__ __device__ inline int steps_for(int64_t K) {
   return static_cast<int>((K + per_step - 1) / per_step);
 }
 
+// Steps to ask for at once for rows of `steps` steps: the largest power of two up to `cap` that leaves at most
+// a third of the last batch empty (an empty slot re-reads a chunk).
+inline int batch_depth(int steps, int cap) {
+  for (int u = cap; u > 1; u >>= 1) {
+    const int waste = (steps + u - 1) / u * u - steps;
+    if (waste * 3 <= steps) return u;
+  }
+  return 1;
+}
+
 // Stages rows [0, M) of x (f32 or bf16, row stride ld_x, optionally gathered through row_of[m]) into the
 // LDS image `xs` for MT rows of `steps` steps each; everything past K, and rows M .. MT - 1, are zero.
 // Called by the whole workgroup; the caller synchronises afterwards. Rows whose address and stride allow it
@@ -257,9 +267,10 @@ __device__ __forceinline__ void chunk_fma(const Chunk<F>& c, const float* xs, in
 //   ... stage x in LDS, __syncthreads() ...
 //   st.run(rows_fn, done_fn, first_group, group_stride, n_groups);
 //
-// rows_fn(group, rows, scales, xs) fills the R row pointers (and NVFP4 scale rows) of group `group` and the
-// LDS image its products read; done_fn(group, acc) receives the lane sums acc[MT][R] of a finished group (the
-// caller reduces them across the wave). Steps [s_begin, s_end) of every row are taken, in batches of U.
+// rows_fn(group, rows, scales, xs) fills the R row pointers (and NVFP4 scale rows) of group `group` and, per row,
+// the LDS image its products read (one image for all rows in a GEMV; one per row where every row meets its own
+// activations); done_fn(group, acc) receives the lane sums acc[MT][R] of a finished group (the caller reduces
+// them across the wave). Steps [s_begin, s_end) of every row are taken, in batches of U.
 template <int F, int MT, int R, int U>
 struct RowStreamer {
   Chunk<F> buf_a[U][R], buf_b[U][R];
@@ -276,7 +287,7 @@ struct RowStreamer {
   __device__ __forceinline__ void issue(Chunk<F> (&buf)[U][R], RowsFn& rows_fn, int group, int batch) {
     const uint8_t* rows[R];
     const uint8_t* scales[R];
-    const float* xs;
+    const float* xs[R];
     rows_fn(group, rows, scales, xs);
     const int last_step = s_end > s_begin ? s_end - 1 : s_begin;
 #pragma unroll
@@ -290,18 +301,19 @@ struct RowStreamer {
     }
   }
 
-  __device__ __forceinline__ void consume(const Chunk<F> (&buf)[U][R], const float* xs, int batch, float (&acc)[MT][R]) {
+  __device__ __forceinline__ void consume(const Chunk<F> (&buf)[U][R], const float* const (&xs)[R], int batch,
+                                          float (&acc)[MT][R]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int s = s_begin + batch * U + u;
       if (s < s_end) {
-        const float* xl = xs + x_slot<F>(s, lane, 0);
+        const int slot = x_slot<F>(s, lane, 0);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           float a[MT];
 #pragma unroll
           for (int m = 0; m < MT; ++m) a[m] = acc[m][r];
-          chunk_fma<F, MT>(buf[u][r], xl, per_row, a);
+          chunk_fma<F, MT>(buf[u][r], xs[r] + slot, per_row, a);
 #pragma unroll
           for (int m = 0; m < MT; ++m) acc[m][r] = a[m];
         }
@@ -336,7 +348,7 @@ struct RowStreamer {
       first = false;
       const uint8_t* rows[R];
       const uint8_t* scales[R];
-      const float* xs;
+      const float* xs[R];
       rows_fn(group, rows, scales, xs);
       consume(cur, xs, batch, acc);
       if (last_batch) {
