@@ -22,12 +22,15 @@ constexpr int kMaxPairs = 64;
 // ---- routing ---------------------------------------------------------------------------------------------
 
 // One wavefront per token; a lane keeps its NPL logits (elements lane, lane + 64, ...) in registers, so the row
-// is read once. E <= 64 * NPL.
+// is read once. E <= 64 * NPL. The picks: with few experts (NPL <= 4) every element is ranked against all the
+// others (its rank among the biased logits, ties to the lower index, is its pick number); with many, top_k
+// rounds of a wave-wide argmax.
 template <int NPL>
 __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict__ logits, const float* __restrict__ bias,
                                                          int32_t* __restrict__ ids, float* __restrict__ weights,
                                                          float* __restrict__ entropy, float* __restrict__ confidence, int T,
                                                          int E, int top_k) {
+  __shared__ float picked_logit[kWaves][64];
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int64_t t = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
   if (t >= T) return;
@@ -47,7 +50,7 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
   float z = 0.0f, p_num[NPL];
 #pragma unroll
   for (int j = 0; j < NPL; ++j) {
-    p_num[j] = lane + j * kWave < E ? expf(v[j] - m) : 0.0f;
+    p_num[j] = lane + j * kWave < E ? __expf(v[j] - m) : 0.0f;
     z += p_num[j];
   }
   z = wave_sum(z);
@@ -56,7 +59,7 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
   for (int j = 0; j < NPL; ++j) {
     if (lane + j * kWave < E) {
       const float p = p_num[j] / z;
-      h -= p * logf(p > 1e-9f ? p : 1e-9f);
+      h -= p * __logf(p > 1e-9f ? p : 1e-9f);
     }
   }
   h = wave_sum(h);
@@ -64,56 +67,82 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
     entropy[t] = h;
     confidence[t] = 1.0f / z;  // the largest probability is exp(0) / z
   }
-  // top_k rounds of argmax over the biased logits; ties to the lower index. Lane r keeps pick r.
-  int my_id = E;
-  float my_logit = NAN, lmax = -INFINITY;
-  for (int r = 0; r < top_k; ++r) {
-    float best = -INFINITY;
-    int best_i = E;
+  if constexpr (NPL <= 4) {
+    int rank[NPL];
+#pragma unroll
+    for (int j = 0; j < NPL; ++j) rank[j] = 0;
+#pragma unroll
+    for (int j2 = 0; j2 < NPL; ++j2) {
+      for (int l2 = 0; l2 < kWave; ++l2) {
+        const float other = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(biased[j2]), l2));
+        const int oi = l2 + j2 * kWave;
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) {
+          const int i = lane + j * kWave;
+          rank[j] += (other > biased[j] || (other == biased[j] && oi < i)) && oi < E;
+        }
+      }
+    }
+    int ranked = 0;
 #pragma unroll
     for (int j = 0; j < NPL; ++j) {
       const int i = lane + j * kWave;
-      if (biased[j] > best || (biased[j] == best && i < best_i && i < E)) {
-        best = biased[j];
-        best_i = i;
+      // A NaN ranks nowhere (it is greater than nothing and nothing is greater than it): keep it out.
+      const bool ok = i < E && biased[j] == biased[j];
+      ranked += __popcll(__ballot(ok));
+      if (ok && rank[j] < top_k) {
+        ids[t * top_k + rank[j]] = i;
+        picked_logit[wave][rank[j]] = v[j];
       }
     }
+    // Fewer rankable logits than picks: the rest get the id E, as a search that finds nothing returns.
+    if (lane >= ranked && lane < top_k) {
+      ids[t * top_k + lane] = E;
+      picked_logit[wave][lane] = NAN;
+    }
+  } else {
+    for (int r = 0; r < top_k; ++r) {
+      float best = -INFINITY;
+      int best_i = E;
 #pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) {
-      const float ov = __shfl_xor(best, off);
-      const int oi = __shfl_xor(best_i, off);
-      if (ov > best || (ov == best && oi < best_i)) {
-        best = ov;
-        best_i = oi;
+      for (int j = 0; j < NPL; ++j) {
+        const int i = lane + j * kWave;
+        if (biased[j] > best || (biased[j] == best && i < best_i && i < E)) {
+          best = biased[j];
+          best_i = i;
+        }
       }
-    }
-    // The owner of the pick retires it and hands its unbiased logit to every lane.
-    float picked = NAN;
 #pragma unroll
-    for (int j = 0; j < NPL; ++j) {
-      if (lane + j * kWave == best_i) {
-        picked = v[j];
-        biased[j] = -INFINITY;
-        v[j] = -INFINITY;
+      for (int off = 1; off < kWave; off <<= 1) {
+        const float ov = __shfl_xor(best, off);
+        const int oi = __shfl_xor(best_i, off);
+        if (ov > best || (ov == best && oi < best_i)) {
+          best = ov;
+          best_i = oi;
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < NPL; ++j) {
+        if (lane + j * kWave == best_i) {
+          ids[t * top_k + r] = best_i;
+          picked_logit[wave][r] = v[j];
+          biased[j] = -INFINITY;
+        }
+      }
+      if (best_i >= E && lane == 0) {
+        ids[t * top_k + r] = E;
+        picked_logit[wave][r] = NAN;
       }
     }
-    const int owner = best_i < E ? (best_i & (kWave - 1)) : 0;
-    picked = __shfl(picked, owner);
-    if (best_i >= E) picked = NAN;
-    if (lane == r) {
-      my_id = best_i;
-      my_logit = picked;
-    }
-    lmax = picked > lmax ? picked : lmax;
   }
-  // Weights: softmax over the picks of their unbiased logits, summed in pick order (lane r holds pick r).
-  const float e_mine = lane < top_k ? expf(my_logit - lmax) : 0.0f;
+  __builtin_amdgcn_wave_barrier();
+  __threadfence_block();
+  // Weights: softmax over the picks of their unbiased logits, summed in pick order.
+  float lmax = -INFINITY;
+  for (int r = 0; r < top_k; ++r) lmax = picked_logit[wave][r] > lmax ? picked_logit[wave][r] : lmax;
   float esum = 0.0f;
-  for (int r = 0; r < top_k; ++r) esum += __shfl(e_mine, r);
-  if (lane < top_k) {
-    ids[t * top_k + lane] = my_id;
-    weights[t * top_k + lane] = e_mine / esum;
-  }
+  for (int r = 0; r < top_k; ++r) esum += __expf(picked_logit[wave][r] - lmax);
+  if (lane < top_k) weights[t * top_k + lane] = __expf(picked_logit[wave][lane] - lmax) / esum;
 }
 
 // Sorts the P pairs by expert (stable) in LDS. order[g] = pair at sorted position g; returns through

@@ -63,6 +63,44 @@ __device__ __forceinline__ void stage_x(float* xs, const void* x, int x_dtype, i
   const int per_row = steps * kWave * E;
   const int esize = x_dtype == LX_BF16 ? 2 : 4;
   const bool vec = reinterpret_cast<uintptr_t>(x) % 16 == 0 && (ld_x * esize) % 16 == 0 && K % 8 == 0;
+  if (vec) {
+    // All rows at once: item = (row m, vector v of the row), four items in flight per thread.
+    const int vec_shift = x_dtype == LX_BF16 ? 3 : 2;
+    const int n_vec = per_row >> vec_shift, k_vec = static_cast<int>(K) >> vec_shift;
+    const int items = MT * n_vec;
+    for (int it0 = threadIdx.x; it0 < items; it0 += blockDim.x * 4) {
+      u32x4 r[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int it = it0 + u * blockDim.x;
+        const int m = it / n_vec, v = it - m * n_vec;
+        r[u] = u32x4{0u, 0u, 0u, 0u};
+        if (it < items && m < M && v < k_vec) {
+          const int64_t base = static_cast<int64_t>(row_of ? row_of[m] : m) * ld_x;
+          r[u] = *(reinterpret_cast<const u32x4*>(static_cast<const char*>(x) + base * esize) + v);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int it = it0 + u * blockDim.x;
+        if (it < items) {
+          const int m = it / n_vec, v = it - m * n_vec;
+          const int k = v << vec_shift, s = k / (kWave * E), within = k % (kWave * E);
+          float* at = xs + m * per_row + x_slot<F>(s, within / E, within % E);
+          if (x_dtype == LX_BF16) {
+            *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(r[u].x << 16), __uint_as_float(r[u].x & 0xffff0000u),
+                                                  __uint_as_float(r[u].y << 16), __uint_as_float(r[u].y & 0xffff0000u)};
+            *reinterpret_cast<f32x4*>(at + 256) = f32x4{__uint_as_float(r[u].z << 16), __uint_as_float(r[u].z & 0xffff0000u),
+                                                        __uint_as_float(r[u].w << 16), __uint_as_float(r[u].w & 0xffff0000u)};
+          } else {
+            *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(r[u].x), __uint_as_float(r[u].y), __uint_as_float(r[u].z),
+                                                  __uint_as_float(r[u].w)};
+          }
+        }
+      }
+    }
+    return;
+  }
   for (int m = 0; m < MT; ++m) {
     float* dst = xs + m * per_row;
     if (m >= M) {
@@ -70,63 +108,19 @@ __device__ __forceinline__ void stage_x(float* xs, const void* x, int x_dtype, i
       continue;
     }
     const int64_t base = static_cast<int64_t>(row_of ? row_of[m] : m) * ld_x;
-    if (vec && x_dtype == LX_BF16) {
-      const u32x4* src = reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(x) + base);
-      const int n_vec = per_row / 8, k_vec = static_cast<int>(K / 8);
-      for (int v0 = threadIdx.x; v0 < n_vec; v0 += blockDim.x * 4) {
-        u32x4 r[4];
+    for (int k0 = threadIdx.x; k0 < per_row; k0 += blockDim.x * 8) {
+      float r[8];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int v = v0 + u * blockDim.x;
-          r[u] = v < k_vec ? src[v] : u32x4{0u, 0u, 0u, 0u};
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int v = v0 + u * blockDim.x;
-          if (v < n_vec) {
-            const int k = v * 8, s = k / (kWave * E), within = k % (kWave * E);
-            float* at = dst + x_slot<F>(s, within / E, within % E);
-            *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(r[u].x << 16), __uint_as_float(r[u].x & 0xffff0000u),
-                                                  __uint_as_float(r[u].y << 16), __uint_as_float(r[u].y & 0xffff0000u)};
-            *reinterpret_cast<f32x4*>(at + 256) = f32x4{__uint_as_float(r[u].z << 16), __uint_as_float(r[u].z & 0xffff0000u),
-                                                        __uint_as_float(r[u].w << 16), __uint_as_float(r[u].w & 0xffff0000u)};
-          }
-        }
+      for (int u = 0; u < 8; ++u) {
+        const int k = k0 + u * blockDim.x;
+        r[u] = k < K ? load_as_f32(x, x_dtype, base + k) : 0.0f;
       }
-    } else if (vec) {
-      const f32x4* src = reinterpret_cast<const f32x4*>(static_cast<const float*>(x) + base);
-      const int n_vec = per_row / 4, k_vec = static_cast<int>(K / 4);
-      for (int v0 = threadIdx.x; v0 < n_vec; v0 += blockDim.x * 4) {
-        f32x4 r[4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int v = v0 + u * blockDim.x;
-          r[u] = v < k_vec ? src[v] : f32x4{0.f, 0.f, 0.f, 0.f};
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const int v = v0 + u * blockDim.x;
-          if (v < n_vec) {
-            const int k = v * 4, s = k / (kWave * E), within = k % (kWave * E);
-            *reinterpret_cast<f32x4*>(dst + x_slot<F>(s, within / E, within % E)) = r[u];
-          }
-        }
-      }
-    } else {
-      for (int k0 = threadIdx.x; k0 < per_row; k0 += blockDim.x * 8) {
-        float r[8];
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int k = k0 + u * blockDim.x;
-          r[u] = k < K ? load_as_f32(x, x_dtype, base + k) : 0.0f;
-        }
-#pragma unroll
-        for (int u = 0; u < 8; ++u) {
-          const int k = k0 + u * blockDim.x;
-          if (k < per_row) {
-            const int s = k / (kWave * E), within = k % (kWave * E);
-            dst[x_slot<F>(s, within / E, within % E)] = r[u];
-          }
+      for (int u = 0; u < 8; ++u) {
+        const int k = k0 + u * blockDim.x;
+        if (k < per_row) {
+          const int s = k / (kWave * E), within = k % (kWave * E);
+          dst[x_slot<F>(s, within / E, within % E)] = r[u];
         }
       }
     }
