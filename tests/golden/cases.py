@@ -1,0 +1,144 @@
+"""The seeded cases behind the golden vectors in this folder.
+
+Every case builds its inputs from torch's CPU generator (the same bits on any machine of this image; each
+fixture also stores a checksum of its inputs, which the tests check first) and names the backend calls whose
+outputs were recorded. ``run_case(lx, name)`` performs the calls on any library that speaks the lx_* ABI and
+returns {output name: CPU tensor}; make_golden.py runs it on the reference's CPU backend, the tests on the
+oracle and on the GPU library.
+"""
+
+import torch
+
+import ops
+from dromos_amd.abi import W_BF16, W_FP8, W_INT8, W_NVFP4
+from dromos_amd.formats import Weight, master_weight, quantize_reference, quantize_with, random_stack, random_weight
+
+FORMATS = {"bf16": W_BF16, "int8": W_INT8, "fp8": W_FP8, "nvfp4": W_NVFP4}
+
+
+def _bits(t):
+    """Any tensor -> integer view of its bytes, for exact comparison and storage."""
+    t = t.detach().cpu().contiguous()
+    if t.dtype in (torch.float32,):
+        return t.view(torch.int32)
+    if t.dtype in (torch.bfloat16,):
+        return t.view(torch.int16)
+    return t
+
+
+def checksum(tensors):
+    """Order-sensitive 64-bit checksum of a list of tensors' bytes."""
+    h = 1469598103934665603
+    for t in tensors:
+        b = _bits(t).flatten().to(torch.int64)
+        w = torch.arange(1, b.numel() + 1, dtype=torch.int64)
+        h = (h * 1099511628211 + int(((b * w) % 1000003).sum())) % (1 << 61)
+    return h
+
+
+def _quant_master():
+    g = torch.Generator().manual_seed(4101)
+    w = master_weight(24, 96, g)
+    w[3] = 0  # a zero row: scale 1, zero codes
+    w[5, 16:32] = 0  # a zero NVFP4 block
+    w[7, :8] = torch.tensor([0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 3.5, -3.5]).to(torch.bfloat16) * 0.01  # near ties
+    return w
+
+
+def quantize(lx, fmt):
+    w = _quant_master().to(lx.device)
+    q = quantize_with(lx, w, FORMATS[fmt])
+    out = {"data": q.data, "scale": q.scale}
+    if fmt == "nvfp4":
+        out["global"] = torch.tensor([q.glob], dtype=torch.float32)
+    out["dequantized"] = ops.dequantize(lx, q, 24, 96)
+    return [w], out
+
+
+def gemv(lx, fmt, x_dtype, y_dtype):
+    M, N, K = 3, 40, 352
+    g = torch.Generator().manual_seed(4200 + FORMATS[fmt])
+    x = torch.randn(M, K, generator=g).to(x_dtype)
+    w = random_weight(FORMATS[fmt], N, K, 4300 + FORMATS[fmt])
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g).to(y_dtype)
+    y = ops.gemv_w(lx, x.to(lx.device), w.to(lx.device), bias.to(lx.device), y0.clone().to(lx.device), alpha=0.75, beta=0.5)
+    return [x, w.data, bias, y0], {"y": y}
+
+
+def gemm(lx, fmt):
+    M, N, K = 12, 48, 320
+    g = torch.Generator().manual_seed(4400 + FORMATS[fmt])
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = random_weight(FORMATS[fmt], N, K, 4500 + FORMATS[fmt])
+    bias = torch.randn(N, generator=g)
+    y = ops.gemm_w(lx, x.to(lx.device), w.to(lx.device), bias=bias.to(lx.device), alpha=1.5)
+    return [x, w.data, bias], {"y": y}
+
+
+def route(lx):
+    T, E, top_k = 5, 64, 8
+    g = torch.Generator().manual_seed(4600)
+    logits = (torch.randn(T, E, generator=g) * 2).float()
+    logits[1, 10] = logits[1, 3]  # a tie: the lower index wins
+    bias = (torch.randn(E, generator=g) * 0.5).float()
+    bias[10] = bias[3]
+    ids, weights, entropy, confidence = ops.route(lx, logits.to(lx.device), bias.to(lx.device), top_k)
+    return [logits, bias], {"ids": ids, "weights": weights, "entropy": entropy, "confidence": confidence}
+
+
+def _expert_inputs(fmt, T):
+    E, L, I, top_k = 6, 128, 64, 2
+    g = torch.Generator().manual_seed(4700 + T)
+    latent = torch.randn(T, L, generator=g).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E, generator=g)[:top_k] for _ in range(T)]).to(torch.int32)
+    weights = torch.softmax(torch.randn(T, top_k, generator=g), -1).float()
+    gu = random_stack(FORMATS[fmt], E, 2 * I, L, 48)
+    dn = random_stack(FORMATS[fmt], E, L, I, 49)
+    return E, L, I, top_k, latent, ids, weights, gu, dn
+
+
+def experts_decode(lx, fmt):
+    E, L, I, top_k, latent, ids, weights, gu, dn = _expert_inputs(fmt, 3)
+    d = lx.device
+    out = ops.experts_decode(lx, latent.to(d), ids.to(d), weights.to(d), gu.to(d), dn.to(d), I, top_k)
+    return [latent, ids, weights, gu.data, dn.data], {"out": out}
+
+
+def experts_grouped(lx, fmt):
+    E, L, I, top_k, latent, ids, weights, gu, dn = _expert_inputs(fmt, 12)
+    d = lx.device
+    out = ops.experts_grouped(lx, latent.to(d), ids.to(d), weights.to(d), gu.to(d), dn.to(d), I, E, top_k)
+    return [latent, ids, weights, gu.data, dn.data], {"out": out}
+
+
+def experts_bf16(lx):
+    E, L, I, top_k, latent, ids, weights, gu, dn = _expert_inputs("bf16", 4)
+    d = lx.device
+    out = ops.experts_bf16(lx, latent.to(d), ids.to(d), weights.to(d), gu.data.to(d), dn.data.to(d), I, top_k)
+    return [latent, ids, weights, gu.data, dn.data], {"out": out}
+
+
+CASES = {}
+for _f in ("int8", "fp8", "nvfp4"):
+    CASES[f"quantize_{_f}"] = (quantize, (_f,))
+for _f in FORMATS:
+    CASES[f"gemv_{_f}_bf16x_f32y"] = (gemv, (_f, torch.bfloat16, torch.float32))
+    CASES[f"gemm_{_f}"] = (gemm, (_f,))
+    CASES[f"experts_decode_{_f}"] = (experts_decode, (_f,))
+    CASES[f"experts_grouped_{_f}"] = (experts_grouped, (_f,))
+CASES["gemv_int8_f32x_bf16y"] = (gemv, ("int8", torch.float32, torch.bfloat16))
+CASES["gemv_bf16_f32x_f32y"] = (gemv, ("bf16", torch.float32, torch.float32))
+CASES["route"] = (route, ())
+CASES["experts_bf16"] = (experts_bf16, ())
+
+# Outputs whose bits every backend must reproduce (codec and index work); the rest are f32 sums whose last
+# bits depend on the summation order (the reference's own differ between its ISA levels).
+EXACT = {"data", "scale", "global", "dequantized", "ids"}
+
+
+def run_case(lx, name):
+    fn, args = CASES[name]
+    inputs, outputs = fn(lx, *args)
+    lx.sync()
+    return checksum(inputs), {k: _bits(v) for k, v in outputs.items() if v is not None}
