@@ -1,7 +1,8 @@
 #!/usr/bin/env python3
 """Measures the decode matrix-product path on one MI355X: weight-stream GB/s and fraction of the 8 TB/s HBM peak.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cases headline|all] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cases headline|gemv|all] [--no-cpu]
+    python bench.py --pmc-probe      (for rocprofv3 --pmc: a plain copy of known size, then headline launches)
 
 A step is one pass of the hot path over one batch: one lx_gemv_w call (the headline), one skinny GEMM, or one
 routed-experts step, always on a weight copy that was not touched recently (the copies rotate through more
@@ -174,7 +175,7 @@ def make_moe_case(lx, torch, fmt, T, E, L, I, top_k, seed, steps_total):
 def cpu_baseline(torch, fmt, M, N, K, seed, seconds=12.0):
     """The same GEMV on the host cores: the reference's own CPU backend when oracle/_ref holds it (kind
     "reference"), else this repository's plain-C restatement (kind "port"). A bounded sample: calls are
-    repeated on rotated weight copies (> 256 MiB, past the last-level cache) for about `seconds`."""
+    repeated on rotated weight copies (1 GiB in all, past any last-level cache) for about `seconds`."""
     from dromos_amd.abi import DTYPE, F32, FORMATS, Kernels
     from dromos_amd.formats import Weight, master_weight, quantize_with
 
@@ -194,7 +195,7 @@ def cpu_baseline(torch, fmt, M, N, K, seed, seconds=12.0):
     master = master_weight(N, K, g)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w0 = quantize_with(lib, master, FORMATS[fmt])
-    copies = max(2, -(-(288 << 20) // w0.nbytes()))
+    copies = max(2, -(-(1 << 30) // w0.nbytes()))
     ws = [w0] + [Weight(w0.fmt, w0.data.clone(), None if w0.scale is None else w0.scale.clone(), w0.glob) for _ in range(copies - 1)]
     structs = [w.lx() for w in ws]
     y = torch.empty(M, N, dtype=torch.float32)
@@ -231,6 +232,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--cases", default="headline", choices=["headline", "gemv", "all"])
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="no timing: one 256 MiB device copy (the counters' yardstick) and 20 eager headline launches")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported (one MI355X per box)")
@@ -242,6 +245,18 @@ def main():
     from dromos_amd.abi import load_hip
 
     lx = load_hip()  # raises when the library is not built: there is no fallback
+    if args.pmc_probe:
+        a = torch.zeros(256 << 20, dtype=torch.uint8, device="cuda")
+        b = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
+        for _ in range(3):
+            a.copy_(b)  # reads 256 MiB and writes 256 MiB
+        step, nbytes, keep = make_gemv_case(lx, torch, "int8", 1, 14336, 4096, 1001, "gemv_w")
+        for i in range(20):
+            step(i)
+        torch.cuda.synchronize()
+        print(json.dumps({"pmc_probe": {"copy_bytes_read": 256 << 20, "copy_bytes_written": 256 << 20,
+                                        "gemv_algorithmic_bytes": nbytes, "gemv_launches": 20}}))
+        return
     timer = Timer(lx, torch)
     K_STEPS, W = args.steps, args.warmup
 
@@ -323,13 +338,13 @@ def main():
 
 def load_traffic():
     """HBM bytes per launch of the headline kernel from the committed rocprofv3 --pmc summary, or None."""
-    p = ROOT / "profiles" / "gemv_w_int8_14336x4096_m1_traffic.json"
+    p = ROOT / "profiles" / "gemv_w_int8_14336x4096_m1_traffic.txt"
     if not p.exists():
         return None
-    try:
-        return json.loads(p.read_text()).get("hbm_bytes_per_launch")
-    except (ValueError, OSError):
-        return None
+    for line in p.read_text().splitlines():
+        if line.startswith("hbm_bytes_per_launch:"):
+            return int(float(line.split(":", 1)[1]))
+    return None
 
 
 if __name__ == "__main__":
