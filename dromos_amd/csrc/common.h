@@ -125,6 +125,10 @@ struct Fmt<LX_W_NVFP4> {
   static constexpr int kBitsPerK = 4;
 };
 
+// A dword as two bf16 (low half first). Taking the dword by value matters: a bit cast written directly on an
+// element of a vector, `__builtin_bit_cast(bf16x2, v[i])`, has compiled to element 0 for every i.
+__device__ __forceinline__ bf16x2 as_bf16x2(uint32_t d) { return __builtin_bit_cast(bf16x2, d); }
+
 // The values of one dword of a row: 2 (bf16), 4 (int8, fp8) or 8 (nvfp4 codes, unscaled).
 template <int F>
 struct DwordVals {

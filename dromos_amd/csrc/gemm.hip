@@ -37,40 +37,120 @@ struct GemmArgs {
   int64_t ld_y;
   int M, N, K;
   float alpha, beta;
-  int chunks, steps, steps_per_wave;
+  int chunks, steps, steps_per_wave, S;
   int64_t row_bytes, scale_row_bytes;
+  int tiles_per_wg, x_vecs, x_row_vecs, x_pitch, x_iters;  // the LDS activation image (XL kernels)
 };
 
-// The epilogue's operation order (engine/cpu/gemm.cpp:21-34).
-__device__ __forceinline__ void write_out(const GemmArgs& a, int wtype, int m, int n, float sum) {
-  float t = row_factor(wtype, a.scale, a.global, n) * sum;
-  if (a.bias) t += load_as_f32(a.bias, a.bias_dtype, n);
+// The epilogue's operation order (engine/cpu/gemm.cpp:21-34); rf is the row factor, b the bias (0 without one).
+__device__ __forceinline__ void write_out(const GemmArgs& a, int m, int n, float sum, float rf, float b) {
+  float t = rf * sum;
+  if (a.bias) t += b;
   float v = a.alpha * t;
   const int64_t at = m * a.ld_y + n;
   if (a.beta != 0.0f) v = a.beta * load_as_f32(a.y, a.y_dtype, at) + v;
   store_from_f32(a.y, a.y_dtype, at, v);
 }
 
-template <int F, int MT, bool XF32>
+__device__ __forceinline__ void write_out(const GemmArgs& a, int wtype, int m, int n, float sum) {
+  write_out(a, m, n, sum, row_factor(wtype, a.scale, a.global, n), a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f);
+}
+
+// XL: the activation rows (at most 16, MT == 1) are staged once per workgroup into LDS as bf16, behind the
+// wavefronts' regions: rows of x_row_vecs * 8 values (K rounded up to whole weight batches, zero from K on),
+// x_pitch = that + 8 elements apart (16 bytes off a multiple of the banks' span, so the 16 rows of a fragment read
+// fall into different banks). A workgroup then holds `tiles_per_wg` tiles of S wavefronts each, which share the
+// image. Otherwise (any M up to 64) the fragments are read from global memory and a workgroup is one tile.
+template <int F, int MT, bool XF32, bool XL>
 __global__ void __launch_bounds__(kMaxSplit* kWave) skinny_kernel(const GemmArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
-  const int lane = threadIdx.x & (kWave - 1);
-  const int n0 = blockIdx.x * kTileRows;
-  const int64_t n = min(n0 + (lane & 15), a.N - 1);  // past the end: read a valid row, write nothing
-  const uint8_t* rows[1] = {a.w + n * a.row_bytes};
-  const uint8_t* scales[1] = {a.scale + n * a.scale_row_bytes};
+  static_assert(!XL || MT == 1, "only one activation tile is staged in LDS");
+  constexpr int kRegion = wave_region_bytes<1, MT>();
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int S = a.S, tile_in_wg = XL ? wave / S : 0, slice = XL ? wave - tile_in_wg * S : wave;
+  // A tile past the last one (an odd count of tiles and two to a workgroup) repeats the last tile; its outputs are
+  // not written.
+  const int tile_raw = blockIdx.x * (XL ? a.tiles_per_wg : 1) + tile_in_wg;
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const bool tile_live = tile_raw < n_tiles;
+  const int n0 = min(tile_raw, n_tiles - 1) * kTileRows;
+  // Rows past the end of the matrix stand for its last row: read, and never written.
+  const TileRows tiles[1] = {{a.w + n0 * a.row_bytes, a.scale + n0 * a.scale_row_bytes, min(kTileRows, a.N - n0)}};
+  uint8_t* const lds_bytes = reinterpret_cast<uint8_t*>(lds4);
+  uint16_t* const ximg = reinterpret_cast<uint16_t*>(lds_bytes + (blockDim.x / kWave) * kRegion);
   const void* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
-    const int64_t m = min(mt * 16 + (lane & 15), a.M - 1);
-    xrow[mt] = static_cast<const char*>(a.xs.x) + m * a.xs.ld * (XF32 ? 4 : 2);
+    const int m = min(mt * 16 + (lane & 15), a.M - 1);
+    if constexpr (XL) xrow[mt] = ximg + m * a.x_pitch;
+    else xrow[mt] = static_cast<const char*>(a.xs.x) + static_cast<int64_t>(m) * a.xs.ld * (XF32 ? 4 : 2);
   }
-  mfma_tile<F, 1, MT, XF32>(rows, scales, a.chunks, a.steps, a.steps_per_wave, xrow, a.K, lds4, [&](int mt, int q, f32x4(&sums)[1]) {
-    const int m = mt * 16 + (q & 15), nq = n0 + 4 * (q >> 4);
-    if (m < a.M) {
+  // Staging slots: (row m, pass j) in row-major order; a thread's piece of a slot is vector j * blockDim + thread
+  // of row m. The first four slots are asked for before the weights (a wait for them then leaves the weights
+  // in flight), with clamped addresses: what lies past K is replaced by zeros when it is stored.
+  u32x4 xr[4][XF32 ? 2 : 1];
+  auto x_piece = [&](int m, int j, u32x4 (&r)[XF32 ? 2 : 1]) {
+    const int v = min(static_cast<int>(threadIdx.x) + j * static_cast<int>(blockDim.x), a.x_vecs - 1);
+    const char* src = static_cast<const char*>(a.xs.x) + (static_cast<int64_t>(min(m, a.M - 1)) * a.xs.ld + v * 8) * (XF32 ? 4 : 2);
+    r[0] = *reinterpret_cast<const u32x4*>(src);
+    if constexpr (XF32) r[1] = *reinterpret_cast<const u32x4*>(src + 16);
+  };
+  auto x_store = [&](int m, int j, const u32x4 (&r)[XF32 ? 2 : 1]) {
+    const int v = threadIdx.x + j * blockDim.x;
+    u32x4 val = r[0];
+    if constexpr (XF32) {
+      bf16x2 q[4] = {pack_bf16(__uint_as_float(r[0].x), __uint_as_float(r[0].y)), pack_bf16(__uint_as_float(r[0].z), __uint_as_float(r[0].w)),
+                     pack_bf16(__uint_as_float(r[1].x), __uint_as_float(r[1].y)), pack_bf16(__uint_as_float(r[1].z), __uint_as_float(r[1].w))};
+      val = __builtin_bit_cast(u32x4, q);
+    }
+    if (v >= a.x_vecs) val = u32x4{0u, 0u, 0u, 0u};
+    if (v < a.x_row_vecs) *reinterpret_cast<u32x4*>(ximg + m * a.x_pitch + v * 8) = val;
+  };
+  if constexpr (XL) {
+    int m = 0, j = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      x_piece(m, j, xr[u]);
+      if (++j == a.x_iters) j = 0, ++m;
+    }
+  }
+  const bool bias_f32 = a.bias && a.bias_dtype == LX_F32;
+  float rf[4], bs[4];
+  auto between = [&] {
+    // The epilogue's row factors and f32 biases: a lane always finishes the same four weight rows.
+    const int nq = n0 + 4 * (lane >> 4);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = min(nq + r, a.N - 1);
+      rf[r] = row_factor(F, a.scale, a.global, n);
+      bs[r] = bias_f32 ? static_cast<const float*>(a.bias)[n] : 0.0f;
+    }
+    if constexpr (XL) {
+      int m = 0, j = 0;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (m < a.M) x_store(m, j, xr[u]);
+        if (++j == a.x_iters) j = 0, ++m;
+      }
+      while (m < a.M) {
+        u32x4 r[XF32 ? 2 : 1];
+        x_piece(m, j, r);
+        x_store(m, j, r);
+        if (++j == a.x_iters) j = 0, ++m;
+      }
+      __syncthreads();
+    }
+  };
+  constexpr int XS = XL ? kXLds : XF32 ? kXGlobalF32 : kXGlobalBf16;
+  mfma_tile<F, 1, MT, XS>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.K,
+                          reinterpret_cast<f32x4*>(lds_bytes + tile_in_wg * S * kRegion), S, slice, between,
+                          [&](int mt, int q, f32x4(&sums)[1]) {
+    const int m = mt * 16 + (q & 15), nq = n0 + 4 * (q >> 4);  // q % 64 == lane: rf and bs are this slot's
+    if (m < a.M && tile_live) {
 #pragma unroll
       for (int r = 0; r < 4; ++r)
-        if (nq + r < a.N) write_out(a, F, m, nq + r, sums[0][r]);
+        if (nq + r < a.N)
+          write_out(a, m, nq + r, sums[0][r], rf[r], bias_f32 || !a.bias ? bs[r] : load_as_f32(a.bias, a.bias_dtype, nq + r));
     }
   });
 }
@@ -104,27 +184,51 @@ __global__ void __launch_bounds__(256) gemm_plain_kernel(const GemmArgs a, int w
   }
 }
 
-template <int F, int MT, bool XF32>
-int launch_skinny_x(const GemmArgs& a, int S, hipStream_t stream) {
-  const size_t lds = S > 1 ? sizeof(f32x4) * S * MT * kWave : 0;
-  auto kernel = skinny_kernel<F, MT, XF32>;
+constexpr size_t kLdsMax = 160 * 1024;
+
+template <int F, int MT, bool XF32, bool XL>
+int launch_skinny_x(const GemmArgs& a, size_t lds, unsigned grid, unsigned threads, hipStream_t stream) {
+  auto kernel = skinny_kernel<F, MT, XF32, XL>;
   if (lds > 48 * 1024) {
     static thread_local bool raised = false;
     if (!raised) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024) !=
-          hipSuccess)
+      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax) != hipSuccess)
         (void)hipGetLastError();
       raised = true;
     }
   }
-  const unsigned grid = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(S * kWave), lds, stream, a);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, a);
   return status_of(hipGetLastError());
 }
 
 template <int F, int MT>
-int launch_skinny(const GemmArgs& a, int S, hipStream_t stream) {
-  return a.xs.dtype == LX_F32 ? launch_skinny_x<F, MT, true>(a, S, stream) : launch_skinny_x<F, MT, false>(a, S, stream);
+int launch_skinny(GemmArgs a, hipStream_t stream) {
+  const int S = a.S;
+  const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
+  if constexpr (MT == 1) {
+    // The activation image: rows as long as the last weight batch reaches, zero past K.
+    constexpr int kBatchElems = (kLoadsInFlight / 1) * 4 * Fmt<F>::kElems;
+    const int row_elems = (a.K + kBatchElems - 1) / kBatchElems * kBatchElems;
+    const size_t image = static_cast<size_t>(a.M) * (row_elems + 8) * 2;
+    // Two tiles to a workgroup when they fit: twice the wavefronts behind one image.
+    int tiles_per_wg = 2 * S <= kMaxSplit && n_tiles >= 512 ? 2 : 1;
+    if (tile_lds_bytes(tiles_per_wg * S, 1, 1) + image > kLdsMax) tiles_per_wg = 1;
+    const size_t lds = tile_lds_bytes(tiles_per_wg * S, 1, 1) + image;
+    if (lds <= kLdsMax) {
+      const unsigned threads = tiles_per_wg * S * kWave;
+      a.tiles_per_wg = tiles_per_wg;
+      a.x_vecs = a.K / 8;
+      a.x_row_vecs = row_elems / 8;
+      a.x_pitch = row_elems + 8;
+      a.x_iters = (a.x_row_vecs + threads - 1) / threads;
+      const unsigned grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
+      return a.xs.dtype == LX_F32 ? launch_skinny_x<F, 1, true, true>(a, lds, grid, threads, stream)
+                                  : launch_skinny_x<F, 1, false, true>(a, lds, grid, threads, stream);
+    }
+  }
+  const size_t lds = tile_lds_bytes(S, 1, MT);
+  return a.xs.dtype == LX_F32 ? launch_skinny_x<F, MT, true, false>(a, lds, n_tiles, S * kWave, stream)
+                              : launch_skinny_x<F, MT, false, false>(a, lds, n_tiles, S * kWave, stream);
 }
 
 template <int F>
@@ -145,7 +249,9 @@ int launch_format(GemmArgs a, const char* x0, char* y0, int M, int x_esize, int 
   a.steps = load_steps_for<F>(a.K);
   int S = split_for<F>(a.K, 1);
   if (const char* e = getenv("DRO_SKINNY_SPLIT")) S = atoi(e);
-  a.steps_per_wave = (a.steps + S - 1) / S;
+  // Slices are whole weight batches (the row's last one may be cut short by the row's end).
+  a.steps_per_wave = ((a.steps + S - 1) / S + kLoadsInFlight - 1) / kLoadsInFlight * kLoadsInFlight;
+  a.S = S;
   // Up to 64 activation rows a pass; every pass is the same arithmetic per row.
   for (int m0 = 0; m0 < M; m0 += 64) {
     a.M = M - m0 < 64 ? M - m0 : 64;
@@ -153,10 +259,10 @@ int launch_format(GemmArgs a, const char* x0, char* y0, int M, int x_esize, int 
     a.y = y0 + static_cast<int64_t>(m0) * a.ld_y * y_esize;
     int st;
     switch ((a.M + 15) / 16) {
-      case 1: st = launch_skinny<F, 1>(a, S, stream); break;
-      case 2: st = launch_skinny<F, 2>(a, S, stream); break;
-      case 3: st = launch_skinny<F, 3>(a, S, stream); break;
-      default: st = launch_skinny<F, 4>(a, S, stream); break;
+      case 1: st = launch_skinny<F, 1>(a, stream); break;
+      case 2: st = launch_skinny<F, 2>(a, stream); break;
+      case 3: st = launch_skinny<F, 3>(a, stream); break;
+      default: st = launch_skinny<F, 4>(a, stream); break;
     }
     if (st) return st;
   }

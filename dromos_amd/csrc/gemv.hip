@@ -18,7 +18,7 @@ namespace dro {
 namespace {
 
 constexpr int kThreads = 256;  // the plain kernel's workgroup
-constexpr int kMaxThreads = 1024;  // the streaming kernel's workgroup is chosen per launch, up to this
+constexpr int kMaxThreads = 512;  // the streaming kernel's workgroup is chosen per launch, up to this
 constexpr int kMaxWaves = kMaxThreads / kWave;
 constexpr int kLdsFloats = 32 * 1024;  // 128 KB of x at most: one workgroup per compute unit then
 
@@ -61,11 +61,13 @@ __device__ __forceinline__ void write_out(const GemvArgs& a, int wtype, int m, i
 // group's steps when S > 1), and every wavefront asks for its whole share of the weights (up to two batches of
 // U steps) before anything else: many short-lived wavefronts, each with all its loads in flight, keep the
 // memory system busier than a few long-lived ones.
-template <int F, int MT, int R, int U>
+// XB: the activations are bf16 and go into the packed image (two products per instruction); otherwise the f32 image.
+// ONE: a wavefront's share of a row's steps fits one batch of U (the usual case at decode sizes).
+template <int F, int MT, int R, int U, bool XB, bool ONE>
 __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs a) {
   extern __shared__ __align__(16) float lds[];
   const int steps = a.steps;
-  const int per_row = x_row_floats<F>(steps);
+  const int per_row = x_row_words<F, XB>(steps);
   float* xs = lds;
   float* partial = lds + MT * per_row;  // [waves][MT * R] when S > 1
 
@@ -119,17 +121,25 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs
     }
   };
 
-  RowStreamer<F, MT, R, U> st(a.chunks, s_begin, s_end, per_row);
+  RowStreamer<F, MT, R, U, XB, ONE> st(a.chunks, s_begin, s_end, per_row);
+  auto stage_all = [&] {
+    if constexpr (XB) stage_x_pairs<F, MT>(reinterpret_cast<uint32_t*>(xs), static_cast<const uint16_t*>(a.x), a.ld_x, nullptr, a.M, a.K, steps);
+    else stage_x<F, MT>(xs, a.x, a.x_dtype, a.ld_x, nullptr, a.M, a.K, steps);
+  };
   if constexpr (MT == 1) {
     // Ask for x, then for the weights, and only then wait for x: loads return in order.
     XRegs xr;
     stage_x_load<F>(xr, a.x, a.x_dtype, a.ld_x, a.K, steps);
     st.prefetch(rows_fn, group, 0, 1);
-    if (xr.ready) stage_x_store<F>(xr, xs, a.x_dtype, steps);
-    else stage_x<F, MT>(xs, a.x, a.x_dtype, a.ld_x, nullptr, a.M, a.K, steps);
+    if (xr.ready) {
+      if constexpr (XB) stage_x_store_pairs<F>(xr, reinterpret_cast<uint32_t*>(xs), steps);
+      else stage_x_store<F>(xr, xs, a.x_dtype, steps);
+    } else {
+      stage_all();
+    }
   } else {
     st.prefetch(rows_fn, group, 0, 1);
-    stage_x<F, MT>(xs, a.x, a.x_dtype, a.ld_x, nullptr, a.M, a.K, steps);
+    stage_all();
   }
   __syncthreads();
   st.run(rows_fn, done_fn, group, 0, 1);
@@ -179,39 +189,50 @@ struct Shape {
 // so rows of few steps are taken several at a time.
 Shape shape_for(int wtype, int steps) {
   Shape s{wtype == LX_W_NVFP4 ? 512 : 256, batch_depth(steps, 8)};
-  if (const char* e = getenv("DRO_GEMV_THREADS")) s.threads = atoi(e);
-  if (const char* e = getenv("DRO_GEMV_DEPTH")) s.depth = atoi(e);
   return s;
 }
 
-template <int F, int MT, int R, int U>
+template <int F, int MT, int R, int U, bool XB>
 int launch_stream(GemvArgs a, const Shape& shape, hipStream_t stream) {
   const int waves = shape.threads / kWave;
-  const size_t lds = sizeof(float) * (static_cast<size_t>(MT) * x_row_floats<F>(a.steps) + waves * MT * R);
+  const size_t lds = sizeof(float) * (static_cast<size_t>(MT) * x_row_words<F, XB>(a.steps) + waves * MT * R);
   const int groups_per_wg = waves / a.split;
   const int64_t n_groups = (a.N + R - 1) / R;
   const int64_t grid = (n_groups + groups_per_wg - 1) / groups_per_wg;
-  auto kernel = gemv_stream_kernel<F, MT, R, U>;
-  if (lds > 48 * 1024) {
-    static thread_local bool raised = false;
-    if (!raised) {
-      if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                              160 * 1024 - 256) != hipSuccess)
-        (void)hipGetLastError();
-      raised = true;
+  auto launch = [&](auto kernel) {
+    if (lds > 48 * 1024) {
+      static thread_local bool raised = false;  // one per kernel: the lambda is instantiated per kernel type
+      if (!raised) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
+                                160 * 1024 - 256) != hipSuccess)
+          (void)hipGetLastError();
+        raised = true;
+      }
     }
-  }
-  hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(shape.threads), lds, stream, a);
-  return status_of(hipGetLastError());
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(shape.threads), lds, stream, a);
+    return status_of(hipGetLastError());
+  };
+  return a.steps_per_part <= U ? launch(gemv_stream_kernel<F, MT, R, U, XB, true>) : launch(gemv_stream_kernel<F, MT, R, U, XB, false>);
 }
 
-template <int F, int MT>
+// A wavefront asks for about 8 KB (one activation row) or 16 KB (several: the rows' products share the
+// activation reads) of weights at once: rows of few steps are taken several at a time.
+template <int F, int MT, bool XB>
 int launch_rows(const GemvArgs& a, const Shape& shape, hipStream_t stream) {
-  switch (shape.depth) {
-    case 8: return launch_stream<F, MT, 1, 8>(a, shape, stream);
-    case 4: return launch_stream<F, MT, 2, 4>(a, shape, stream);
-    case 2: return launch_stream<F, MT, 4, 2>(a, shape, stream);
-    default: return launch_stream<F, MT, 4, 1>(a, shape, stream);
+  if constexpr (MT == 1) {
+    switch (shape.depth) {
+      case 8: return launch_stream<F, MT, 1, 8, XB>(a, shape, stream);
+      case 4: return launch_stream<F, MT, 2, 4, XB>(a, shape, stream);
+      case 2: return launch_stream<F, MT, 4, 2, XB>(a, shape, stream);
+      default: return launch_stream<F, MT, 4, 1, XB>(a, shape, stream);
+    }
+  } else {
+    switch (shape.depth) {
+      case 8: return launch_stream<F, MT, 2, 8, XB>(a, shape, stream);
+      case 4: return launch_stream<F, MT, 4, 4, XB>(a, shape, stream);
+      case 2: return launch_stream<F, MT, 4, 2, XB>(a, shape, stream);
+      default: return launch_stream<F, MT, 4, 1, XB>(a, shape, stream);
+    }
   }
 }
 
@@ -224,8 +245,10 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
                            (F != LX_W_NVFP4 || reinterpret_cast<uintptr_t>(a.scale) % 2 == 0);
   // Activation rows a pass can hold in LDS: a function of K only. More rows than that run as several
   // passes over the weights; each row's arithmetic is the same in any pass, so its bits do not change.
+  const bool xb = a.x_dtype == LX_BF16;
+  const int64_t row_words = xb ? x_row_words<F, true>(steps) : x_row_words<F, false>(steps);
   int fit = 8;
-  while (fit >= 1 && static_cast<int64_t>(fit) * x_row_floats<F>(steps) + kMaxWaves * fit * 4 > kLdsFloats) fit /= 2;
+  while (fit >= 1 && fit * row_words + kMaxWaves * fit * 4 > kLdsFloats) fit /= 2;
   if (!vector_rows || fit < 1) {
     const int waves = kThreads / kWave;
     const unsigned grid = static_cast<unsigned>((a.N + waves - 1) / waves);
@@ -253,10 +276,10 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
     const Shape shape = shape_for(F, steps);
     int st;
     switch (mt) {
-      case 1: st = launch_rows<F, 1>(a, shape, stream); break;
-      case 2: st = launch_rows<F, 2>(a, shape, stream); break;
-      case 4: st = launch_rows<F, 4>(a, shape, stream); break;
-      default: st = launch_rows<F, 8>(a, shape, stream); break;
+      case 1: st = xb ? launch_rows<F, 1, true>(a, shape, stream) : launch_rows<F, 1, false>(a, shape, stream); break;
+      case 2: st = xb ? launch_rows<F, 2, true>(a, shape, stream) : launch_rows<F, 2, false>(a, shape, stream); break;
+      case 4: st = xb ? launch_rows<F, 4, true>(a, shape, stream) : launch_rows<F, 4, false>(a, shape, stream); break;
+      default: st = xb ? launch_rows<F, 8, true>(a, shape, stream) : launch_rows<F, 8, false>(a, shape, stream); break;
     }
     if (st) return st;
   }

@@ -132,16 +132,17 @@ template <int F, int MT>
 __device__ __forceinline__ void gate_up_tile(const GroupedArgs& a, int e, int g0, int rows, f32x4* lds) {
   const int lane = threadIdx.x & (kWave - 1);
   const int i0 = blockIdx.x * kTileRows;
-  const int64_t gate_row = static_cast<int64_t>(e) * 2 * a.I + min(i0 + (lane & 15), a.I - 1), up_row = gate_row + a.I;
-  const uint8_t* wrows[2] = {a.gu.data + gate_row * a.row_bytes, a.gu.data + up_row * a.row_bytes};
-  const uint8_t* scales[2] = {a.gu.scale + gate_row * a.scale_row_bytes, a.gu.scale + up_row * a.scale_row_bytes};
+  const int64_t gate_row = static_cast<int64_t>(e) * 2 * a.I + i0, up_row = gate_row + a.I;
+  const int valid = min(kTileRows, a.I - i0);
+  const TileRows tiles[2] = {{a.gu.data + gate_row * a.row_bytes, a.gu.scale + gate_row * a.scale_row_bytes, valid},
+                             {a.gu.data + up_row * a.row_bytes, a.gu.scale + up_row * a.scale_row_bytes, valid}};
   const void* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int pair = a.t.order[g0 + min(mt * 16 + (lane & 15), rows - 1)];
     xrow[mt] = a.latent + static_cast<int64_t>(pair / a.top_k) * a.L;
   }
-  mfma_tile<F, 2, MT, false>(wrows, scales, a.chunks, a.steps, a.steps_per_wave, xrow, a.L, lds, [&](int mt, int q, f32x4(&sums)[2]) {
+  mfma_tile<F, 2, MT, kXGlobalBf16>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.L, lds, blockDim.x / kWave, __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), [] {}, [&](int mt, int q, f32x4(&sums)[2]) {
     const int m = mt * 16 + (q & 15), i = i0 + 4 * (q >> 4);
     if (m >= rows) return;
     const int64_t stack_row = static_cast<int64_t>(e) * 2 * a.I + i;
@@ -174,13 +175,12 @@ template <int F, int MT>
 __device__ __forceinline__ void down_tile(const GroupedArgs& a, int e, int g0, int rows, f32x4* lds) {
   const int lane = threadIdx.x & (kWave - 1);
   const int l0 = blockIdx.x * kTileRows;
-  const int64_t row = static_cast<int64_t>(e) * a.L + min(l0 + (lane & 15), a.L - 1);
-  const uint8_t* wrows[1] = {a.dn.data + row * a.row_bytes};
-  const uint8_t* scales[1] = {a.dn.scale + row * a.scale_row_bytes};
+  const int64_t row = static_cast<int64_t>(e) * a.L + l0;
+  const TileRows tiles[1] = {{a.dn.data + row * a.row_bytes, a.dn.scale + row * a.scale_row_bytes, min(kTileRows, a.L - l0)}};
   const void* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) xrow[mt] = a.inter + static_cast<int64_t>(g0 + min(mt * 16 + (lane & 15), rows - 1)) * a.I;
-  mfma_tile<F, 1, MT, false>(wrows, scales, a.chunks, a.steps, a.steps_per_wave, xrow, a.I, lds, [&](int mt, int q, f32x4(&sums)[1]) {
+  mfma_tile<F, 1, MT, kXGlobalBf16>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.I, lds, blockDim.x / kWave, __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), [] {}, [&](int mt, int q, f32x4(&sums)[1]) {
     const int m = mt * 16 + (q & 15), l = l0 + 4 * (q >> 4);
     if (m >= rows) return;
     const int64_t stack_row = static_cast<int64_t>(e) * a.L + l;
@@ -248,7 +248,7 @@ int launch_stage(Kernel kernel, GroupedArgs a, int64_t K, int NT, int out_rows, 
   a.steps_per_wave = (a.steps + S - 1) / S;
   const int64_t P = static_cast<int64_t>(a.T) * a.top_k;
   const int mt_max = static_cast<int>(((P < kTileTokens ? P : kTileTokens) + 15) / 16);
-  const size_t lds = S > 1 ? sizeof(f32x4) * S * NT * mt_max * kWave : 0;
+  const size_t lds = tile_lds_bytes(S, NT, mt_max);
   if (lds > 48 * 1024)
     if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024) !=
         hipSuccess)

@@ -6,32 +6,56 @@
 // the arithmetic in a second register buffer, across group boundaries too, so a wavefront always has a
 // batch in flight while it multiplies the previous one.
 //
-// The activations sit in LDS as f32, laid out so that the 16 bytes a lane reads next are always 16 bytes
-// after its neighbour's (no bank conflicts): the k values of chunk (s, l) are stored as kElems / 4 groups of
-// four, group q at float index  s * 64 * kElems + q * 256 + l * 4.  The image is zero past K, so a lane
-// whose chunk lies past the end of the row (its load is clamped to the row's last chunk) adds exact zeros.
+// The activations sit in LDS, laid out so that the 16 bytes a lane reads next are always 16 bytes after its
+// neighbour's (no bank conflicts). Two images (XB says which):
+//   f32 (XB = false, any activation type): the k values of chunk (s, l) are stored as kElems / 4 groups of
+//     four, group q at word index  s * 64 * kElems + q * 256 + l * 4;  products are f32 FMAs.
+//   packed bf16 (XB = true, bf16 activations): groups of eight k (four words of two bf16), group j at word
+//     index  s * 32 * kElems + j * 256 + l * 4;  the weights are expanded to bf16 pairs (exactly: every stored
+//     format fits) and v_dot2c_f32_bf16 adds two products per instruction: half the LDS bytes and about half
+//     the instructions.
+// Either image is zero past K, so a lane whose chunk lies past the end of the row (its load is clamped to the
+// row's last chunk) adds exact zeros.
 //
 // Every (activation row, weight row) pair keeps one f32 accumulator per lane, fed in ascending step order,
 // and the 64 lane sums are combined by one fixed tree (wave_sum). The order never depends on how many
 // activation rows share the pass (MT), how many weight rows the wave holds (R) or the batch depth (U), so an
-// output's bits depend only on its own x row, its weight row and the K split.
+// output's bits depend only on its own x row (and its type), its weight row and the K split.
 #pragma once
 
 #include "common.h"
 
 namespace dro {
 
-// Float index in the LDS image of x of element j of chunk (s, l); see the layout above.
+// Word (4-byte) index in the f32 image of element j of chunk (s, l); see the layout above.
 template <int F>
 __device__ __forceinline__ int x_slot(int s, int l, int j) {
   constexpr int E = Fmt<F>::kElems;
   return s * (kWave * E) + (j >> 2) * 256 + l * 4 + (j & 3);
 }
 
-// Floats the LDS image of one x row takes for a K of `steps` wave steps.
+// Word index in the packed bf16 image of the pair that holds element j of chunk (s, l) (j & 1 picks the half).
+template <int F>
+__device__ __forceinline__ int x_pair_slot(int s, int l, int j) {
+  constexpr int E = Fmt<F>::kElems;
+  return s * (kWave * E / 2) + (j >> 3) * 256 + l * 4 + ((j & 7) >> 1);
+}
+
+// Word index of a lane's chunk (s, lane) in either image.
+template <int F, bool XB>
+__device__ __forceinline__ int x_chunk_word(int s, int lane) {
+  return XB ? x_pair_slot<F>(s, lane, 0) : x_slot<F>(s, lane, 0);
+}
+
+// Words the LDS image of one x row takes for a K of `steps` wave steps.
 template <int F>
 __host__ __device__ constexpr int x_row_floats(int steps) {
   return steps * kWave * Fmt<F>::kElems;
+}
+
+template <int F, bool XB>
+__host__ __device__ constexpr int x_row_words(int steps) {
+  return steps * kWave * Fmt<F>::kElems / (XB ? 2 : 1);
 }
 
 // Wave steps that cover K values of format F.
@@ -127,6 +151,52 @@ __device__ __forceinline__ void stage_x(float* xs, const void* x, int x_dtype, i
   }
 }
 
+// The packed bf16 image of rows [0, M) of bf16 x (row stride ld_x, optionally gathered through row_of[m]) for
+// MT rows of `steps` steps each; everything past K, and rows M .. MT - 1, are zero. As stage_x otherwise.
+template <int F, int MT>
+__device__ __forceinline__ void stage_x_pairs(uint32_t* xs, const uint16_t* x, int64_t ld_x, const int* row_of, int M, int64_t K,
+                                              int steps) {
+  constexpr int E = Fmt<F>::kElems;
+  const int per_row = x_row_words<F, true>(steps);
+  const bool vec = reinterpret_cast<uintptr_t>(x) % 16 == 0 && (ld_x * 2) % 16 == 0 && K % 8 == 0;
+  if (vec) {
+    const int n_vec = per_row >> 2, k_vec = static_cast<int>(K) >> 3;
+    const int items = MT * n_vec;
+    for (int it0 = threadIdx.x; it0 < items; it0 += blockDim.x * 4) {
+      u32x4 r[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int it = it0 + u * blockDim.x;
+        const int m = it / n_vec, v = it - m * n_vec;
+        r[u] = u32x4{0u, 0u, 0u, 0u};
+        if (it < items && m < M && v < k_vec) {
+          const int64_t base = static_cast<int64_t>(row_of ? row_of[m] : m) * ld_x;
+          r[u] = *(reinterpret_cast<const u32x4*>(x + base) + v);
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int it = it0 + u * blockDim.x;
+        if (it < items) {
+          const int m = it / n_vec, v = it - m * n_vec;
+          const int k = v << 3, st = k / (kWave * E), within = k % (kWave * E);
+          *reinterpret_cast<u32x4*>(xs + m * per_row + x_pair_slot<F>(st, within / E, within % E)) = r[u];
+        }
+      }
+    }
+    return;
+  }
+  uint16_t* halves = reinterpret_cast<uint16_t*>(xs);
+  for (int m = 0; m < MT; ++m) {
+    const int64_t base = m < M ? static_cast<int64_t>(row_of ? row_of[m] : m) * ld_x : 0;
+    for (int k = threadIdx.x; k < per_row * 2; k += blockDim.x) {
+      const int st = k / (kWave * E), within = k % (kWave * E);
+      const int j = within % E;
+      halves[2 * (m * per_row + x_pair_slot<F>(st, within / E, j)) + (j & 1)] = m < M && k < K ? x[base + k] : uint16_t{0};
+    }
+  }
+}
+
 // The same staging in two phases for one activation row, so a kernel can ask for x, then for its first
 // weights, and only then wait for x: XRegs holds a thread's share of the row between the two calls. Usable
 // when the row can be read 16 bytes at a time and a thread's share is at most kVecs vectors; otherwise
@@ -175,6 +245,21 @@ __device__ __forceinline__ void stage_x_store(const XRegs& r, float* xs, int x_d
         *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(r.v[u].x), __uint_as_float(r.v[u].y), __uint_as_float(r.v[u].z),
                                               __uint_as_float(r.v[u].w)};
       }
+    }
+  }
+}
+
+// The second phase for the packed bf16 image (the row is bf16: its vectors go in as they are).
+template <int F>
+__device__ __forceinline__ void stage_x_store_pairs(const XRegs& r, uint32_t* xs, int steps) {
+  constexpr int E = Fmt<F>::kElems;
+  const int n_vec = x_row_words<F, true>(steps) >> 2;
+#pragma unroll
+  for (int u = 0; u < XRegs::kVecs; ++u) {
+    const int v = threadIdx.x + u * blockDim.x;
+    if (v < n_vec) {
+      const int k = v << 3, st = k / (kWave * E), within = k % (kWave * E);
+      *reinterpret_cast<u32x4*>(xs + x_pair_slot<F>(st, within / E, within % E)) = r.v[u];
     }
   }
 }
@@ -254,9 +339,90 @@ __device__ __forceinline__ void chunk_fma(const Chunk<F>& c, const float* xs, in
   }
 }
 
+// The pairs of one dword of a chunk as bf16 (exact for every format): BF16 1, INT8 / FP8 2, NVFP4 4 pairs.
+template <int F>
+__device__ __forceinline__ void dword_pairs(uint32_t d, bf16x2* out);
+
+template <>
+__device__ __forceinline__ void dword_pairs<LX_W_BF16>(uint32_t d, bf16x2* out) {
+  out[0] = as_bf16x2(d);
+}
+
+template <>
+__device__ __forceinline__ void dword_pairs<LX_W_INT8>(uint32_t d, bf16x2* out) {
+  float v[4];
+  decode_dword<LX_W_INT8>(d, v);
+  const f32x2 lo = {v[0], v[1]}, hi = {v[2], v[3]};
+  out[0] = __builtin_convertvector(lo, bf16x2);
+  out[1] = __builtin_convertvector(hi, bf16x2);
+}
+
+template <>
+__device__ __forceinline__ void dword_pairs<LX_W_FP8>(uint32_t d, bf16x2* out) {
+  out[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d, 1.0f, false);
+  out[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp8(d, 1.0f, true);
+}
+
+template <>
+__device__ __forceinline__ void dword_pairs<LX_W_NVFP4>(uint32_t d, bf16x2* out) {
+  out[0] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 0);
+  out[1] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 1);
+  out[2] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 2);
+  out[3] = __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(d, 1.0f, 3);
+}
+
+// chunk_fma on the packed bf16 image: xs points at the image's words of row 0 for this lane's chunk, per_row words
+// separate the rows; a += w0 * x0 + w1 * x1 per instruction, pairs in ascending k.
+template <int F, int MT>
+__device__ __forceinline__ void chunk_dot2(const Chunk<F>& c, const uint32_t* xs, int per_row, float (&acc)[MT]) {
+  constexpr int P = DwordVals<F>::kCount / 2;  // pairs per dword
+  if constexpr (F == LX_W_NVFP4) {
+    // Two blocks of 16 codes (two dwords, i.e. two groups of eight k): summed from zero, scaled once.
+#pragma unroll
+    for (int b = 0; b < 2; ++b) {
+      const float scale = b == 0 ? e4m3_byte_to_f32<0>(c.scales) : e4m3_byte_to_f32<1>(c.scales);
+      float part[MT];
+#pragma unroll
+      for (int m = 0; m < MT; ++m) part[m] = 0.0f;
+#pragma unroll
+      for (int d = 0; d < 2; ++d) {
+        bf16x2 w[4];
+        dword_pairs<F>(c.w[2 * b + d], w);
+#pragma unroll
+        for (int m = 0; m < MT; ++m) {
+          const u32x4 xv = *reinterpret_cast<const u32x4*>(xs + m * per_row + (2 * b + d) * 256);
+#pragma unroll
+          for (int p = 0; p < 4; ++p) part[m] = __builtin_amdgcn_fdot2_f32_bf16(w[p], as_bf16x2(xv[p]), part[m], false);
+        }
+      }
+#pragma unroll
+      for (int m = 0; m < MT; ++m) acc[m] = __builtin_fmaf(part[m], scale, acc[m]);
+    }
+  } else {
+    constexpr int G = 4 * P / 4;  // groups of eight k in the chunk: BF16 1, INT8 / FP8 2
+#pragma unroll
+    for (int g = 0; g < G; ++g) {
+      bf16x2 w[4];
+      if constexpr (P == 1) {
+#pragma unroll
+        for (int d = 0; d < 4; ++d) dword_pairs<F>(c.w[d], w + d);
+      } else {
+        dword_pairs<F>(c.w[2 * g], w);
+        dword_pairs<F>(c.w[2 * g + 1], w + 2);
+      }
+#pragma unroll
+      for (int m = 0; m < MT; ++m) {
+        const u32x4 xv = *reinterpret_cast<const u32x4*>(xs + m * per_row + g * 256);
+#pragma unroll
+        for (int p = 0; p < 4; ++p) acc[m] = __builtin_amdgcn_fdot2_f32_bf16(w[p], as_bf16x2(xv[p]), acc[m], false);
+      }
+    }
+  }
+}
+
 // Streams a sequence of groups of R rows through a wavefront.
 //
-//   RowStreamer<F, MT, R, U> st(chunks, s_begin, s_end, per_row);
+//   RowStreamer<F, MT, R, U, XB> st(chunks, s_begin, s_end, per_row);      // per_row in words of the image XB names
 //   st.prefetch(rows_fn, first_group, group_stride, n_groups);   // weights do not depend on x: ask first
 //   ... stage x in LDS, __syncthreads() ...
 //   st.run(rows_fn, done_fn, first_group, group_stride, n_groups);
@@ -265,9 +431,10 @@ __device__ __forceinline__ void chunk_fma(const Chunk<F>& c, const float* xs, in
 // the LDS image its products read (one image for all rows in a GEMV; one per row where every row meets its own
 // activations); done_fn(group, acc) receives the lane sums acc[MT][R] of a finished group (the caller reduces
 // them across the wave). Steps [s_begin, s_end) of every row are taken, in batches of U.
-template <int F, int MT, int R, int U>
+// ONE: the stream is a single group whose steps fit one batch (s_end - s_begin <= U): one buffer, no loop.
+template <int F, int MT, int R, int U, bool XB = false, bool ONE = false>
 struct RowStreamer {
-  Chunk<F> buf_a[U][R], buf_b[U][R];
+  Chunk<F> buf_a[U][R], buf_b[ONE ? 1 : U][ONE ? 1 : R];
   int chunks, s_begin, s_end, per_row, batches, lane;
 
   __device__ __forceinline__ RowStreamer(int chunks_, int s_begin_, int s_end_, int per_row_)
@@ -301,13 +468,14 @@ struct RowStreamer {
     for (int u = 0; u < U; ++u) {
       const int s = s_begin + batch * U + u;
       if (s < s_end) {
-        const int slot = x_slot<F>(s, lane, 0);
+        const int slot = x_chunk_word<F, XB>(s, lane);
 #pragma unroll
         for (int r = 0; r < R; ++r) {
           float a[MT];
 #pragma unroll
           for (int m = 0; m < MT; ++m) a[m] = acc[m][r];
-          chunk_fma<F, MT>(buf[u][r], xs[r] + slot, per_row, a);
+          if constexpr (XB) chunk_dot2<F, MT>(buf[u][r], reinterpret_cast<const uint32_t*>(xs[r]) + slot, per_row, a);
+          else chunk_fma<F, MT>(buf[u][r], xs[r] + slot, per_row, a);
 #pragma unroll
           for (int m = 0; m < MT; ++m) acc[m][r] = a[m];
         }
@@ -319,8 +487,10 @@ struct RowStreamer {
   template <class RowsFn>
   __device__ __forceinline__ void prefetch(RowsFn& rows_fn, int first_group, int stride, int n_groups) {
     issue(buf_a, rows_fn, first_group, 0);
-    if (batches > 1) issue(buf_b, rows_fn, first_group, 1);
-    else if (n_groups > 1) issue(buf_b, rows_fn, first_group + stride, 0);
+    if constexpr (!ONE) {
+      if (batches > 1) issue(buf_b, rows_fn, first_group, 1);
+      else if (n_groups > 1) issue(buf_b, rows_fn, first_group + stride, 0);
+    }
   }
 
   // Groups first_group, first_group + stride, ... (n_groups of them); prefetch() has asked for the first two
@@ -332,6 +502,14 @@ struct RowStreamer {
     for (int m = 0; m < MT; ++m)
 #pragma unroll
       for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+    if constexpr (ONE) {
+      const uint8_t* rows[R];
+      const uint8_t* scales[R];
+      const float* xs[R];
+      rows_fn(first_group, rows, scales, xs);
+      consume(buf_a, xs, 0, acc);
+      done_fn(first_group, acc);
+    } else {
     int group = first_group, batch = 0, left = n_groups;
     bool first = true;  // the first half-iteration's next batch is already on its way
     // One half-iteration: ask for the batch after (group, batch) into `next`, multiply `cur`.
@@ -360,6 +538,7 @@ struct RowStreamer {
       half(buf_a, buf_b);
       if (left == 0) break;
       half(buf_b, buf_a);
+    }
     }
   }
 };

@@ -5,7 +5,8 @@
 // consecutive output columns n of one activation row m (D[i = 4 * (lane / 16) + r][j = lane % 16], i the
 // weight row, j the activation row): a 16-byte store per lane.
 //
-// Weights are read where they lie, 16 bytes per lane per load: lane (g = lane / 16, i = lane % 16) reads chunk
+// Weights are read as they lie, 16 bytes per lane per load, 256 contiguous bytes of a row per instruction, and
+// handed through LDS to the lanes of the matrix instruction: lane (g = lane / 16, i = lane % 16) works on chunk
 // 4 * t + g of row i at load step t, which is kElems consecutive k, i.e. kElems / 8 matrix instructions' worth.
 // The instruction sums over k in whatever order the operands present it, so instruction j of a load step simply
 // takes each lane's elements [8j, 8j + 8) on both sides: the activation fragment of lane (g, m) for that
@@ -90,32 +91,38 @@ __device__ __forceinline__ bf16x8 weight_fragment<LX_W_NVFP4>(const u32x4& w, ui
   return __builtin_bit_cast(bf16x8, p);
 }
 
-// Where a wavefront's activation fragments come from: rows of bf16 or f32 in global memory whose addresses and
-// strides are multiples of 16 bytes. XF32 says which; the caller resolves each lane's row pointers (one per
-// activation tile, clamped into the matrix: the columns of a clamped row are computed and never written).
-template <bool XF32>
+// Where a wavefront's activation fragments come from (XS): rows of bf16 (kXGlobalBf16) or f32 (kXGlobalF32) in
+// global memory whose addresses and strides are multiples of 16 bytes, or rows of bf16 staged in LDS (kXLds, the
+// rows a multiple of 16 bytes apart). The caller resolves each lane's row pointers (one per activation tile,
+// clamped into the matrix: the columns of a clamped row are computed and never written).
+constexpr int kXGlobalBf16 = 0, kXGlobalF32 = 1, kXLds = 2;
+
+template <int XS>
 struct XFrag {
-  u32x4 raw[XF32 ? 2 : 1];
+  u32x4 raw[XS == kXGlobalF32 ? 2 : 1];
 };
 
-// x[row, k .. k + 8) as loaded; k is clamped into the row (a fragment past K is zeroed when it is used).
-template <bool XF32>
-__device__ __forceinline__ void load_x_fragment(XFrag<XF32>& f, const void* row, int k, int K) {
-  const int kc = min(k, K - 8);
-  if constexpr (XF32) {
-    const u32x4* p = reinterpret_cast<const u32x4*>(static_cast<const float*>(row) + kc);
+// x[row, k .. k + 8) as loaded; in global memory k is clamped into the row (a fragment past K is zeroed when it
+// is used); an LDS image covers every k that is asked for.
+template <int XS>
+__device__ __forceinline__ void load_x_fragment(XFrag<XS>& f, const void* row, int k, int K) {
+  if constexpr (XS == kXGlobalF32) {
+    const u32x4* p = reinterpret_cast<const u32x4*>(static_cast<const float*>(row) + min(k, K - 8));
     f.raw[0] = p[0];
     f.raw[1] = p[1];
+  } else if constexpr (XS == kXGlobalBf16) {
+    f.raw[0] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(row) + min(k, K - 8));
   } else {
-    f.raw[0] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(row) + kc);
+    f.raw[0] = *reinterpret_cast<const u32x4*>(static_cast<const uint16_t*>(row) + k);
   }
 }
 
-// The fragment as the B operand: bf16 as it is, f32 rounded to bf16 (nearest even); zero past K.
-template <bool XF32>
-__device__ __forceinline__ bf16x8 x_operand(const XFrag<XF32>& f, int k, int K) {
+// The fragment as the B operand: bf16 as it is, f32 rounded to bf16 (nearest even); zero past K when MASK (an
+// activation image that is itself zero past K needs none).
+template <int XS, bool MASK>
+__device__ __forceinline__ bf16x8 x_operand(const XFrag<XS>& f, int k, int K) {
   u32x4 v;
-  if constexpr (XF32) {
+  if constexpr (XS == kXGlobalF32) {
     bf16x2 q[4] = {pack_bf16(__uint_as_float(f.raw[0].x), __uint_as_float(f.raw[0].y)),
                    pack_bf16(__uint_as_float(f.raw[0].z), __uint_as_float(f.raw[0].w)),
                    pack_bf16(__uint_as_float(f.raw[1].x), __uint_as_float(f.raw[1].y)),
@@ -124,70 +131,165 @@ __device__ __forceinline__ bf16x8 x_operand(const XFrag<XF32>& f, int k, int K) 
   } else {
     v = f.raw[0];
   }
-  if (k >= K) v = u32x4{0u, 0u, 0u, 0u};
+  if constexpr (MASK)
+    if (k >= K) v = u32x4{0u, 0u, 0u, 0u};
   return __builtin_bit_cast(bf16x8, v);
 }
 
-// Load steps asked for at once: bounded by the registers the activation fragments of a batch take
-// (steps x instructions per step x activation tiles x 4 or 8 registers), at most kLoadsInFlight / NT.
-template <int F, int NT, int MT, bool XF32>
+// Load steps whose activation fragments are held at once: from global memory, bounded by the registers they
+// take (steps x instructions per step x activation tiles x 4 or 8 registers), at most kLoadsInFlight / NT; from
+// LDS the steps of one staging group or fewer (the reads are short and sit right before their use).
+template <int F, int NT, int MT, int XS>
 constexpr int batch_steps() {
   constexpr int J = Fmt<F>::kElems / 8;
-  int u = 16 / (J * MT * (XF32 ? 2 : 1));
+  if (XS == kXLds) return J * MT <= 2 ? 4 : J * MT <= 4 ? 2 : 1;
+  int u = 16 / (J * MT * (XS == kXGlobalF32 ? 2 : 1));
   const int cap = kLoadsInFlight / NT;
   u = u > cap ? cap : u;
-  return u < 1 ? 1 : u;
+  return u >= 8 ? 8 : u >= 4 ? 4 : u >= 2 ? 2 : 1;  // a power of two: it divides the weight batch
 }
 
+// Sixteen consecutive weight rows starting at `data` (their scale rows at `scale`), of which the first `valid`
+// exist: a row past them stands for the last valid one (its outputs are computed and never written).
+struct TileRows {
+  const uint8_t* data;
+  const uint8_t* scale;
+  int valid;
+};
+
+// A wavefront's private LDS: the staging image of one tile's 4 load steps (16 rows x 16 chunks, the rows 16
+// bytes apart in the banks so that both the row-wise writes and the fragment reads are conflict-free), reused
+// afterwards for the wavefront's partial sums.
+constexpr int kStagePitch = 16 * 16 + 16;
+constexpr int kStageBytes = kTileRows * kStagePitch;
+
+template <int NT, int MT>
+constexpr int wave_region_bytes() {
+  return NT * MT * kWave * 16 > kStageBytes ? NT * MT * kWave * 16 : kStageBytes;
+}
+
+inline size_t tile_lds_bytes(int S, int NT, int MT) {
+  const size_t partial = static_cast<size_t>(NT) * MT * kWave * 16;
+  return S * (partial > kStageBytes ? partial : static_cast<size_t>(kStageBytes));
+}
+
+// Orders this wavefront's LDS accesses as written (the hardware runs a wavefront's LDS instructions in order;
+// this keeps the compiler from moving one lane's read above another lane's write).
+__device__ __forceinline__ void wave_lds_order() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+
+// The weights of one batch (kLoadsInFlight / NT load steps of NT tiles) as they arrive from memory.
+template <int F, int NT>
+struct WeightBatch {
+  static constexpr int WU = kLoadsInFlight / NT;
+  static_assert(WU % 4 == 0, "weight steps are staged four at a time");
+  u32x4 raw[WU / 4][NT][4];
+  uint32_t sc[WU][NT];
+};
+
 // acc[t][mt] += tile t's rows times activation tile mt over load steps [t_begin, t_end).
-// rows[t] / scales[t] point at this lane's weight row of tile t (row i = lane % 16 of the tile, clamped into the
-// matrix by the caller); xrow[mt] at this lane's activation row of tile mt. `chunks` is the number of 16-byte
-// chunks in a weight row. Every load of a batch, weights and activations, is asked for before the first use.
-template <int F, int NT, int MT, bool XF32>
-__device__ __forceinline__ void mfma_slice(const uint8_t* const (&rows)[NT], const uint8_t* const (&scales)[NT], int chunks,
-                                           int t_begin, int t_end, const void* const (&xrow)[MT], int K, f32x4 (&acc)[NT][MT]) {
+// xrow[mt] points at this lane's activation row of tile mt. `chunks` is the number of 16-byte chunks in a weight
+// row. The weights of a batch are asked for at once, in the order they lie in memory: one load instruction reads
+// 256 contiguous bytes of each of four rows (lane -> row 4q + lane / 16, chunk lane % 16 of a 4-step group).
+// They pass through `stage` (this wavefront's kStageBytes of LDS) to reach the lanes that feed them to the
+// matrix instruction: lane (g, i) takes chunk 4s + g of row i for step s of the group.
+// between() runs once, after the first batch's loads are on their way and before anything is consumed: the
+// place to stage activations into LDS (it may hold a workgroup barrier: every wavefront calls it).
+template <int F, int NT, int MT, int XS, class Between>
+__device__ __forceinline__ void mfma_slice(const TileRows (&tiles)[NT], int64_t row_bytes, int64_t scale_row_bytes, int chunks,
+                                           int t_begin, int t_end, const void* const (&xrow)[MT], int K, f32x4 (&acc)[NT][MT],
+                                           uint8_t* stage, Between&& between) {
   constexpr int E = Fmt<F>::kElems;
   constexpr int J = E / 8;  // matrix instructions per load step
-  constexpr int U = batch_steps<F, NT, MT, XF32>();
+  constexpr int WU = WeightBatch<F, NT>::WU;
+  constexpr int G = WU / 4;
+  constexpr int U = batch_steps<F, NT, MT, XS>();
   const int lane = threadIdx.x & (kWave - 1);
-  const int g = lane >> 4;
-  for (int tb = t_begin; tb < t_end; tb += U) {
-    u32x4 wv[U][NT];
-    uint32_t sc[U][NT];
-    XFrag<XF32> xf[U][J][MT];
+  const int g = lane >> 4, i = lane & 15;
+  const uint8_t* own_scale[NT];
+  const uint8_t* stage_row[NT][4];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      // A step past the slice, or a chunk past the row's end, re-reads a valid chunk of the same row; its
-      // activation fragment is zero (past K) or the step is skipped.
-      const int t = min(tb + u, t_end - 1);
-      const int c = min(4 * t + g, chunks - 1);
+  for (int n = 0; n < NT; ++n) {
+    own_scale[n] = tiles[n].scale + min(i, tiles[n].valid - 1) * scale_row_bytes;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) stage_row[n][q] = tiles[n].data + min(4 * q + g, tiles[n].valid - 1) * row_bytes;
+  }
+  u32x4* const put = reinterpret_cast<u32x4*>(stage + g * kStagePitch + i * 16);              // + q * 4 rows
+  const u32x4* const get = reinterpret_cast<const u32x4*>(stage + i * kStagePitch + g * 16);  // + s * 4 chunks
+  WeightBatch<F, NT> wb;
+  auto issue = [&](int tb) {
+#pragma unroll
+    for (int grp = 0; grp < G; ++grp) {
+      // A chunk past the row's end re-reads the row's last chunk: the steps it lands in are past K or skipped.
+      const int c = min(4 * (tb + 4 * grp) + i, chunks - 1);
+#pragma unroll
+      for (int n = 0; n < NT; ++n)
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+          wb.raw[grp][n][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(stage_row[n][q]) + c);
+    }
+#pragma unroll
+    for (int u = 0; u < WU; ++u)
 #pragma unroll
       for (int n = 0; n < NT; ++n) {
-        wv[u][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(rows[n]) + c);
-        sc[u][n] = 0;
-        if constexpr (F == LX_W_NVFP4) sc[u][n] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(scales[n]) + c);
+        wb.sc[u][n] = 0;
+        if constexpr (F == LX_W_NVFP4)
+          wb.sc[u][n] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale[n]) + min(4 * (tb + u) + g, chunks - 1));
       }
-    }
+  };
+  if (t_begin < t_end) issue(t_begin);
+  between();
+  // Steps past the slice's end (a last, partial batch) run on re-read weights against zero activations. An LDS
+  // image is zero from K to the end of the row's last batch, and with it every slice but the row's last is
+  // whole batches (the caller sees to both), so nothing is masked.
+  constexpr bool MASK = XS != kXLds;
+  const int k_end = min(K, 4 * t_end * E);
+  for (int tb = t_begin; tb < t_end; tb += WU) {
+    if (tb != t_begin) issue(tb);
+    XFrag<XS> xf[U][J][MT];
+    auto load_x = [&](int ub) {
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int k0 = (4 * min(tb + u, t_end - 1) + g) * E;
+      for (int u = 0; u < U; ++u) {
+        const int k0 = (4 * (tb + ub + u) + g) * E;
 #pragma unroll
-      for (int j = 0; j < J; ++j)
+        for (int j = 0; j < J; ++j)
 #pragma unroll
-        for (int mt = 0; mt < MT; ++mt) load_x_fragment<XF32>(xf[u][j][mt], xrow[mt], k0 + 8 * j, K);
-    }
+          for (int mt = 0; mt < MT; ++mt) load_x_fragment<XS>(xf[u][j][mt], xrow[mt], k0 + 8 * j, K);
+      }
+    };
+    if constexpr (XS != kXLds) load_x(0);  // in flight together with the weights
+    // Four steps at a time: through the staging image into fragment order, then into the matrix instructions.
+    u32x4 wv[WU][NT];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (tb + u < t_end) {
-        const int k0 = (4 * (tb + u) + g) * E;
+    for (int ub = 0; ub < WU; ub += U) {
+      if (XS != kXLds && ub > 0) load_x(ub);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if ((ub + u) % 4 == 0) {
+          const int grp = (ub + u) / 4;
+#pragma unroll
+          for (int n = 0; n < NT; ++n) {
+#pragma unroll
+            for (int q = 0; q < 4; ++q) put[q * (4 * kStagePitch / 16)] = wb.raw[grp][n][q];
+            wave_lds_order();
+#pragma unroll
+            for (int sstep = 0; sstep < 4; ++sstep) wv[4 * grp + sstep][n] = get[sstep * 4];
+            wave_lds_order();
+          }
+        }
+        if (XS == kXLds && u == 0) load_x(ub);
+        const int k0 = (4 * (tb + ub + u) + g) * E;
 #pragma unroll
         for (int j = 0; j < J; ++j) {
 #pragma unroll
           for (int n = 0; n < NT; ++n) {
-            const bf16x8 wf = weight_fragment<F>(wv[u][n], sc[u][n], j);
+            const bf16x8 wf = weight_fragment<F>(wv[ub + u][n], wb.sc[ub + u][n], j);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
-              acc[n][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, x_operand<XF32>(xf[u][j][mt], k0 + 8 * j, K), acc[n][mt], 0, 0, 0);
+              acc[n][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, x_operand<XS, MASK>(xf[u][j][mt], k0 + 8 * j, k_end), acc[n][mt], 0, 0, 0);
           }
         }
       }
@@ -195,23 +297,26 @@ __device__ __forceinline__ void mfma_slice(const uint8_t* const (&rows)[NT], con
   }
 }
 
-// The whole workgroup: wavefront w of S takes load steps [w * per, (w + 1) * per), the partial tiles are added
-// in ascending w through `lds` (S * NT * MT * 64 f32x4), and epi(mt, q, sums) is called once for every
-// (activation tile mt, lane slot q) with the NT finished sums: sums[t][r] belongs to weight row 4 * (q / 16) + r
-// of tile t and activation row mt * 16 + q % 16.
-template <int F, int NT, int MT, bool XF32, class Epi>
-__device__ __forceinline__ void mfma_tile(const uint8_t* const (&rows)[NT], const uint8_t* const (&scales)[NT], int chunks,
-                                          int steps, int steps_per_wave, const void* const (&xrow)[MT], int K, f32x4* lds,
-                                          Epi&& epi) {
-  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int S = blockDim.x / kWave;
+// One tile's S wavefronts (a workgroup may hold several tiles' worth: `slice` is this wavefront's index among
+// its tile's S, `lds` the tile's regions): wavefront w takes load steps [w * per, (w + 1) * per), the partial
+// tiles are added in ascending w through `lds` (tile_lds_bytes(S, NT, MT) bytes, a region per wavefront), and
+// epi(mt, q, sums) is called once for every (activation tile mt, lane slot q) with the NT finished sums:
+// sums[t][r] belongs to weight row 4 * (q / 16) + r of tile t and activation row mt * 16 + q % 16.
+// Every wavefront of the workgroup must make the call: it holds workgroup barriers.
+template <int F, int NT, int MT, int XS, class Between, class Epi>
+__device__ __forceinline__ void mfma_tile(const TileRows (&tiles)[NT], int64_t row_bytes, int64_t scale_row_bytes, int chunks,
+                                          int steps, int steps_per_wave, const void* const (&xrow)[MT], int K, f32x4* lds, int S,
+                                          int slice, Between&& between, Epi&& epi) {
+  constexpr int kRegion = wave_region_bytes<NT, MT>();
+  const int lane = threadIdx.x & (kWave - 1);
+  uint8_t* const base = reinterpret_cast<uint8_t*>(lds);
   f32x4 acc[NT][MT];
 #pragma unroll
   for (int n = 0; n < NT; ++n)
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[n][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int t_begin = min(steps, wave * steps_per_wave), t_end = min(steps, t_begin + steps_per_wave);
-  mfma_slice<F, NT, MT, XF32>(rows, scales, chunks, t_begin, t_end, xrow, K, acc);
+  const int t_begin = min(steps, slice * steps_per_wave), t_end = min(steps, t_begin + steps_per_wave);
+  mfma_slice<F, NT, MT, XS>(tiles, row_bytes, scale_row_bytes, chunks, t_begin, t_end, xrow, K, acc, base + slice * kRegion, between);
   if (S == 1) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -222,18 +327,20 @@ __device__ __forceinline__ void mfma_tile(const uint8_t* const (&rows)[NT], cons
     }
     return;
   }
+  wave_lds_order();
+  f32x4* const mine = reinterpret_cast<f32x4*>(base + slice * kRegion);
 #pragma unroll
   for (int n = 0; n < NT; ++n)
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) lds[((wave * NT + n) * MT + mt) * kWave + lane] = acc[n][mt];
+    for (int mt = 0; mt < MT; ++mt) mine[(n * MT + mt) * kWave + lane] = acc[n][mt];
   __syncthreads();
-  for (int item = threadIdx.x; item < MT * kWave; item += blockDim.x) {
+  for (int item = slice * kWave + lane; item < MT * kWave; item += S * kWave) {
     const int mt = item / kWave, q = item % kWave;
     f32x4 sums[NT];
 #pragma unroll
     for (int n = 0; n < NT; ++n) {
-      f32x4 s = lds[((0 * NT + n) * MT + mt) * kWave + q];
-      for (int w = 1; w < S; ++w) s += lds[((w * NT + n) * MT + mt) * kWave + q];
+      f32x4 s = reinterpret_cast<const f32x4*>(base)[(n * MT + mt) * kWave + q];
+      for (int w = 1; w < S; ++w) s += reinterpret_cast<const f32x4*>(base + w * kRegion)[(n * MT + mt) * kWave + q];
       sums[n] = s;
     }
     epi(mt, q, sums);
