@@ -187,11 +187,11 @@ __device__ __forceinline__ void group_pairs(const int32_t* ids, int P, int slot,
 // sorted positions first..: the pair (gate row i, up row I + i) is the wavefront's two streamed rows, all of
 // their loads in flight before the activations are waited for. MT only sets how many activation rows share
 // the pass; a row's arithmetic is the same for any MT. The whole workgroup calls it (it stages x).
-template <int F, int U, int MT>
+template <int F, int U, int MT, bool ONE>
 __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, int e, int first, int cnt, const int* s_order,
                                              const int* s_rows) {
   const int steps = steps_for<F>(a.L);
-  const int per_row = x_row_floats<F>(steps);
+  const int per_row = x_row_words<F, true>(steps);  // the packed bf16 image: the latent rows are bf16
   const int64_t rb = row_bytes<F>(a.L);
   const int chunks = static_cast<int>(rb / 16);
   const int64_t scale_row = F == LX_W_NVFP4 ? a.L / 16 : 0;
@@ -226,7 +226,8 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
       }
     }
   };
-  RowStreamer<F, MT, 2, U> st(chunks, 0, steps, per_row);
+  RowStreamer<F, MT, 2, U, true, ONE> st(chunks, 0, steps, per_row);
+  uint32_t* const image = reinterpret_cast<uint32_t*>(lds);
   if constexpr (MT == 1) {
     // Ask for x, then for the weights, and only then wait for x: loads return in order.
     const int token = s_rows ? s_rows[0] : first / a.top_k;
@@ -234,11 +235,11 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
     XRegs xr;
     stage_x_load<F>(xr, xrow, LX_BF16, a.L, a.L, steps);
     st.prefetch(rows_fn, i, 0, 1);
-    if (xr.ready) stage_x_store<F>(xr, lds, LX_BF16, steps);
-    else stage_x<F, 1>(lds, xrow, LX_BF16, a.L, nullptr, 1, a.L, steps);
+    if (xr.ready) stage_x_store_pairs<F>(xr, image, steps);
+    else stage_x_pairs<F, 1>(image, xrow, a.L, nullptr, 1, a.L, steps);
   } else {
     st.prefetch(rows_fn, i, 0, 1);
-    stage_x<F, MT>(lds, a.latent, LX_BF16, a.L, s_rows, cnt, a.L, steps);
+    stage_x_pairs<F, MT>(image, a.latent, a.L, s_rows, cnt, a.L, steps);
   }
   __syncthreads();
   st.run(rows_fn, done_fn, i, 0, 1);
@@ -246,7 +247,8 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
 
 // grid = (I / wavefronts per workgroup, group slots); mt_cap (a power of two, the LDS image's rows) bounds a
 // pass's pairs. One token: every slot is its own group and nothing is sorted.
-template <int F, int U>
+// ONE: a row's steps fit one batch of U.
+template <int F, int U, bool ONE>
 __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeArgs a, int mt_cap) {
   extern __shared__ __align__(16) float lds[];
   __shared__ int s_ids[kMaxPairs], s_order[kMaxPairs], s_info[4], s_rows[8];
@@ -254,7 +256,7 @@ __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeAr
   if (a.T == 1) {
     if (static_cast<int>(blockIdx.y) >= P) return;
     const int e = __builtin_amdgcn_readfirstlane(a.ids[blockIdx.y]);
-    gate_up_rows<F, U, 1>(a, lds, e, blockIdx.y, 1, nullptr, nullptr);
+    gate_up_rows<F, U, 1, ONE>(a, lds, e, blockIdx.y, 1, nullptr, nullptr);
     return;
   }
   group_pairs(a.ids, P, blockIdx.y, s_ids, s_order, s_info);
@@ -267,10 +269,10 @@ __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeAr
     __syncthreads();
     if (threadIdx.x < 8) s_rows[threadIdx.x] = static_cast<int>(threadIdx.x) < cnt ? s_order[first + threadIdx.x] / a.top_k : 0;
     __syncthreads();
-    if (cnt <= 1) gate_up_rows<F, U, 1>(a, lds, e, first, cnt, s_order, s_rows);
-    else if (cnt <= 2) gate_up_rows<F, U, 2>(a, lds, e, first, cnt, s_order, s_rows);
-    else if (cnt <= 4) gate_up_rows<F, U, 4>(a, lds, e, first, cnt, s_order, s_rows);
-    else gate_up_rows<F, U, 8>(a, lds, e, first, cnt, s_order, s_rows);
+    if (cnt <= 1) gate_up_rows<F, U, 1, ONE>(a, lds, e, first, cnt, s_order, s_rows);
+    else if (cnt <= 2) gate_up_rows<F, U, 2, ONE>(a, lds, e, first, cnt, s_order, s_rows);
+    else if (cnt <= 4) gate_up_rows<F, U, 4, ONE>(a, lds, e, first, cnt, s_order, s_rows);
+    else gate_up_rows<F, U, 8, ONE>(a, lds, e, first, cnt, s_order, s_rows);
   }
 }
 
@@ -284,7 +286,7 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
   constexpr int R = 4;
   const int t = blockIdx.y;
   const int steps = steps_for<F>(a.I);
-  const int per_row = x_row_floats<F>(steps);
+  const int per_row = x_row_words<F, true>(steps);  // the packed bf16 image: the intermediate rows are bf16
   const int64_t rb = row_bytes<F>(a.I);
   const int chunks = static_cast<int>(rb / 16);
   const int64_t scale_row = F == LX_W_NVFP4 ? a.I / 16 : 0;
@@ -320,11 +322,11 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
     }
   };
   const int n_groups = (top_k + R - 1) / R;
-  RowStreamer<F, 1, R, U> st(chunks, 0, steps, per_row);
+  RowStreamer<F, 1, R, U, true> st(chunks, 0, steps, per_row);
   st.prefetch(rows_fn, 0, 1, n_groups);
   if (threadIdx.x < 8) s_rows[threadIdx.x] = t * top_k + min(static_cast<int>(threadIdx.x), top_k - 1);
   __syncthreads();
-  stage_x<F, 8>(lds, a.inter, LX_BF16, a.I, s_rows, top_k, a.I, steps);
+  stage_x_pairs<F, 8>(reinterpret_cast<uint32_t*>(lds), a.inter, a.I, s_rows, top_k, a.I, steps);
   __syncthreads();
   st.run(rows_fn, done_fn, 0, 1, n_groups);
   if (lane == 0 && l < a.L) a.out[static_cast<int64_t>(t) * a.L + l] = o;
@@ -376,7 +378,7 @@ bool streamable(const Stack& s, int64_t K, int max_rows) {
   const int steps = steps_for<F>(K);
   return rb % 16 == 0 && reinterpret_cast<uintptr_t>(s.data) % 16 == 0 &&
          (F != LX_W_NVFP4 || reinterpret_cast<uintptr_t>(s.scale) % 2 == 0) &&
-         static_cast<int64_t>(max_rows) * x_row_floats<F>(steps) * 4 <= 128 * 1024;
+         static_cast<int64_t>(max_rows) * x_row_words<F, true>(steps) * 4 <= 128 * 1024;
 }
 
 template <class Kernel>
@@ -392,11 +394,13 @@ int launch_gate_up_u(const DecodeArgs& a, hipStream_t s) {
   const int P = a.T * a.top_k;
   // With distinct experts per token a group has at most T pairs; the LDS image holds that many rows.
   const int mt_cap = a.T <= 1 ? 1 : a.T <= 2 ? 2 : a.T <= 4 ? 4 : 8;
-  const size_t lds = sizeof(float) * mt_cap * x_row_floats<F>(steps_for<F>(a.L));
-  auto kernel = decode_gate_up_kernel<F, U>;
-  allow_big_lds(kernel, lds);
-  hipLaunchKernelGGL(kernel, dim3((a.I + kWaves - 1) / kWaves, P), dim3(kThreads), lds, s, a, mt_cap);
-  return status_of(hipGetLastError());
+  const size_t lds = sizeof(float) * mt_cap * x_row_words<F, true>(steps_for<F>(a.L));
+  auto launch = [&](auto kernel) {
+    allow_big_lds(kernel, lds);
+    hipLaunchKernelGGL(kernel, dim3((a.I + kWaves - 1) / kWaves, P), dim3(kThreads), lds, s, a, mt_cap);
+    return status_of(hipGetLastError());
+  };
+  return steps_for<F>(a.L) <= U ? launch(decode_gate_up_kernel<F, U, true>) : launch(decode_gate_up_kernel<F, U, false>);
 }
 
 template <int F>
@@ -410,7 +414,7 @@ int launch_gate_up(const DecodeArgs& a, hipStream_t s) {
 
 template <int F, int U>
 int launch_down_u(const DecodeArgs& a, hipStream_t s) {
-  const size_t lds = sizeof(float) * 8 * x_row_floats<F>(steps_for<F>(a.I));
+  const size_t lds = sizeof(float) * 8 * x_row_words<F, true>(steps_for<F>(a.I));
   auto kernel = decode_down_kernel<F, U>;
   allow_big_lds(kernel, lds);
   hipLaunchKernelGGL(kernel, dim3((a.L + kWaves - 1) / kWaves, a.T), dim3(kThreads), lds, s, a);
