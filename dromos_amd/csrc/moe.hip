@@ -282,7 +282,6 @@ __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeAr
 template <int F, int U>
 __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs a) {
   extern __shared__ __align__(16) float lds[];
-  __shared__ int s_rows[8];
   constexpr int R = 4;
   const int t = blockIdx.y;
   const int steps = steps_for<F>(a.I);
@@ -323,10 +322,13 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
   };
   const int n_groups = (top_k + R - 1) / R;
   RowStreamer<F, 1, R, U, true> st(chunks, 0, steps, per_row);
+  // Ask for the intermediate rows, then for the weights, and only then wait for the rows: loads return in order.
+  const uint16_t* const rows_of_t = a.inter + static_cast<int64_t>(t) * top_k * a.I;  // the token's top_k rows, in slot order
+  XRowRegs xr;
+  stage_rows_load<F>(xr, rows_of_t, a.I, nullptr, top_k, a.I, steps);
   st.prefetch(rows_fn, 0, 1, n_groups);
-  if (threadIdx.x < 8) s_rows[threadIdx.x] = t * top_k + min(static_cast<int>(threadIdx.x), top_k - 1);
-  __syncthreads();
-  stage_x_pairs<F, 8>(reinterpret_cast<uint32_t*>(lds), a.inter, a.I, s_rows, top_k, a.I, steps);
+  if (xr.ready) stage_rows_store<F, 8>(xr, reinterpret_cast<uint32_t*>(lds), top_k, a.I, steps);
+  else stage_x_pairs<F, 8>(reinterpret_cast<uint32_t*>(lds), rows_of_t, a.I, nullptr, top_k, a.I, steps);
   __syncthreads();
   st.run(rows_fn, done_fn, 0, 1, n_groups);
   if (lane == 0 && l < a.L) a.out[static_cast<int64_t>(t) * a.L + l] = o;

@@ -264,6 +264,56 @@ __device__ __forceinline__ void stage_x_store_pairs(const XRegs& r, uint32_t* xs
   }
 }
 
+// Two-phase staging of up to MT bf16 rows (optionally gathered through row_of[m]) into the packed image: slots
+// (row m, pass j) in row-major order, a thread's piece of a slot being vector j * blockDim + thread of row m. Usable
+// when the rows can be read 16 bytes at a time and there are at most kSlots slots; otherwise `ready` is false and
+// the caller falls back to stage_x_pairs.
+struct XRowRegs {
+  static constexpr int kSlots = 4;
+  u32x4 v[kSlots];
+  int iters;  // passes per row
+  bool ready;
+};
+
+template <int F>
+__device__ __forceinline__ void stage_rows_load(XRowRegs& r, const uint16_t* x, int64_t ld_x, const int* row_of, int M, int64_t K,
+                                                int steps) {
+  const int n_vec = x_row_words<F, true>(steps) >> 2, k_vec = static_cast<int>(K) >> 3;
+  r.iters = (n_vec + blockDim.x - 1) / blockDim.x;
+  r.ready = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && ((ld_x * 2) & 15) == 0 && (K & 7) == 0 && M * r.iters <= XRowRegs::kSlots;
+  if (!r.ready) return;
+  int m = 0, j = 0;
+#pragma unroll
+  for (int u = 0; u < XRowRegs::kSlots; ++u) {
+    // Clamped addresses (no predicated loads); what lies past K or M is replaced by zeros when it is stored.
+    const int v = min(static_cast<int>(threadIdx.x) + j * static_cast<int>(blockDim.x), k_vec - 1);
+    const int mc = min(m, M - 1);
+    r.v[u] = *(reinterpret_cast<const u32x4*>(x + static_cast<int64_t>(row_of ? row_of[mc] : mc) * ld_x) + v);
+    if (++j == r.iters) j = 0, ++m;
+  }
+}
+
+template <int F, int MT>
+__device__ __forceinline__ void stage_rows_store(const XRowRegs& r, uint32_t* xs, int M, int64_t K, int steps) {
+  constexpr int E = Fmt<F>::kElems;
+  const int per_row = x_row_words<F, true>(steps);
+  const int n_vec = per_row >> 2, k_vec = static_cast<int>(K) >> 3;
+  int m = 0, j = 0;
+#pragma unroll
+  for (int u = 0; u < XRowRegs::kSlots; ++u) {
+    const int v = threadIdx.x + j * blockDim.x;
+    if (m < M && v < n_vec) {
+      const int k = v << 3, st = k / (kWave * E), within = k % (kWave * E);
+      *reinterpret_cast<u32x4*>(xs + m * per_row + x_pair_slot<F>(st, within / E, within % E)) =
+          v < k_vec ? r.v[u] : u32x4{0u, 0u, 0u, 0u};
+    }
+    if (++j == r.iters) j = 0, ++m;
+  }
+  // Rows M .. MT - 1 are zero.
+  for (int i = threadIdx.x; i < (MT - M) * n_vec; i += blockDim.x)
+    *reinterpret_cast<u32x4*>(xs + M * per_row + i * 4) = u32x4{0u, 0u, 0u, 0u};
+}
+
 // What a lane holds of one weight row for one step: its 16 bytes, and for NVFP4 the two block scales.
 template <int F>
 struct Chunk {
