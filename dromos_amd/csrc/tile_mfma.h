@@ -143,7 +143,7 @@ template <int F, int NT, int MT, int XS>
 constexpr int batch_steps() {
   constexpr int J = Fmt<F>::kElems / 8;
   if (XS == kXLds) return J * MT <= 2 ? 4 : J * MT <= 4 ? 2 : 1;
-  int u = 16 / (J * MT * (XS == kXGlobalF32 ? 2 : 1));
+  int u = 8 / (J * MT * (XS == kXGlobalF32 ? 2 : 1));
   const int cap = kLoadsInFlight / NT;
   u = u > cap ? cap : u;
   return u >= 8 ? 8 : u >= 4 ? 4 : u >= 2 ? 2 : 1;  // a power of two: it divides the weight batch
@@ -190,37 +190,41 @@ struct WeightBatch {
   uint32_t sc[WU][NT];
 };
 
-// acc[t][mt] += tile t's rows times activation tile mt over load steps [t_begin, t_end).
-// xrow[mt] points at this lane's activation row of tile mt. `chunks` is the number of 16-byte chunks in a weight
-// row. The weights of a batch are asked for at once, in the order they lie in memory: one load instruction reads
-// 256 contiguous bytes of each of four rows (lane -> row 4q + lane / 16, chunk lane % 16 of a 4-step group).
-// They pass through `stage` (this wavefront's kStageBytes of LDS) to reach the lanes that feed them to the
-// matrix instruction: lane (g, i) takes chunk 4s + g of row i for step s of the group.
-// between() runs once, after the first batch's loads are on their way and before anything is consumed: the
-// place to stage activations into LDS (it may hold a workgroup barrier: every wavefront calls it).
-template <int F, int NT, int MT, int XS, class Between>
-__device__ __forceinline__ void mfma_slice(const TileRows (&tiles)[NT], int64_t row_bytes, int64_t scale_row_bytes, int chunks,
-                                           int t_begin, int t_end, const void* const (&xrow)[MT], int K, f32x4 (&acc)[NT][MT],
-                                           uint8_t* stage, Between&& between) {
-  constexpr int E = Fmt<F>::kElems;
-  constexpr int J = E / 8;  // matrix instructions per load step
-  constexpr int WU = WeightBatch<F, NT>::WU;
-  constexpr int G = WU / 4;
-  constexpr int U = batch_steps<F, NT, MT, XS>();
-  const int lane = threadIdx.x & (kWave - 1);
-  const int g = lane >> 4, i = lane & 15;
+// A wavefront's view of NT tiles of weights: where its loads come from and how they reach fragment order.
+// The weights of a batch are asked for at once, in the order they lie in memory: one load instruction reads 256
+// contiguous bytes of each of four rows (lane -> row 4q + lane / 16, chunk lane % 16 of a 4-step group). They pass
+// through `stage` (this wavefront's kStageBytes of LDS) to reach the lanes that feed them to the matrix
+// instruction: lane (g, i) takes chunk 4s + g of row i for step s of the group.
+template <int F, int NT>
+struct TileStream {
+  static constexpr int E = Fmt<F>::kElems;
+  static constexpr int J = E / 8;  // matrix instructions per load step
+  static constexpr int WU = WeightBatch<F, NT>::WU;
+  static constexpr int G = WU / 4;
   const uint8_t* own_scale[NT];
   const uint8_t* stage_row[NT][4];
+  u32x4* put;        // + q * 4 rows
+  const u32x4* get;  // + s * 4 chunks
+  int chunks, g, i;
+
+  __device__ __forceinline__ TileStream(const TileRows (&tiles)[NT], int64_t row_bytes, int64_t scale_row_bytes, int chunks_,
+                                        uint8_t* stage)
+      : chunks(chunks_) {
+    const int lane = threadIdx.x & (kWave - 1);
+    g = lane >> 4;
+    i = lane & 15;
 #pragma unroll
-  for (int n = 0; n < NT; ++n) {
-    own_scale[n] = tiles[n].scale + min(i, tiles[n].valid - 1) * scale_row_bytes;
+    for (int n = 0; n < NT; ++n) {
+      own_scale[n] = tiles[n].scale + min(i, tiles[n].valid - 1) * scale_row_bytes;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) stage_row[n][q] = tiles[n].data + min(4 * q + g, tiles[n].valid - 1) * row_bytes;
+      for (int q = 0; q < 4; ++q) stage_row[n][q] = tiles[n].data + min(4 * q + g, tiles[n].valid - 1) * row_bytes;
+    }
+    put = reinterpret_cast<u32x4*>(stage + g * kStagePitch + i * 16);
+    get = reinterpret_cast<const u32x4*>(stage + i * kStagePitch + g * 16);
   }
-  u32x4* const put = reinterpret_cast<u32x4*>(stage + g * kStagePitch + i * 16);              // + q * 4 rows
-  const u32x4* const get = reinterpret_cast<const u32x4*>(stage + i * kStagePitch + g * 16);  // + s * 4 chunks
-  WeightBatch<F, NT> wb;
-  auto issue = [&](int tb) {
+
+  // Asks for the batch of load steps [tb, tb + WU).
+  __device__ __forceinline__ void issue(WeightBatch<F, NT>& wb, int tb) const {
 #pragma unroll
     for (int grp = 0; grp < G; ++grp) {
       // A chunk past the row's end re-reads the row's last chunk: the steps it lands in are past K or skipped.
@@ -239,16 +243,15 @@ __device__ __forceinline__ void mfma_slice(const TileRows (&tiles)[NT], int64_t 
         if constexpr (F == LX_W_NVFP4)
           wb.sc[u][n] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale[n]) + min(4 * (tb + u) + g, chunks - 1));
       }
-  };
-  if (t_begin < t_end) issue(t_begin);
-  between();
-  // Steps past the slice's end (a last, partial batch) run on re-read weights against zero activations. An LDS
-  // image is zero from K to the end of the row's last batch, and with it every slice but the row's last is
-  // whole batches (the caller sees to both), so nothing is masked.
-  constexpr bool MASK = XS != kXLds;
-  const int k_end = min(K, 4 * t_end * E);
-  for (int tb = t_begin; tb < t_end; tb += WU) {
-    if (tb != t_begin) issue(tb);
+  }
+
+  // acc[t][mt] += the batch at tb times activation tile mt; steps from t_end on count for nothing (k_end = the
+  // first k that does not count: fragments from there on are zero, by mask or by the image's own zeros).
+  template <int MT, int XS>
+  __device__ __forceinline__ void consume(const WeightBatch<F, NT>& wb, int tb, const void* const (&xrow)[MT], int K, int k_end,
+                                          f32x4 (&acc)[NT][MT]) const {
+    constexpr int U = batch_steps<F, NT, MT, XS>();
+    constexpr bool MASK = XS != kXLds;
     XFrag<XS> xf[U][J][MT];
     auto load_x = [&](int ub) {
 #pragma unroll
@@ -294,6 +297,28 @@ __device__ __forceinline__ void mfma_slice(const TileRows (&tiles)[NT], int64_t 
         }
       }
     }
+  }
+};
+
+// acc[t][mt] += tile t's rows times activation tile mt over load steps [t_begin, t_end).
+// xrow[mt] points at this lane's activation row of tile mt. `chunks` is the number of 16-byte chunks in a weight
+// row. between() runs once, after the first batch's loads are on their way and before anything is consumed: the
+// place to stage activations into LDS (it may hold a workgroup barrier: every wavefront calls it).
+// Steps past the slice's end (a last, partial batch) run on re-read weights against zero activations. An LDS
+// image is zero from K to the end of the row's last batch, and with it every slice but the row's last is whole
+// batches (the caller sees to both), so nothing is masked.
+template <int F, int NT, int MT, int XS, class Between>
+__device__ __forceinline__ void mfma_slice(const TileRows (&tiles)[NT], int64_t row_bytes, int64_t scale_row_bytes, int chunks,
+                                           int t_begin, int t_end, const void* const (&xrow)[MT], int K, f32x4 (&acc)[NT][MT],
+                                           uint8_t* stage, Between&& between) {
+  const TileStream<F, NT> ts(tiles, row_bytes, scale_row_bytes, chunks, stage);
+  WeightBatch<F, NT> wb;
+  if (t_begin < t_end) ts.issue(wb, t_begin);
+  between();
+  const int k_end = min(K, 4 * t_end * Fmt<F>::kElems);
+  for (int tb = t_begin; tb < t_end; tb += TileStream<F, NT>::WU) {
+    if (tb != t_begin) ts.issue(wb, tb);
+    ts.template consume<MT, XS>(wb, tb, xrow, K, k_end, acc);
   }
 }
 
