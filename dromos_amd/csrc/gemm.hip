@@ -399,7 +399,6 @@ int launch_format(GemmArgs a, const char* x0, char* y0, int M, int x_esize, int 
   a.chunks = static_cast<int>(rb / 16);
   a.steps = load_steps_for<F>(a.K);
   int S = split_for<F>(a.K, 1);
-  if (const char* e = getenv("DRO_SKINNY_SPLIT")) S = atoi(e);
   // Slices are whole weight batches (the row's last one may be cut short by the row's end).
   a.steps_per_wave = ((a.steps + S - 1) / S + kLoadsInFlight - 1) / kLoadsInFlight * kLoadsInFlight;
   a.S = S;
