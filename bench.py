@@ -208,7 +208,7 @@ def cpu_baseline(torch, fmt, M, N, K, seed, seconds=12.0):
     for i in range(3):
         call(i)
     times, i, t_end = [], 3, time.perf_counter() + seconds
-    while time.perf_counter() < t_end and len(times) < 2000:
+    while time.perf_counter() < t_end and len(times) < 200000:
         t0 = time.perf_counter()
         call(i)
         times.append(time.perf_counter() - t0)

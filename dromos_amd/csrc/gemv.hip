@@ -221,7 +221,10 @@ template <int F, int MT, bool XB>
 int launch_rows(const GemvArgs& a, const Shape& shape, hipStream_t stream) {
   if constexpr (MT == 1) {
     switch (shape.depth) {
-      case 8: return launch_stream<F, MT, 1, 8, XB>(a, shape, stream);
+      case 8:
+        // Rows of exactly seven steps (K = 14336 in NVFP4) are asked for whole, without an eighth, repeated load.
+        if (a.split == 1 && a.steps == 7) return launch_stream<F, MT, 1, 7, XB>(a, shape, stream);
+        return launch_stream<F, MT, 1, 8, XB>(a, shape, stream);
       case 4: return launch_stream<F, MT, 2, 4, XB>(a, shape, stream);
       case 2: return launch_stream<F, MT, 4, 2, XB>(a, shape, stream);
       default: return launch_stream<F, MT, 4, 1, XB>(a, shape, stream);
