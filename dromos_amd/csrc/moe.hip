@@ -145,42 +145,44 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
   if (lane < top_k) weights[t * top_k + lane] = __expf(picked_logit[wave][lane] - lmax) / esum;
 }
 
-// Sorts the P pairs by expert (stable) in LDS. order[g] = pair at sorted position g; returns through
-// group_begin / group_end the positions of group `slot` (the slot-th distinct expert in ascending id order),
-// and the number of groups. Run by the whole workgroup.
-__device__ __forceinline__ void group_pairs(const int32_t* ids, int P, int slot, int* s_ids, int* s_order, int* s_info) {
-  if (threadIdx.x < P) s_ids[threadIdx.x] = ids[threadIdx.x];
-  __syncthreads();
-  if (threadIdx.x < P) {
-    const int mine = s_ids[threadIdx.x];
-    int rank = 0;
-    for (int q = 0; q < P; ++q) {
-      const int other = s_ids[q];
-      rank += other < mine || (other == mine && q < static_cast<int>(threadIdx.x));
-    }
-    s_order[rank] = threadIdx.x;
+// The pairs of a step with more than one token, sorted by expert (stable), as the gate/up stage reads them:
+//   table[0]                  number of groups (distinct experts)
+//   table[1 + g], g <= groups first sorted position of group g (table[1 + groups] = P)
+//   table[kTableOrder + p]    the pair at sorted position p
+//   table[kTableExpert + p]   its expert
+constexpr int kTableOrder = 2 + kMaxPairs, kTableExpert = kTableOrder + kMaxPairs, kTableInts = kTableExpert + kMaxPairs;
+constexpr int64_t kTableBytes = 1024;
+static_assert(kTableInts * 4 <= kTableBytes, "the sort table fits its part of the workspace");
+
+// One wavefront sorts the P <= 64 pairs: a pair's rank is the number of pairs with a smaller expert id, or the same
+// id and a smaller index.
+__global__ void __launch_bounds__(kWave) decode_sort_kernel(const int32_t* __restrict__ ids, int P, int* __restrict__ table) {
+  __shared__ int s_ids[kMaxPairs], s_order[kMaxPairs];
+  const int p = threadIdx.x;
+  // A lane past P holds an id above every other: it ranks behind all pairs and is never written.
+  const int mine = p < P ? ids[p] : 0x7fffffff;
+  int rank = 0;
+  for (int q = 0; q < P; ++q) {
+    const int other = __builtin_amdgcn_readlane(mine, q);
+    rank += other < mine || (other == mine && q < p);
+  }
+  if (p < P) {
+    s_ids[p] = mine;
+    s_order[rank] = p;
   }
   __syncthreads();
-  if (threadIdx.x < kWave) {  // the first wavefront: P <= 64 positions
-    const int g = threadIdx.x;
-    const bool starts = g < P && (g == 0 || s_ids[s_order[g]] != s_ids[s_order[g - 1]]);
-    const uint64_t mask = __ballot(starts);
-    if (g == 0) {
-      const int groups = __popcll(mask);
-      int begin = P, end = P;
-      if (slot < groups) {
-        uint64_t mm = mask;
-        for (int i = 0; i < slot; ++i) mm &= mm - 1;  // drop the lower set bits
-        begin = __ffsll(static_cast<unsigned long long>(mm)) - 1;
-        mm &= mm - 1;
-        end = mm ? __ffsll(static_cast<unsigned long long>(mm)) - 1 : P;
-      }
-      s_info[0] = groups;
-      s_info[1] = begin;
-      s_info[2] = end;
-    }
+  const bool starts = p < P && (p == 0 || s_ids[s_order[p]] != s_ids[s_order[p - 1]]);
+  const uint64_t mask = __ballot(starts);
+  const int groups = __popcll(mask);
+  if (starts) table[1 + __popcll(mask & ((1ull << p) - 1))] = p;
+  if (p == 0) {
+    table[0] = groups;
+    table[1 + groups] = P;
   }
-  __syncthreads();
+  if (p < P) {
+    table[kTableOrder + p] = s_order[p];
+    table[kTableExpert + p] = s_ids[s_order[p]];
+  }
 }
 
 // One intermediate row i per wavefront (i = blockIdx.x * waves + wave) of expert e for the cnt <= MT pairs at
@@ -246,12 +248,13 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
 }
 
 // grid = (I / wavefronts per workgroup, group slots); mt_cap (a power of two, the LDS image's rows) bounds a
-// pass's pairs. One token: every slot is its own group and nothing is sorted.
+// pass's pairs. One token: every slot is its own group and nothing is sorted; more: the groups come from the
+// table decode_sort_kernel wrote.
 // ONE: a row's steps fit one batch of U.
 template <int F, int U, bool ONE>
 __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeArgs a, int mt_cap) {
   extern __shared__ __align__(16) float lds[];
-  __shared__ int s_ids[kMaxPairs], s_order[kMaxPairs], s_info[4], s_rows[8];
+  __shared__ int s_rows[8];
   const int P = a.T * a.top_k;
   if (a.T == 1) {
     if (static_cast<int>(blockIdx.y) >= P) return;
@@ -259,31 +262,37 @@ __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeAr
     gate_up_rows<F, U, 1, ONE>(a, lds, e, blockIdx.y, 1, nullptr, nullptr);
     return;
   }
-  group_pairs(a.ids, P, blockIdx.y, s_ids, s_order, s_info);
-  if (static_cast<int>(blockIdx.y) >= s_info[0]) return;
-  const int begin = s_info[1], end = s_info[2];
-  const int e = s_ids[s_order[begin]];
+  if (static_cast<int>(blockIdx.y) >= a.table[0]) return;
+  const int begin = a.table[1 + blockIdx.y], end = a.table[2 + blockIdx.y];
+  const int e = a.table[kTableExpert + begin];
+  const int* const order = a.table + kTableOrder;
   // A group larger than the image (an expert repeated within a token) runs mt_cap pairs at a time.
   for (int first = begin; first < end; first += mt_cap) {
     const int cnt = min(mt_cap, end - first);
     __syncthreads();
-    if (threadIdx.x < 8) s_rows[threadIdx.x] = static_cast<int>(threadIdx.x) < cnt ? s_order[first + threadIdx.x] / a.top_k : 0;
+    if (threadIdx.x < 8) s_rows[threadIdx.x] = static_cast<int>(threadIdx.x) < cnt ? order[first + threadIdx.x] / a.top_k : 0;
     __syncthreads();
-    if (cnt <= 1) gate_up_rows<F, U, 1, ONE>(a, lds, e, first, cnt, s_order, s_rows);
-    else if (cnt <= 2) gate_up_rows<F, U, 2, ONE>(a, lds, e, first, cnt, s_order, s_rows);
-    else if (cnt <= 4) gate_up_rows<F, U, 4, ONE>(a, lds, e, first, cnt, s_order, s_rows);
-    else gate_up_rows<F, U, 8, ONE>(a, lds, e, first, cnt, s_order, s_rows);
+    if (cnt <= 1) gate_up_rows<F, U, 1, ONE>(a, lds, e, first, cnt, order, s_rows);
+    else if (cnt <= 2) gate_up_rows<F, U, 2, ONE>(a, lds, e, first, cnt, order, s_rows);
+    else if (cnt <= 4) gate_up_rows<F, U, 4, ONE>(a, lds, e, first, cnt, order, s_rows);
+    else gate_up_rows<F, U, 8, ONE>(a, lds, e, first, cnt, order, s_rows);
   }
 }
 
-// grid = (L / wavefronts per workgroup, T): one output row l per wavefront. Its stream is the token's top_k
+// One workgroup per (l block, token): one output row l per wavefront. Its stream is the token's top_k
 // experts' copies of row l, four at a time, each against its own slot's intermediate row, and
 // out[t, l] = w0 * c0 + sum_{k >= 1} w_k * c_k in slot order (engine/cpu/moe.cpp:315-327), c_k = rowfactor * dot.
 template <int F, int U>
 __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs a) {
   extern __shared__ __align__(16) float lds[];
   constexpr int R = 4;
-  const int t = blockIdx.y;
+  // Workgroup ids run over (l block / 8, token, l block % 8), the last fastest: consecutive ids land on different
+  // dies, so the eight l blocks of a token spread over them while the tokens of one l block follow each other on
+  // the same die, where an expert row that two tokens share is still in that die's L2.
+  const int n_lblocks = (a.L + (blockDim.x / kWave) - 1) / (blockDim.x / kWave);
+  const int t = (blockIdx.x >> 3) % a.T;
+  const int lblock = (blockIdx.x / (8 * a.T)) * 8 + (blockIdx.x & 7);
+  if (lblock >= n_lblocks) return;
   const int steps = steps_for<F>(a.I);
   const int per_row = x_row_words<F, true>(steps);  // the packed bf16 image: the intermediate rows are bf16
   const int64_t rb = row_bytes<F>(a.I);
@@ -291,7 +300,7 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
   const int64_t scale_row = F == LX_W_NVFP4 ? a.I / 16 : 0;
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int top_k = a.top_k;
-  const int l = blockIdx.x * (blockDim.x / kWave) + wave;
+  const int l = lblock * (blockDim.x / kWave) + wave;
   const int lc = min(l, a.L - 1);
 
   // Group c holds slots 4c .. 4c + 3 (a slot past top_k repeats the last one and is not added).
@@ -419,7 +428,8 @@ int launch_down_u(const DecodeArgs& a, hipStream_t s) {
   const size_t lds = sizeof(float) * 8 * x_row_words<F, true>(steps_for<F>(a.I));
   auto kernel = decode_down_kernel<F, U>;
   allow_big_lds(kernel, lds);
-  hipLaunchKernelGGL(kernel, dim3((a.L + kWaves - 1) / kWaves, a.T), dim3(kThreads), lds, s, a);
+  const int n_lblocks = (a.L + kWaves - 1) / kWaves;
+  hipLaunchKernelGGL(kernel, dim3((n_lblocks + 7) / 8 * 8 * a.T), dim3(kThreads), lds, s, a);
   return status_of(hipGetLastError());
 }
 
@@ -459,6 +469,7 @@ int experts_decode(const void* latent, const int32_t* ids, const float* weights,
   a.gu = as_stack(gate_up);
   a.dn = as_stack(down);
   a.inter = static_cast<uint16_t*>(inter);
+  a.table = reinterpret_cast<const int*>(static_cast<const char*>(inter) + round256(2 * static_cast<int64_t>(T) * top_k * I));
   a.out = out;
   a.T = T;
   a.L = L;
@@ -473,6 +484,10 @@ int experts_decode(const void* latent, const int32_t* ids, const float* weights,
     }
   };
   int st;
+  if (T > 1 && can_stream(gate_up.type, a.gu, L)) {
+    hipLaunchKernelGGL(decode_sort_kernel, dim3(1), dim3(kWave), 0, s, ids, T * top_k, const_cast<int*>(a.table));
+    if ((st = status_of(hipGetLastError()))) return st;
+  }
   if (!can_stream(gate_up.type, a.gu, L)) {
     st = gate_up_plain(a, gate_up.type, s);
   } else {
@@ -532,7 +547,8 @@ int lx_moe_experts_decode(const void* latent, const int32_t* ids, const float* w
 
 int64_t lx_moe_decode_workspace_bytes(int T, int I, int top_k) {
   if (T <= 0 || I <= 0 || top_k <= 0) return 0;
-  return round256(2 * static_cast<int64_t>(T) * top_k * I);
+  // The intermediate rows, and behind them the table of the pairs sorted by expert.
+  return round256(2 * static_cast<int64_t>(T) * top_k * I) + kTableBytes;
 }
 
 int64_t lx_moe_bf16x_workspace_bytes(int T, int I, int top_k) { return lx_moe_decode_workspace_bytes(T, I, top_k); }

@@ -18,6 +18,7 @@ struct DecodeArgs {
   const float* weights;    // [T, top_k]
   Stack gu, dn;
   uint16_t* inter;  // bf16 [T * top_k, I], by pair
+  const int* table;  // the pairs sorted by expert (more than one token): see decode_sort_kernel
   float* out;       // f32 [T, L]
   int T, L, I, top_k;
 };
