@@ -200,6 +200,9 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int64_t stack_row0 = static_cast<int64_t>(e) * 2 * a.I;
   const int i = blockIdx.x * (blockDim.x / kWave) + wave;
+  // The two rows' factors are asked for now: the epilogue should not wait for a load of its own.
+  const int64_t my_gate_row = stack_row0 + min(i, a.I - 1);
+  const float sg = stack_factor(F, a.gu, e, my_gate_row), su = stack_factor(F, a.gu, e, my_gate_row + a.I);
   auto rows_fn = [&](int ii, const uint8_t* (&rows)[2], const uint8_t* (&scales)[2], const float* (&x_image)[2]) {
     const int64_t gate_row = stack_row0 + min(ii, a.I - 1), up_row = gate_row + a.I;
     rows[0] = a.gu.data + gate_row * rb;
@@ -216,8 +219,6 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
       acc[m][1] = wave_sum(acc[m][1]);
     }
     if (lane == 0 && ii < a.I) {
-      const int64_t gate_row = stack_row0 + ii, up_row = gate_row + a.I;
-      const float sg = stack_factor(F, a.gu, e, gate_row), su = stack_factor(F, a.gu, e, up_row);
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
         if (m < cnt) {
@@ -303,12 +304,18 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
   const int l = lblock * (blockDim.x / kWave) + wave;
   const int lc = min(l, a.L - 1);
 
+  // The token's experts, routing weights and row factors are asked for first: everything else hangs on the ids,
+  // and the epilogue should not wait for a load of its own. Slot k's values sit in lane k.
+  const int my_slot = min(lane, top_k - 1);
+  const int my_e = a.ids[t * top_k + my_slot];
+  const float my_weight = a.weights[t * top_k + my_slot];
+  const float my_factor = stack_factor(F, a.dn, my_e, static_cast<int64_t>(my_e) * a.L + lc);
   // Group c holds slots 4c .. 4c + 3 (a slot past top_k repeats the last one and is not added).
   auto rows_fn = [&](int c, const uint8_t* (&rows)[R], const uint8_t* (&scales)[R], const float* (&x_image)[R]) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
       const int k = min(c * R + r, top_k - 1);
-      const int e = a.ids[t * top_k + k];
+      const int e = __builtin_amdgcn_readlane(my_e, k);
       const int64_t row = static_cast<int64_t>(e) * a.L + lc;
       rows[r] = a.dn.data + row * rb;
       scales[r] = a.dn.scale + row * scale_row;
@@ -322,9 +329,8 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
       const int k = c * R + r;
       const float sum = wave_sum(acc[0][r]);
       if (k < top_k) {
-        const int e = a.ids[t * top_k + k];
-        const float contrib = stack_factor(F, a.dn, e, static_cast<int64_t>(e) * a.L + lc) * sum;
-        const float wc = a.weights[t * top_k + k] * contrib;
+        const float contrib = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_factor), k)) * sum;
+        const float wc = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(my_weight), k)) * contrib;
         o = k == 0 ? wc : o + wc;
       }
     }
