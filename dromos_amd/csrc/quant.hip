@@ -64,6 +64,54 @@ __device__ __forceinline__ float block_max(float v, float* shared) {
   return m;
 }
 
+// Per-token activation quantisation (engine/cuda/kernels.h:479-493; engine/cpu/quant.cpp:159-203): one workgroup per
+// row. Unlike the weight quantisers it multiplies by a reciprocal: inv = qmax / a and q = round(x * inv); FP4:
+// g = a / 2688, s_b = e4m3(a_b / (6 g)), r = 1 / (s_b g), code = e2m1(x * r). A zero row gets scale 1 and zeros.
+__global__ void __launch_bounds__(kThreads) quantize_act_kernel(const void* __restrict__ x, int x_dtype, int64_t ld_x, int math,
+                                                                uint8_t* __restrict__ q, int64_t ld_q, float* __restrict__ scale,
+                                                                uint8_t* __restrict__ block_scale, int64_t ld_bs, int K) {
+  __shared__ float shared[kWaves];
+  const int64_t m = blockIdx.x, base = m * ld_x;
+  float a = 0.0f;
+  for (int k = threadIdx.x; k < K; k += kThreads) a = fmaxf(a, fabsf(load_as_f32(x, x_dtype, base + k)));
+  a = block_max(a, shared);
+  uint8_t* const row = q + m * ld_q;
+  if (math == LX_MATH_INT8 || math == LX_MATH_FP8) {
+    const float qmax = math == LX_MATH_INT8 ? 127.0f : 448.0f;
+    const float inv = a > 0.0f ? qmax / a : 0.0f;
+    for (int k = threadIdx.x; k < K; k += kThreads) {
+      const float v = load_as_f32(x, x_dtype, base + k) * inv;
+      if (math == LX_MATH_INT8) row[k] = static_cast<uint8_t>(static_cast<int8_t>(static_cast<int>(fminf(fmaxf(rintf(v), -127.0f), 127.0f))));
+      else row[k] = static_cast<uint8_t>(e4m3_encode(v));
+    }
+    if (threadIdx.x == 0) scale[m] = a > 0.0f ? a / qmax : 1.0f;
+    return;
+  }
+  const float g = a > 0.0f ? a / 2688.0f : 1.0f;
+  if (threadIdx.x == 0) scale[m] = g;
+  for (int b = threadIdx.x; b < K / 16; b += kThreads) {  // a thread per block of 16
+    float v[16], amax = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      v[j] = load_as_f32(x, x_dtype, base + 16 * b + j);
+      amax = fmaxf(amax, fabsf(v[j]));
+    }
+    const uint32_t s8 = e4m3_encode(amax / (6.0f * g));
+    block_scale[m * ld_bs + b] = static_cast<uint8_t>(s8);
+    const float d = e4m3_decode(s8) * g;
+    const float r = d > 0.0f ? 1.0f / d : 0.0f;
+#pragma unroll
+    for (int p = 0; p < 8; ++p) {
+      uint32_t lo = 0, hi = 0;
+      if (d > 0.0f) {
+        lo = e2m1_encode(v[2 * p] * r);
+        hi = e2m1_encode(v[2 * p + 1] * r);
+      }
+      row[8 * b + p] = static_cast<uint8_t>(lo | (hi << 4));
+    }
+  }
+}
+
 // One workgroup per row: absmax, then the row's codes. FP8 = false is INT8.
 template <bool FP8>
 __global__ void __launch_bounds__(kThreads) quantize_rows_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ q,
@@ -243,6 +291,22 @@ int lx_dequantize_weight(const lx_weight* w, void* out, int64_t rows, int cols, 
   hipLaunchKernelGGL(dequantize_kernel, dim3(static_cast<unsigned>((n + kThreads - 1) / kThreads)), dim3(kThreads), 0, s,
                      static_cast<int>(w->type), static_cast<const uint8_t*>(w->data), static_cast<const uint8_t*>(w->scale),
                      w->global, static_cast<uint16_t*>(out), rows, cols);
+  return status_of(hipGetLastError());
+}
+
+int lx_quantize_act(const void* x, lx_dtype x_dtype, int ld_x, lx_math math, void* q, int ld_q, float* scale, void* block_scale,
+                    int ld_bs, int M, int K, void* stream) {
+  if (M <= 0) return kOk;
+  if (!x || !q || !scale || K <= 0 || (x_dtype != LX_F32 && x_dtype != LX_BF16) || (M > 1 && ld_x < K)) return fail(kInvalid);
+  if (math != LX_MATH_INT8 && math != LX_MATH_FP8 && math != LX_MATH_FP4) return fail(kInvalid);
+  if (math == LX_MATH_FP4) {
+    if (K % 16 != 0 || !block_scale || (M > 1 && (ld_q < K / 2 || ld_bs < K / 16))) return fail(kInvalid);
+  } else if (M > 1 && ld_q < K) {
+    return fail(kInvalid);
+  }
+  hipLaunchKernelGGL(quantize_act_kernel, dim3(static_cast<unsigned>(M)), dim3(kThreads), 0, as_stream(stream), x, static_cast<int>(x_dtype),
+                     static_cast<int64_t>(ld_x), static_cast<int>(math), static_cast<uint8_t*>(q), static_cast<int64_t>(ld_q), scale,
+                     static_cast<uint8_t*>(block_scale), static_cast<int64_t>(ld_bs), K);
   return status_of(hipGetLastError());
 }
 

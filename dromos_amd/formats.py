@@ -192,6 +192,35 @@ def quantize_reference(w, fmt):
     return Weight(W_NVFP4, packed, s8, glob.item())
 
 
+def quantize_act_reference(x, math):
+    """Per-token activation quantisation by the contract's rules (engine/cuda/kernels.h:479-493), restated in torch
+    with IEEE f32 operations: INT8 q = rne(x * (127 / a)), FP8 q = e4m3(x * (448 / a)), FP4 g = a / 2688,
+    s_b = e4m3(a_b / (6 g)), code = e2m1(x * (1 / (s_b g))). Returns (q bytes, scale f32 [M], block scales or None).
+    The reference's own tests derive the same three tensors this way (tests/kernels/wformats.py)."""
+    xf = x.float().cpu()
+    a = xf.abs().amax(-1)
+    live = a > 0
+    safe = torch.where(live, a, torch.ones_like(a))
+    if math in (1, 2):
+        qmax = 127.0 if math == 1 else 448.0
+        inv = torch.where(live, _div(qmax, safe), torch.zeros_like(a))
+        v = xf * inv.unsqueeze(-1)
+        q = torch.round(v).clamp(-127, 127).to(torch.int8).view(torch.uint8) if math == 1 else e4m3_bytes(v)
+        return q, torch.where(live, _div(safe, qmax), torch.ones_like(a)), None
+    M, K = xf.shape
+    assert K % 16 == 0
+    g = torch.where(live, _div(safe, 2688.0), torch.ones_like(a))
+    blocks = xf.reshape(M, K // 16, 16)
+    bmax = blocks.abs().amax(-1)
+    s8 = e4m3_bytes(_div(bmax, (6.0 * g).unsqueeze(-1)))
+    d = s8.view(torch.float8_e4m3fn).float() * g.unsqueeze(-1)
+    on = d > 0
+    r = torch.where(on, _div(1.0, torch.where(on, d, torch.ones_like(d))), torch.zeros_like(d))
+    codes = torch.where(on.unsqueeze(-1), e2m1_codes(blocks * r.unsqueeze(-1)).int(), 0).to(torch.uint8).reshape(M, K)
+    packed = (codes[:, 0::2] | (codes[:, 1::2] << 4)).contiguous()
+    return packed, g, s8
+
+
 def alloc_quantized(fmt, N, K, device):
     """Empty buffers of the right sizes for lx_quantize_weight to fill."""
     if fmt == W_INT8:

@@ -99,6 +99,16 @@ LX_API int lx_quantize_w8(const void* w, int8_t* q, float* scale, int64_t rows, 
 LX_API int lx_quantize_weight(const void* w, lx_weight* out, int64_t rows, int cols, void* stream);
 LX_API int lx_dequantize_weight(const lx_weight* w, void* out, int64_t rows, int cols, void* stream);
 
+/* ---- per-token activation quantiser (replaces engine/cuda/kernels.h:479-493) ---------------------------
+ * x [M, K] (x_dtype, row stride ld_x). Per row, a = max |x|: INT8 q = rne(x * (127 / a)) clamped to +-127,
+ * scale[m] = a / 127; FP8 q = e4m3(x * (448 / a)), scale[m] = a / 448; FP4 (K % 16 == 0) two e2m1 per byte,
+ * block_scale e4m3 [M, ld_bs] one per 16 k, scale[m] = g = a / 2688, s_b = e4m3(a_b / (6 g)),
+ * q = e2m1(x * (1 / (s_b g))), 0 where s_b = 0. A zero row: scale 1, q = 0. ld_q and ld_bs are in bytes.
+ * Bytes identical to engine/cpu/quant.cpp:159-203. (The low-precision maths that consume it are not on this
+ * path yet: lx_gemm_w and lx_moe_experts_grouped answer 801 for them.) */
+LX_API int lx_quantize_act(const void* x, lx_dtype x_dtype, int ld_x, lx_math math, void* q, int ld_q, float* scale,
+                           void* block_scale, int ld_bs, int M, int K, void* stream);
+
 /* ---- routing and routed experts (replaces engine/cuda/kernels.h:203-209, 220-225, 495-511, 606-611)
  * lx_moe_route: per row of f32 logits [T, E]: entropy and confidence of the softmax, ids = top_k by
  * logit + selection_bias (ties to the lower index), weights = softmax of the picked unbiased logits.

@@ -231,6 +231,63 @@ ORC_API int lx_quantize_weight(const void* w, lx_weight* out, int64_t rows, int 
   }
 }
 
+/* Per-token activation quantisation (contract engine/cuda/kernels.h:479-493; engine/cpu/quant.cpp:159-203,273-292).
+ * Unlike the weight quantisers it multiplies by a reciprocal: inv = qmax / a, q = round(x * inv); FP4 r = 1 / (s_b g).
+ * Pinned bit for bit against oracle/_ref and the golden vectors (tests/test_oracle_quant.py, tests/test_golden.py). */
+static void quant_act_row(const void* x, int x_dtype, int64_t base, int math, int K, uint8_t* q, float* scale, uint8_t* block_scale) {
+  float a = 0.0f;
+  for (int k = 0; k < K; ++k) a = fmaxf(a, fabsf(load_f32(x, x_dtype, base + k)));
+  if (math == LX_MATH_INT8 || math == LX_MATH_FP8) {
+    const float qmax = math == LX_MATH_INT8 ? 127.0f : 448.0f;
+    const float inv = a > 0.0f ? qmax / a : 0.0f;
+    for (int k = 0; k < K; ++k) {
+      const float v = load_f32(x, x_dtype, base + k) * inv;
+      if (math == LX_MATH_INT8) ((int8_t*)q)[k] = (int8_t)(int)fminf(fmaxf(rintf(v), -127.0f), 127.0f);
+      else q[k] = orc_f32_to_e4m3(v);
+    }
+    *scale = a > 0.0f ? a / qmax : 1.0f;
+    return;
+  }
+  const float g = a > 0.0f ? a / 2688.0f : 1.0f;
+  *scale = g;
+  for (int b = 0; b < K / 16; ++b) {
+    float v[16], amax = 0.0f;
+    for (int j = 0; j < 16; ++j) {
+      v[j] = load_f32(x, x_dtype, base + 16 * b + j);
+      amax = fmaxf(amax, fabsf(v[j]));
+    }
+    const uint8_t s8 = orc_f32_to_e4m3(amax / (6.0f * g));
+    block_scale[b] = s8;
+    const float d = orc_e4m3_to_f32(s8) * g;
+    const float r = d > 0.0f ? 1.0f / d : 0.0f;
+    for (int p = 0; p < 8; ++p) {
+      uint32_t lo = 0, hi = 0;
+      if (d > 0.0f) {
+        lo = orc_f32_to_e2m1(v[2 * p] * r);
+        hi = orc_f32_to_e2m1(v[2 * p + 1] * r);
+      }
+      q[8 * b + p] = (uint8_t)(lo | (hi << 4));
+    }
+  }
+}
+
+ORC_API int lx_quantize_act(const void* x, int x_dtype, int ld_x, int math, void* q, int ld_q, float* scale, void* block_scale,
+                            int ld_bs, int M, int K, void* stream) {
+  (void)stream;
+  if (M <= 0) return ORC_OK;
+  if (!x || !q || !scale || K <= 0 || !dtype_ok(x_dtype) || (M > 1 && ld_x < K)) return fail(ORC_INVALID);
+  if (math != LX_MATH_INT8 && math != LX_MATH_FP8 && math != LX_MATH_FP4) return fail(ORC_INVALID);
+  if (math == LX_MATH_FP4) {
+    if (K % 16 != 0 || !block_scale || (M > 1 && (ld_q < K / 2 || ld_bs < K / 16))) return fail(ORC_INVALID);
+  } else if (M > 1 && ld_q < K) {
+    return fail(ORC_INVALID);
+  }
+  for (int64_t m = 0; m < M; ++m)
+    quant_act_row(x, x_dtype, m * ld_x, math, K, (uint8_t*)q + m * ld_q, scale + m,
+                  block_scale ? (uint8_t*)block_scale + m * ld_bs : NULL);
+  return ORC_OK;
+}
+
 /* Element (n, k) of an [N, K] weight, exact, without its row factor (engine/cpu/quant.cpp:143-154). */
 static float weight_element(int type, const void* data, const void* scale, int64_t n, int64_t k, int64_t K) {
   switch (type) {

@@ -154,6 +154,58 @@ def gemv_nvfp4_global_is_linear(lx):
     assert torch.equal(y2, 2.0 * y1)
 
 
+# ---- activation quantiser ----------------------------------------------------------------------------------
+
+
+def quantize_act_case(lx, math, M, K, seed, x_dtype=torch.float32, pad=0, x_pad=0):
+    """Bytes, row scales and block scales equal the contract's rules; nothing is written past a row."""
+    from dromos_amd.formats import quantize_act_reference
+
+    g = torch.Generator().manual_seed(seed)
+    x_buf = (torch.randn(M, K + x_pad, generator=g) * torch.rand(M, 1, generator=g) * 4).to(x_dtype)
+    x_buf[0, :K] *= 1e-3  # a quiet row: small scales, subnormal e4m3 block scales for FP4
+    if M > 2:
+        x_buf[2, :K] = 0  # a zero row
+    x = x_buf[:, :K]
+    q, scale, bs = ops.quantize_act(lx, dev(lx, x_buf), math, pad=pad, K=K)
+    want_q, want_scale, want_bs = quantize_act_reference(x, math)
+    width = want_q.shape[1]
+    q, scale = q.cpu(), scale.cpu()
+    assert torch.equal(q[:, :width], want_q), f"quantised values differ at {(q[:, :width] != want_q).nonzero()[:4].tolist()}"
+    assert torch.equal(scale.view(torch.int32), want_scale.float().view(torch.int32)), "per-row scales differ"
+    assert bool((q[:, width:] == 0xAB).all()), "wrote past the row"
+    if want_bs is not None:
+        bs = bs.cpu()
+        assert torch.equal(bs[:, : K // 16], want_bs), "block scales differ"
+        assert bool((bs[:, K // 16 :] == 0xAB).all()), "wrote past the block scales"
+    if M > 2:
+        assert bool((q[2, :width] == 0).all()) and scale[2].item() == 1.0, "a zero row quantises to 0 with scale 1"
+    return q, scale, bs
+
+
+def quantize_act_fp4_extremes(lx):
+    """Ties of the e2m1 rounding, saturation, and a block whose scale underflows to zero
+    (the cases of tests/kernels/test_quant_act.py:59-72 of the reference)."""
+    from dromos_amd.abi import MATH_FP4
+    from dromos_amd.formats import quantize_act_reference
+
+    M, K = 4, 64
+    x = torch.zeros(M, K)
+    x[0, :16] = torch.tensor([0.25, 0.75, 1.25, 1.75, 2.5, 3.5, 5.0, 6.0, -0.25, -0.75, -2.5, -5.0, 0.1, 7.0, -7.0, 3.0])
+    x[1, :16] = 1.0
+    x[1, 16:32] = 1e-6
+    x[2] = torch.linspace(-3, 3, K)
+    q, scale, bs = ops.quantize_act(lx, dev(lx, x), MATH_FP4)
+    want_q, want_scale, want_bs = quantize_act_reference(x, MATH_FP4)
+    assert torch.equal(q.cpu(), want_q) and torch.equal(scale.cpu(), want_scale.float()) and torch.equal(bs.cpu(), want_bs)
+    # Known answers, by hand: row 1's first block is all ones with the row's absmax 1: g = 1 / 2688,
+    # s_b = e4m3(1 / (6 g)) = e4m3(448) = 0x7e, code = e2m1(1 * (1 / (448 / 2688))) = e2m1(6) = 7; its second block
+    # underflows: scale byte 0 and zero codes; the all-zero row 3 has scale 1.
+    assert bs[1, 0].item() == 0x7E and bool((q[1, :8].cpu() == 0x77).all())
+    assert bs[1, 1].item() == 0 and bool((q[1, 8:16].cpu() == 0).all())
+    assert scale[3].item() == 1.0 and bool((q[3].cpu() == 0).all())
+
+
 # ---- routing ----------------------------------------------------------------------------------------------
 
 

@@ -55,6 +55,18 @@ def quantize(lx, fmt):
     return [w], out
 
 
+def quantize_act(lx, math, x_dtype):
+    g = torch.Generator().manual_seed(4150 + math)
+    x = (torch.randn(9, 160, generator=g) * torch.rand(9, 1, generator=g) * 4).to(x_dtype)
+    x[0] *= 1e-3  # subnormal block scales
+    x[2] = 0  # a zero row
+    q, scale, bs = ops.quantize_act(lx, x.to(lx.device), math)
+    out = {"data": q, "scale": scale}
+    if bs is not None:
+        out["block_scale"] = bs
+    return [x], out
+
+
 def gemv(lx, fmt, x_dtype, y_dtype):
     M, N, K = 3, 40, 352
     g = torch.Generator().manual_seed(4200 + FORMATS[fmt])
@@ -129,12 +141,15 @@ for _f in FORMATS:
     CASES[f"experts_grouped_{_f}"] = (experts_grouped, (_f,))
 CASES["gemv_int8_f32x_bf16y"] = (gemv, ("int8", torch.float32, torch.bfloat16))
 CASES["gemv_bf16_f32x_f32y"] = (gemv, ("bf16", torch.float32, torch.float32))
+for _m, _n in ((1, "int8"), (2, "fp8"), (3, "fp4")):
+    CASES[f"quantize_act_{_n}_bf16"] = (quantize_act, (_m, torch.bfloat16))
+CASES["quantize_act_fp8_f32"] = (quantize_act, (2, torch.float32))
 CASES["route"] = (route, ())
 CASES["experts_bf16"] = (experts_bf16, ())
 
 # Outputs whose bits every backend must reproduce (codec and index work); the rest are f32 sums whose last
 # bits depend on the summation order (the reference's own differ between its ISA levels).
-EXACT = {"data", "scale", "global", "dequantized", "ids"}
+EXACT = {"data", "scale", "global", "dequantized", "ids", "block_scale"}
 
 
 def run_case(lx, name):

@@ -71,6 +71,25 @@ def dequantize(lx, w, N, K):
     return out
 
 
+def quantize_act(lx, x, math, pad=0, status=False, K=None):
+    """lx_quantize_act on the first K columns of x [M, ld_x]; returns (q bytes [M, ld_q], scale [M], block scales
+    [M, ld_bs] or None). pad > 0 widens the output rows, filled with 0xAB, to show nothing is written past a row."""
+    from dromos_amd.abi import MATH_FP4
+
+    M = x.shape[0]
+    K = x.shape[1] if K is None else K
+    ld_q = (K // 2 if math == MATH_FP4 else K) + pad
+    q = torch.full((M, ld_q), 0xAB, dtype=torch.uint8, device=lx.device)
+    scale = torch.full((M,), float("nan"), dtype=torch.float32, device=lx.device)
+    ld_bs = K // 16 + pad if math == MATH_FP4 else 0
+    bs = torch.full((M, max(ld_bs, 1)), 0xAB, dtype=torch.uint8, device=lx.device) if math == MATH_FP4 else None
+    args = (x, DTYPE[x.dtype], x.shape[1], math, q, ld_q, scale, bs, ld_bs, M, K)
+    if status:
+        return lx.status("quantize_act", *args)
+    lx("quantize_act", *args)
+    return q, scale, bs
+
+
 def route(lx, logits, bias, top_k):
     T, E = logits.shape
     ids = torch.full((T, top_k), -1, dtype=torch.int32, device=lx.device)

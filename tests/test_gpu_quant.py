@@ -75,3 +75,43 @@ def test_empty_and_invalid(hip):
     assert hip.status("quantize_w8", w, q, s, ctypes.c_int64(4), 0) == 1
     assert hip.status("quantize_w8", None, q, s, ctypes.c_int64(4), 16) == 1
     assert hip.lib.lx_rt_last_error() == 1 and hip.lib.lx_rt_last_error() == 0
+
+
+# ---- the per-token activation quantiser -------------------------------------------------------------------
+
+ACT_SHAPES = [(1, 2048), (7, 1024), (300, 512), (64, 6400), (5, 4096), (3, 16)]
+
+
+@pytest.mark.parametrize("pad", [0, 8])
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("math", [1, 2, 3])
+@pytest.mark.parametrize("M,K", ACT_SHAPES)
+def test_quantize_act_matches_the_rules(hip, M, K, math, x_dtype, pad):
+    checks.quantize_act_case(hip, math, M, K, seed=M * 31 + K + math, x_dtype=x_dtype, pad=pad * 2, x_pad=pad)
+
+
+@pytest.mark.parametrize("math", [1, 2])
+def test_quantize_act_odd_k(hip, math):
+    checks.quantize_act_case(hip, math, 9, 1001, seed=5, x_pad=3, pad=7)
+
+
+def test_quantize_act_fp4_extremes(hip):
+    checks.quantize_act_fp4_extremes(hip)
+
+
+@pytest.mark.parametrize("math", [1, 2, 3])
+def test_quantize_act_equals_the_oracle(hip, oracle, math):
+    g = torch.Generator().manual_seed(40 + math)
+    x = (torch.randn(257, 4096, generator=g) * torch.rand(257, 1, generator=g) * 4).to(torch.bfloat16)
+    x[4] = 0
+    a, b = ops.quantize_act(hip, x.cuda(), math), ops.quantize_act(oracle, x, math)
+    assert torch.equal(a[0].cpu(), b[0]) and torch.equal(a[1].cpu().view(torch.int32), b[1].view(torch.int32))
+    if math == 3:
+        assert torch.equal(a[2].cpu(), b[2])
+
+
+def test_quantize_act_invalid(hip):
+    x = torch.zeros(4, 24, device="cuda")
+    assert ops.quantize_act(hip, x, 3, status=True) == 1
+    assert ops.quantize_act(hip, x, 0, status=True) == 1
+    assert ops.quantize_act(hip, x[:0], 1, status=True) == 0

@@ -68,3 +68,43 @@ def test_bytes_equal_the_reference_backend(oracle, ref, fmt):
     assert torch.equal(a.scale.view(torch.uint8), b.scale.view(torch.uint8)) and a.glob == b.glob
     da, db = ops.dequantize(oracle, a, 257, 1024), ops.dequantize(ref, b, 257, 1024)
     assert torch.equal(da.view(torch.int16), db.view(torch.int16))
+
+
+# ---- the per-token activation quantiser -------------------------------------------------------------------
+
+ACT_SHAPES = [(1, 2048), (7, 1024), (300, 512), (64, 6400), (5, 4096), (3, 16)]
+
+
+@pytest.mark.parametrize("pad", [0, 8])
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("math", [1, 2, 3])
+@pytest.mark.parametrize("M,K", ACT_SHAPES)
+def test_quantize_act_matches_the_rules(oracle, M, K, math, x_dtype, pad):
+    checks.quantize_act_case(oracle, math, M, K, seed=M * 31 + K + math, x_dtype=x_dtype, pad=pad * 2, x_pad=pad)
+
+
+@pytest.mark.parametrize("math", [1, 2])
+def test_quantize_act_odd_k(oracle, math):
+    checks.quantize_act_case(oracle, math, 9, 1001, seed=5, x_pad=3, pad=7)
+
+
+def test_quantize_act_fp4_extremes(oracle):
+    checks.quantize_act_fp4_extremes(oracle)
+
+
+@pytest.mark.parametrize("math", [1, 2, 3])
+def test_quantize_act_equals_the_reference_backend(oracle, ref, math):
+    g = torch.Generator().manual_seed(40 + math)
+    x = (torch.randn(33, 1024, generator=g) * torch.rand(33, 1, generator=g) * 4).to(torch.bfloat16)
+    x[4] = 0
+    a, b = ops.quantize_act(oracle, x, math), ops.quantize_act(ref, x, math)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1].view(torch.int32), b[1].view(torch.int32))
+    if math == 3:
+        assert torch.equal(a[2], b[2])
+
+
+def test_quantize_act_invalid(oracle):
+    x = torch.zeros(4, 24)
+    assert ops.quantize_act(oracle, x, 3, status=True) == 1  # FP4 needs K % 16 == 0
+    assert ops.quantize_act(oracle, x, 0, status=True) == 1  # BF16 is not a quantised math
+    assert ops.quantize_act(oracle, x[:0], 1, status=True) == 0
