@@ -78,7 +78,7 @@ class Timer:
         return times[len(times) // 2]
 
 
-def make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, invariant=False):
+def make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, invariant=False, math=0):
     """Returns (step, bytes_per_step, cleanup-free holder). Weight copies: one quantised master, cloned."""
     from dromos_amd.abi import DTYPE, F32, FORMATS
     from dromos_amd.formats import Weight, master_weight, quantize_with
@@ -95,7 +95,7 @@ def make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, invariant=False):
     ptrs = [ctypes.pointer(s) for s in structs]
     y = torch.empty(M, N, dtype=torch.float32, device="cuda")
     nbytes = algorithmic_bytes_gemv(fmt, M, N, K)
-    ws_buf = torch.empty(max(int(lx.size("gemm_workspace_bytes", M, K, 0)), 256), dtype=torch.uint8, device="cuda")
+    ws_buf = torch.empty(max(int(lx.size("gemm_workspace_bytes", M, K, math)), 256), dtype=torch.uint8, device="cuda")
 
     def step(i):
         p = ptrs[i % copies]
@@ -104,7 +104,7 @@ def make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, invariant=False):
         elif entry == "gemm_skinny":
             st = lx.status("gemm_skinny", x, DTYPE[x.dtype], K, p, None, F32, y, F32, N, M, N, K, 1.0, 0.0)
         else:
-            st = lx.status("gemm_w", x, DTYPE[x.dtype], K, p, 0, None, F32, y, F32, N, M, N, K, 1.0, 0.0, ws_buf)
+            st = lx.status("gemm_w", x, DTYPE[x.dtype], K, p, math, None, F32, y, F32, N, M, N, K, 1.0, 0.0, ws_buf)
         assert st == 0, st
 
     return step, nbytes, (ws, structs, ptrs, x, y, ws_buf)
@@ -262,16 +262,17 @@ def main():
 
     cases = []
 
-    def run_gemv(name, fmt, M, N, K, seed, entry="gemv_w", invariant=False):
+    def run_gemv(name, fmt, M, N, K, seed, entry="gemv_w", invariant=False, math=0):
         if invariant:
             os.environ["LX_BATCH_INVARIANT"] = "1"
         else:
             os.environ.pop("LX_BATCH_INVARIANT", None)
-        step, nbytes, keep = make_gemv_case(lx, torch, fmt, M, N, K, seed, entry)
+        step, nbytes, keep = make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, math=math)
         us = timer.run(step, K_STEPS, W)
         os.environ.pop("LX_BATCH_INVARIANT", None)
         gbps = nbytes / us / 1e3
-        case = {"case": name, "entry": "lx_" + entry, "format": fmt, "M": M, "N": N, "K": K, "batch_invariant": invariant,
+        case = {"case": name, "entry": "lx_" + entry, "format": fmt, "math": ["bf16", "int8", "fp8", "fp4"][math], "M": M, "N": N, "K": K,
+                "batch_invariant": invariant,
                 "us_per_step": round(us, 3), "bytes_per_step": int(nbytes), "GBps": round(gbps, 1),
                 "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)}
         cases.append(case)
@@ -307,6 +308,10 @@ def main():
                     run_gemv(f"C2 {fmt} M={M}" + (" invariant" if inv else ""), fmt, M, 14336, 4096, 1000 + M, entry="gemm_w", invariant=inv)
             for M in (1, 4):
                 run_gemv(f"C2 {fmt} M={M} invariant", fmt, M, 14336, 4096, 1000 + M, invariant=True)
+        for M in (1, 16, 64):
+            # Not a BASELINE configuration: the low-precision math of the same product (activations quantised per token
+            # inside the call, exact int32 sums); the bytes are the weight-only count.
+            run_gemv(f"C2 int8 M={M} INT8 math", "int8", M, 14336, 4096, 1000 + M, entry="gemm_w", math=1)
         for T in (1, 8, 32, 64):
             run_moe(f"C4 moe bf16 T={T}", "bf16", T, 64, 2048, 1024, 8, 3000 + T)
     elif args.cases == "headline":

@@ -28,6 +28,7 @@ int compute_units();
 int tuned_variant(const char* kernel, int M, int N, int K);
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef int i32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
@@ -209,5 +210,9 @@ __device__ __forceinline__ float weight_element(int type, const void* data, cons
 
 // silu as the reference's CPU computes it (engine/cpu/cpu.h:68), with the device's exp.
 __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
+
+// quant.hip: the launch behind lx_quantize_act, arguments already validated.
+int quantize_act_rows(const void* x, int x_dtype, int64_t ld_x, int math, void* q, int64_t ld_q, float* scale, void* block_scale,
+                      int64_t ld_bs, int M, int K, hipStream_t stream);
 
 }  // namespace dro

@@ -40,6 +40,8 @@ struct GemmArgs {
   int chunks, steps, steps_per_wave, S;
   int64_t row_bytes, scale_row_bytes;
   int tiles_per_wg, x_vecs, x_row_vecs, x_pitch, x_iters;  // the LDS activation image (XL and panel kernels)
+  const int8_t* xq;     // the INT8 math: quantised activations [M, K], rows K bytes apart
+  const float* xscale;  // and their per-row scales
 };
 
 // The epilogue's operation order (engine/cpu/gemm.cpp:21-34); rf is the row factor, b the bias (0 without one).
@@ -281,6 +283,137 @@ __global__ void __launch_bounds__(kPanelThreads) panel_kernel(const GemmArgs a) 
   }
 }
 
+// ---- the INT8 math: int8 weights times per-token quantised activations, exact int32 sums ---------------
+//
+// The weights go into v_mfma_i32_16x16x64_i8 as they are stored (a lane's 16-byte chunk is one operand), so
+// nothing is decoded; the sums are exact, so the K split needs no order. The epilogue is the reference's
+// (engine/cpu/gemm.cpp:21-34): t = (rowscale * xscale) * f32(sum), + bias, * alpha, + beta * y.
+// XL (MT == 1): the activation rows are staged in LDS (rows x_pitch bytes apart, zero from K to the end of the
+// last weight batch), several tiles to a workgroup; otherwise the fragments are read from global memory.
+template <int MT, bool XL>
+__global__ void __launch_bounds__(kMaxSplit* kWave) skinny_i8_kernel(const GemmArgs a) {
+  extern __shared__ __align__(16) f32x4 lds4[];
+  static_assert(!XL || MT == 1, "only one activation tile is staged in LDS");
+  constexpr int kRegion = wave_region_bytes<1, MT>();
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int S = a.S, tile_in_wg = XL ? wave / S : 0, slice = XL ? wave - tile_in_wg * S : wave;
+  const int tile_raw = blockIdx.x * (XL ? a.tiles_per_wg : 1) + tile_in_wg;
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const bool tile_live = tile_raw < n_tiles;
+  const int n0 = min(tile_raw, n_tiles - 1) * kTileRows;
+  const TileRows tiles[1] = {{a.w + n0 * a.row_bytes, a.scale, min(kTileRows, a.N - n0)}};
+  uint8_t* const lds_bytes = reinterpret_cast<uint8_t*>(lds4);
+  uint8_t* const tile_lds = lds_bytes + tile_in_wg * S * kRegion;
+  int8_t* const ximg = reinterpret_cast<int8_t*>(lds_bytes + (blockDim.x / kWave) * kRegion);
+  const int8_t* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = min(mt * 16 + (lane & 15), a.M - 1);
+    xrow[mt] = XL ? ximg + m * a.x_pitch : a.xq + static_cast<int64_t>(m) * a.K;
+  }
+  // The image's rows in 16-byte pieces: slots (row m, pass j) in row-major order, the first four asked for before
+  // the weights.
+  u32x4 xr[4];
+  auto x_piece = [&](int m, int j) {
+    const int v = min(static_cast<int>(threadIdx.x) + j * static_cast<int>(blockDim.x), a.x_vecs - 1);
+    return *reinterpret_cast<const u32x4*>(a.xq + static_cast<int64_t>(min(m, a.M - 1)) * a.K + v * 16);
+  };
+  auto x_store = [&](int m, int j, u32x4 val) {
+    const int v = threadIdx.x + j * blockDim.x;
+    if (v >= a.x_vecs) val = u32x4{0u, 0u, 0u, 0u};
+    if (v < a.x_row_vecs) *reinterpret_cast<u32x4*>(ximg + m * a.x_pitch + v * 16) = val;
+  };
+  if constexpr (XL) {
+    int m = 0, j = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      xr[u] = x_piece(m, j);
+      if (++j == a.x_iters) j = 0, ++m;
+    }
+  }
+  const TileStream<LX_W_INT8, 1> ts(tiles, a.row_bytes, 0, a.chunks, tile_lds + slice * kRegion);
+  WeightBatch<LX_W_INT8, 1> wb;
+  const int t_begin = min(a.steps, slice * a.steps_per_wave), t_end = min(a.steps, t_begin + a.steps_per_wave);
+  if (t_begin < t_end) ts.issue(wb, t_begin);
+  // The epilogue's factors: a lane always finishes the same four weight rows and, per tile, the same activation row.
+  const bool bias_f32 = a.bias && a.bias_dtype == LX_F32;
+  float rf[4], bs[4];
+  {
+    const int nq = n0 + 4 * (lane >> 4);
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = min(nq + r, a.N - 1);
+      rf[r] = reinterpret_cast<const float*>(a.scale)[n];
+      bs[r] = bias_f32 ? static_cast<const float*>(a.bias)[n] : 0.0f;
+    }
+  }
+  if constexpr (XL) {
+    int m = 0, j = 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      if (m < a.M) x_store(m, j, xr[u]);
+      if (++j == a.x_iters) j = 0, ++m;
+    }
+    while (m < a.M) {
+      x_store(m, j, x_piece(m, j));
+      if (++j == a.x_iters) j = 0, ++m;
+    }
+    __syncthreads();
+  }
+  i32x4 acc[1][MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[0][mt] = i32x4{0, 0, 0, 0};
+  const int k_end = min(a.K, 4 * t_end * 16);
+  for (int tb = t_begin; tb < t_end; tb += kLoadsInFlight) {
+    if (tb != t_begin) ts.issue(wb, tb);
+    ts.template consume_i8<MT, XL>(wb, tb, xrow, a.K, k_end, acc);
+  }
+  auto finish = [&](int mt, int q, const i32x4& sum) {
+    const int m = mt * 16 + (q & 15), nq = n0 + 4 * (q >> 4);  // q % 64 == lane: rf and bs are this slot's
+    if (m < a.M && tile_live) {
+      const float xs = a.xscale[m];
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        if (nq + r < a.N)
+          write_out(a, m, nq + r, static_cast<float>(sum[r]), rf[r] * xs,
+                    bias_f32 || !a.bias ? bs[r] : load_as_f32(a.bias, a.bias_dtype, nq + r));
+    }
+  };
+  if (S == 1) {
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) finish(mt, lane, acc[0][mt]);
+    return;
+  }
+  wave_lds_order();
+  i32x4* const mine = reinterpret_cast<i32x4*>(tile_lds + slice * kRegion);
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) mine[mt * kWave + lane] = acc[0][mt];
+  __syncthreads();
+  for (int item = slice * kWave + lane; item < MT * kWave; item += S * kWave) {
+    const int mt = item / kWave, q = item % kWave;
+    i32x4 sum = reinterpret_cast<const i32x4*>(tile_lds)[mt * kWave + q];
+    for (int w = 1; w < S; ++w) sum += reinterpret_cast<const i32x4*>(tile_lds + w * kRegion)[mt * kWave + q];
+    finish(mt, q, sum);
+  }
+}
+
+// Any alignment: one wavefront per output column, lanes striding over k, exact int32 sums.
+__global__ void __launch_bounds__(256) gemm_i8_plain_kernel(const GemmArgs a) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t n = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
+  if (n >= a.N) return;
+  const int8_t* wrow = reinterpret_cast<const int8_t*>(a.w) + n * a.K;
+  for (int m = 0; m < a.M; ++m) {
+    int acc = 0;
+    for (int k = lane; k < a.K; k += kWave) acc += static_cast<int>(a.xq[static_cast<int64_t>(m) * a.K + k]) * static_cast<int>(wrow[k]);
+#pragma unroll
+    for (int off = 1; off < kWave; off <<= 1) acc += __shfl_xor(acc, off);
+    if (lane == 0)
+      write_out(a, m, static_cast<int>(n), static_cast<float>(acc), reinterpret_cast<const float*>(a.scale)[n] * a.xscale[m],
+                a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f);
+  }
+}
+
 // Any shape and alignment: one wavefront per output column, lanes striding over k, activation rows eight at a
 // time. x is rounded to bf16 first when `round_x` (the BF16 math on f32 activations).
 __global__ void __launch_bounds__(256) gemm_plain_kernel(const GemmArgs a, int wtype, int round_x) {
@@ -468,6 +601,105 @@ int gemm_bf16_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w,
   }
 }
 
+// The INT8 math of lx_gemm_w (engine/cpu/gemm.cpp:203-206,231-243): int8 weights only; the activations are
+// quantised per token into the workspace (scales first, rows 64 bytes further, as the reference lays it out).
+int gemm_int8_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w, const void* bias, int bias_dtype, void* y,
+                   int y_dtype, int64_t ld_y, int M, int N, int K, float alpha, float beta, void* workspace, void* stream) {
+  if (M == 0 || N == 0) return kOk;
+  if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(kInvalid);
+  if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype) || (bias && !valid_dtype(bias_dtype))) return fail(kInvalid);
+  if (w.type == LX_W_BF16X) return fail(kNotSupported);
+  if (!x || !y || !valid_weight(&w, K)) return fail(kInvalid);
+  if (w.type != LX_W_INT8) return fail(kNotSupported);
+  hipStream_t s = as_stream(stream);
+  const size_t ws_bytes = static_cast<size_t>((static_cast<int64_t>(M) * 4 + 63) / 64 * 64 + static_cast<int64_t>(M) * K);
+  void* own = nullptr;
+  if (!workspace) {  // the reference falls back to scratch of its own
+    if (hipMallocAsync(&own, ws_bytes, s) != hipSuccess) return fail(kNoMemory);
+    workspace = own;
+  }
+  float* const scales = static_cast<float*>(workspace);
+  int8_t* const q = static_cast<int8_t*>(workspace) + (static_cast<int64_t>(M) * 4 + 63) / 64 * 64;
+  int st = quantize_act_rows(x, x_dtype, ld_x, LX_MATH_INT8, q, K, scales, nullptr, 0, M, K, s);
+  GemmArgs a{};
+  a.w = static_cast<const uint8_t*>(w.data);
+  a.scale = static_cast<const uint8_t*>(w.scale);
+  a.global = 1.0f;
+  a.bias = bias;
+  a.bias_dtype = bias_dtype;
+  a.y_dtype = y_dtype;
+  a.ld_y = ld_y;
+  a.N = N;
+  a.K = K;
+  a.alpha = alpha;
+  a.beta = beta;
+  a.row_bytes = K;
+  const bool aligned = K % 16 == 0 && reinterpret_cast<uintptr_t>(a.w) % 16 == 0 && reinterpret_cast<uintptr_t>(q) % 16 == 0;
+  const int ye = y_dtype == LX_BF16 ? 2 : 4;
+  if (!st && !aligned) {
+    a.M = M;
+    a.xq = q;
+    a.xscale = scales;
+    a.y = y;
+    hipLaunchKernelGGL(gemm_i8_plain_kernel, dim3(static_cast<unsigned>((N + 3) / 4)), dim3(256), 0, s, a);
+    st = status_of(hipGetLastError());
+  } else if (!st) {
+    a.chunks = K / 16;
+    a.steps = load_steps_for<LX_W_INT8>(K);
+    const int S = split_for<LX_W_INT8>(K, 1);
+    a.S = S;
+    a.steps_per_wave = ((a.steps + S - 1) / S + kLoadsInFlight - 1) / kLoadsInFlight * kLoadsInFlight;
+    const unsigned n_tiles = static_cast<unsigned>((N + kTileRows - 1) / kTileRows);
+    for (int m0 = 0; m0 < M && !st; m0 += 64) {
+      a.M = M - m0 < 64 ? M - m0 : 64;
+      a.xq = q + static_cast<int64_t>(m0) * K;
+      a.xscale = scales + m0;
+      a.y = static_cast<char*>(y) + static_cast<int64_t>(m0) * ld_y * ye;
+      auto launch = [&](auto kernel, size_t lds, unsigned grid, unsigned threads) {
+        if (lds > 48 * 1024) {
+          static thread_local bool raised = false;
+          if (!raised) {
+            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax) != hipSuccess)
+              (void)hipGetLastError();
+            raised = true;
+          }
+        }
+        hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, s, a);
+        return status_of(hipGetLastError());
+      };
+      const int mt = (a.M + 15) / 16;
+      if (mt == 1) {
+        // The activation image: rows as long as the last weight batch reaches, zero past K.
+        constexpr int kBatchBytes = kLoadsInFlight * 4 * 16;
+        const int row_bytes = (K + kBatchBytes - 1) / kBatchBytes * kBatchBytes;
+        const size_t image = static_cast<size_t>(a.M) * (row_bytes + 16);
+        int tiles_per_wg = 2 * S <= kMaxSplit && n_tiles >= 512 ? 2 : 1;
+        if (tile_lds_bytes(tiles_per_wg * S, 1, 1) + image > kLdsMax) tiles_per_wg = 1;
+        const size_t lds = tile_lds_bytes(tiles_per_wg * S, 1, 1) + image;
+        if (lds <= kLdsMax) {
+          const unsigned threads = tiles_per_wg * S * kWave;
+          a.tiles_per_wg = tiles_per_wg;
+          a.x_vecs = K / 16;
+          a.x_row_vecs = row_bytes / 16;
+          a.x_pitch = row_bytes + 16;
+          a.x_iters = (a.x_row_vecs + threads - 1) / threads;
+          st = launch(skinny_i8_kernel<1, true>, lds, (n_tiles + tiles_per_wg - 1) / tiles_per_wg, threads);
+          continue;
+        }
+      }
+      const unsigned threads = S * kWave;
+      switch (mt) {
+        case 1: st = launch(skinny_i8_kernel<1, false>, tile_lds_bytes(S, 1, 1), n_tiles, threads); break;
+        case 2: st = launch(skinny_i8_kernel<2, false>, tile_lds_bytes(S, 1, 2), n_tiles, threads); break;
+        case 3: st = launch(skinny_i8_kernel<3, false>, tile_lds_bytes(S, 1, 3), n_tiles, threads); break;
+        default: st = launch(skinny_i8_kernel<4, false>, tile_lds_bytes(S, 1, 4), n_tiles, threads); break;
+      }
+    }
+  }
+  if (own) (void)hipFreeAsync(own, s);
+  return st;
+}
+
 }  // namespace dro
 
 using namespace dro;
@@ -486,10 +718,11 @@ int lx_gemv_w(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, con
 
 int lx_gemm_w(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, lx_math math, const void* bias, lx_dtype bias_dtype,
               void* y, lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* workspace, void* stream) {
-  (void)workspace;  // the BF16 math needs none
   if (!w) return fail(kInvalid);
   if (math != LX_MATH_BF16 && math != LX_MATH_INT8 && math != LX_MATH_FP8 && math != LX_MATH_FP4) return fail(kInvalid);
-  if (math != LX_MATH_BF16) return fail(kNotSupported);
+  if (math == LX_MATH_INT8)
+    return gemm_int8_math(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, workspace, stream);
+  if (math != LX_MATH_BF16) return fail(kNotSupported);  // the BF16 math needs no workspace
   return gemm_bf16_math(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
 }
 

@@ -245,6 +245,18 @@ int quantize_nvfp4(const void* w, lx_weight* out, int64_t rows, int cols, hipStr
 }  // namespace
 }  // namespace dro
 
+namespace dro {
+
+// The launch behind lx_quantize_act (arguments already validated), shared with the INT8 math of lx_gemm_w.
+int quantize_act_rows(const void* x, int x_dtype, int64_t ld_x, int math, void* q, int64_t ld_q, float* scale, void* block_scale,
+                      int64_t ld_bs, int M, int K, hipStream_t stream) {
+  hipLaunchKernelGGL(quantize_act_kernel, dim3(static_cast<unsigned>(M)), dim3(kThreads), 0, stream, x, x_dtype, ld_x, math,
+                     static_cast<uint8_t*>(q), ld_q, scale, static_cast<uint8_t*>(block_scale), ld_bs, K);
+  return status_of(hipGetLastError());
+}
+
+}  // namespace dro
+
 using namespace dro;
 
 extern "C" {
@@ -304,10 +316,7 @@ int lx_quantize_act(const void* x, lx_dtype x_dtype, int ld_x, lx_math math, voi
   } else if (M > 1 && ld_q < K) {
     return fail(kInvalid);
   }
-  hipLaunchKernelGGL(quantize_act_kernel, dim3(static_cast<unsigned>(M)), dim3(kThreads), 0, as_stream(stream), x, static_cast<int>(x_dtype),
-                     static_cast<int64_t>(ld_x), static_cast<int>(math), static_cast<uint8_t*>(q), static_cast<int64_t>(ld_q), scale,
-                     static_cast<uint8_t*>(block_scale), static_cast<int64_t>(ld_bs), K);
-  return status_of(hipGetLastError());
+  return quantize_act_rows(x, x_dtype, ld_x, math, q, ld_q, scale, block_scale, ld_bs, M, K, as_stream(stream));
 }
 
 }  // extern "C"

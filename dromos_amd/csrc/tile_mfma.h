@@ -298,6 +298,54 @@ struct TileStream {
       }
     }
   }
+
+  // The INT8 math on int8 weights: acc[t][mt] += the batch at tb times int8 activation tile mt, exactly, in int32
+  // (v_mfma_i32_16x16x64_i8: a lane's 16-byte chunk of weights against the same 16 k of its activation row).
+  // xrow[mt] points at this lane's int8 activation row; XL says it is an LDS image that is zero past K (and
+  // covers every k asked for), otherwise rows in global memory, clamped and masked at k_end.
+  template <int MT, bool XL>
+  __device__ __forceinline__ void consume_i8(const WeightBatch<F, NT>& wb, int tb, const int8_t* const (&xrow)[MT], int K, int k_end,
+                                             i32x4 (&acc)[NT][MT]) const {
+    static_assert(F == LX_W_INT8, "the INT8 math takes int8 weights");
+    constexpr int U = 4;  // one staging group
+    i32x4 xf[U][MT];
+    auto load_x = [&](int ub) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int k0 = (4 * (tb + ub + u) + g) * 16;
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) xf[u][mt] = *reinterpret_cast<const i32x4*>(xrow[mt] + (XL ? k0 : min(k0, K - 16)));
+      }
+    };
+    if constexpr (!XL) load_x(0);
+#pragma unroll
+    for (int ub = 0; ub < WU; ub += U) {
+      if (!XL && ub > 0) load_x(ub);
+      u32x4 wv[U][NT];
+#pragma unroll
+      for (int n = 0; n < NT; ++n) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) put[q * (4 * kStagePitch / 16)] = wb.raw[ub / 4][n][q];
+        wave_lds_order();
+#pragma unroll
+        for (int sstep = 0; sstep < 4; ++sstep) wv[sstep][n] = get[sstep * 4];
+        wave_lds_order();
+      }
+      if constexpr (XL) load_x(ub);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int k0 = (4 * (tb + ub + u) + g) * 16;
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+#pragma unroll
+          for (int mt = 0; mt < MT; ++mt) {
+            i32x4 xv = xf[u][mt];
+            if (!XL && k0 >= k_end) xv = i32x4{0, 0, 0, 0};
+            acc[n][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, wv[u][n]), xv, acc[n][mt], 0, 0, 0);
+          }
+      }
+    }
+  }
 };
 
 // acc[t][mt] += tile t's rows times activation tile mt over load steps [t_begin, t_end).

@@ -80,8 +80,10 @@ def test_gemm_w_strided_and_untouched_padding(hip):
 def test_other_maths_and_arguments(hip):
     w = random_weight(FORMATS["int8"], 32, 64, 1).to("cuda")
     x = torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda")
-    for math in (MATH_INT8, MATH_FP8, MATH_FP4):
+    for math in (MATH_FP8, MATH_FP4):
         assert ops.gemm_w(hip, x, w, math, status=True) == 801
+    assert ops.gemm_w(hip, x, w, MATH_INT8, status=True) == 0
+    assert ops.gemm_w(hip, x, random_weight(FORMATS["fp8"], 32, 64, 1).to("cuda"), MATH_INT8, status=True) == 801  # int8 weights only
     assert ops.gemm_w(hip, x, w, 7, status=True) == 1
     assert ops.gemm_w(hip, x[:0], w, MATH_BF16, status=True) == 0
     assert ops.gemm_skinny(hip, x.float(), w, status=True) == 801  # bf16 activations only
@@ -143,3 +145,38 @@ def test_baseline_config_against_the_oracle(hip, oracle, fmt, M):
     want = ops.gemm_w(oracle, x, w.to("cpu"), MATH_BF16)
     err = rel_l2(y.cpu(), want)
     assert err <= 1e-2 and err <= 1e-4, err
+
+
+# ---- the INT8 math: exact sums, so every output equals the oracle's bit for bit ---------------------------
+
+
+@pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (5, 300, 4096), (12, 37, 1030), (16, 96, 512), (17, 2048, 1024), (40, 300, 528),
+                                   (64, 1024, 2048), (70, 96, 4096), (130, 50, 1040), (33, 21, 48)])
+def test_int8_math_is_bit_exact(hip, oracle, M, N, K, x_dtype, y_dtype):
+    g = torch.Generator().manual_seed(M * 7 + K)
+    x = torch.randn(M, K, generator=g).to(x_dtype)
+    x[M // 2] = 0
+    w = random_weight(FORMATS["int8"], N, K, M + 3)
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g).to(y_dtype)
+    want = ops.gemm_w(oracle, x, w, MATH_INT8, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    got = ops.gemm_w(hip, x.cuda(), w.to("cuda"), MATH_INT8, bias=bias.cuda(), y=y0.clone().cuda(), alpha=1.25, beta=-0.5)
+    assert torch.equal(got.cpu().view(torch.int16 if y_dtype == torch.bfloat16 else torch.int32),
+                       want.view(torch.int16 if y_dtype == torch.bfloat16 else torch.int32))
+
+
+@pytest.mark.parametrize("M", [1, 16, 64])
+def test_int8_math_baseline_shape(hip, oracle, M):
+    # C2: W 14336 x 4096. Rows of the result do not depend on how many rows ride along (the sums are exact).
+    N, K = 14336, 4096
+    g = torch.Generator().manual_seed(M)
+    x = torch.randn(64, K, generator=g).to(torch.bfloat16)
+    w = random_weight(FORMATS["int8"], N, K, 5)
+    full = ops.gemm_w(hip, x.cuda(), w.to("cuda"), MATH_INT8)
+    part = ops.gemm_w(hip, x[:M].contiguous().cuda(), w.to("cuda"), MATH_INT8)
+    assert torch.equal(part, full[:M])
+    if M == 16:
+        want = ops.gemm_w(oracle, x[:M].contiguous(), w, MATH_INT8)
+        assert torch.equal(part.cpu().view(torch.int32), want.view(torch.int32))

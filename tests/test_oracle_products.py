@@ -77,7 +77,8 @@ def test_gemm_w_bf16_math(oracle, fmt, M):
     y = ops.gemm_w(oracle, x, w, MATH_BF16, bias=bias, alpha=0.5)
     want = ops.gemv_reference(x.to(torch.bfloat16), w.dense(), bias, 0.5, 0.0, None)
     checks.check_product(y, want)
-    assert ops.gemm_w(oracle, x, w, MATH_INT8, status=True) == 801  # outside this path
+    assert ops.gemm_w(oracle, x, w, MATH_INT8, status=True) == (0 if fmt == "int8" else 801)  # int8 weights only
+    assert ops.gemm_w(oracle, x, w, 2, status=True) == 801  # the FP8 and FP4 maths are outside this path
     ys = ops.gemm_skinny(oracle, x.to(torch.bfloat16), w, bias=bias, alpha=0.5)
     assert torch.equal(ys, y)
 
@@ -115,3 +116,45 @@ def test_agrees_with_the_reference_best_level(oracle, ref, fmt):
     x64 = torch.randn(40, 4096, generator=g).to(torch.bfloat16)
     a, b = ops.gemm_w(oracle, x64, w), ops.gemm_w(ref, x64, w)
     assert rel_l2(a, b) < 1e-5
+
+
+def int8_math_reference(x, w, bias, alpha, beta, y0):
+    """The INT8 math from closed forms: the activations by the per-token rule (quantize_act_reference), an exact
+    integer product, and the epilogue's f32 operations in the reference's order (rowscale * xscale) * sum."""
+    from dromos_amd.formats import quantize_act_reference
+
+    q, xs, _ = quantize_act_reference(x, 1)
+    sums = (q.view(torch.int8).double() @ w.data.cpu().double().T).float()  # exact below 2^53, then one rounding to f32
+    t = (w.scale.cpu().float().unsqueeze(0) * xs.float().unsqueeze(1)) * sums
+    if bias is not None:
+        t = t + bias.float()
+    v = alpha * t
+    if beta != 0.0:
+        v = beta * y0.float() + v
+    return v
+
+
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (12, 37, 1030), (40, 300, 528), (70, 96, 4096)])
+def test_gemm_w_int8_math(oracle, M, N, K, x_dtype):
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn(M, K, generator=g).to(x_dtype)
+    x[M // 2] = 0  # a zero row: scale 1, zero sums
+    w = random_weight(FORMATS["int8"], N, K, M + 3)
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g)
+    y = ops.gemm_w(oracle, x, w, MATH_INT8, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    want = int8_math_reference(x, w, bias, 1.25, -0.5, y0)
+    assert torch.equal(y.view(torch.int32), want.view(torch.int32)), "the INT8 math is exact up to the epilogue's f32 operations"
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (12, 37, 1030), (40, 300, 528)])
+def test_int8_math_equals_the_reference_backend(oracle, ref, M, N, K):
+    g = torch.Generator().manual_seed(K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = random_weight(FORMATS["int8"], N, K, K + 1)
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g)
+    a = ops.gemm_w(oracle, x, w, MATH_INT8, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    b = ops.gemm_w(ref, x, w, MATH_INT8, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    assert torch.equal(a.view(torch.int32), b.view(torch.int32))
