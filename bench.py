@@ -309,7 +309,7 @@ def main():
             for M in (1, 4):
                 run_gemv(f"C2 {fmt} M={M} invariant", fmt, M, 14336, 4096, 1000 + M, invariant=True)
         for M in (1, 16, 64):
-            # Not a BASELINE configuration: the low-precision math of the same product (activations quantised per token
+            # Not one of the headline configurations: the low-precision math of the same product (activations quantised per token
             # inside the call, exact int32 sums); the bytes are the weight-only count.
             run_gemv(f"C2 int8 M={M} INT8 math", "int8", M, 14336, 4096, 1000 + M, entry="gemm_w", math=1)
         for T in (1, 8, 32, 64):

@@ -1,5 +1,5 @@
 """GPU parity: the matrix-core products lx_gemm_w (BF16 math) and lx_gemm_skinny through the C ABI, against
-float64 on the decoded values with bf16-rounded activations, against the CPU oracle at the BASELINE shapes, and the
+float64 on the decoded values with bf16-rounded activations, against the CPU oracle at the headline decode shapes, and the
 bitwise invariants: a row's bits do not depend on the batch, and in batch-invariant mode lx_gemv_w and lx_gemm_w
 give the same bits for every row count from 1 up."""
 

@@ -150,7 +150,7 @@ def test_order_class_admission(hip, fmt):
                                        ("fp8", 14336, 4096, 1), ("fp8", 14336, 4096, 4), ("nvfp4", 4096, 14336, 1),
                                        ("nvfp4", 4096, 14336, 8)])
 def test_baseline_configs_against_the_oracle(hip, oracle, fmt, N, K, M):
-    # The BASELINE shapes at full size: N(0, 0.02) bf16 masters, quantised by the library, x ~ N(0, 1) bf16, f32 y.
+    # The headline decode shapes at full size: N(0, 0.02) bf16 masters, quantised by the library, x ~ N(0, 1) bf16, f32 y.
     g = torch.Generator().manual_seed({"bf16": 0, "int8": 1000, "fp8": 1000, "nvfp4": 2000}[fmt] + (0 if fmt == "bf16" else M))
     master = master_weight(N, K, g)
     x = torch.randn(M, K, generator=g).to(torch.bfloat16)

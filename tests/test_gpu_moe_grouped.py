@@ -1,6 +1,6 @@
 """GPU parity: lx_moe_experts_grouped (BF16 math on the matrix cores) and lx_moe_experts through the C ABI, against
 float64 with the bf16-rounded intermediate at the reference tests' shapes (tests/kernels/test_moe_grouped.py:63-70 of
-the reference), against the CPU oracle at the BASELINE shape, and the bitwise invariants (token rows that do not
+the reference), against the CPU oracle at the headline decode shape, and the bitwise invariants (token rows that do not
 depend on the batch, identical bits from run to run out of a garbage-filled workspace)."""
 
 import pytest

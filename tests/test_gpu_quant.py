@@ -58,7 +58,7 @@ def test_dequantize_every_code(hip, oracle):
 
 @pytest.mark.parametrize("fmt", [W_INT8, W_FP8, W_NVFP4])
 def test_baseline_shape_bytes_equal_the_oracle(hip, oracle, fmt):
-    # N(0, 0.02) bf16 masters at a BASELINE-sized row length, quantised on the GPU and by the oracle.
+    # N(0, 0.02) bf16 masters at a decode-sized row length, quantised on the GPU and by the oracle.
     g = torch.Generator().manual_seed(2000 + fmt)
     N, K = (512, 4096) if fmt != W_NVFP4 else (256, 14336)
     w = master_weight(N, K, g)
