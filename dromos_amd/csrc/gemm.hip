@@ -9,6 +9,8 @@
 // reduction-order contract of the skinny GEMM, for every weight format.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "tile_mfma.h"
 
@@ -18,6 +20,8 @@ int gemv_any(const void* x, int x_dtype, int ld_x, const lx_weight& w, const voi
              int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream);
 
 namespace {
+
+constexpr size_t kLdsMax = 160 * 1024;  // LDS a workgroup may take
 
 struct XRows {
   const void* x;
@@ -283,6 +287,205 @@ __global__ void __launch_bounds__(kPanelThreads) panel_kernel(const GemmArgs a) 
   }
 }
 
+// ---- up to 16 activation rows: the lean tile kernel ------------------------------------------------------
+//
+// The same arithmetic as skinny_kernel (one 16 x 16 tile per S wavefronts, contiguous K slices of
+// steps_per_wave steps, each an ascending chain from zero, slices added in ascending order through LDS), written
+// for the registers: a wavefront keeps its eight weight loads, one staging group's fragments, one step's
+// activation fragments and one accumulator, so eight wavefronts fit a SIMD and two 1024-thread workgroups a
+// compute unit. The activation rows sit in LDS behind the wavefronts' staging regions: bf16 (BF16 math: f32
+// activations are rounded on the way in) or the per-token int8 (INT8 math), rows x_pitch bytes apart, zero from K
+// to the end of the last weight batch. MATH: LX_MATH_BF16 (any weight format) or LX_MATH_INT8 (int8 weights).
+template <int F, int MATH, bool XF32>
+__global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_per_eu(8, 8))) tile16_kernel(const GemmArgs a) {
+  extern __shared__ __align__(16) f32x4 lds4[];
+  constexpr bool I8 = MATH == LX_MATH_INT8;
+  constexpr int E = Fmt<F>::kElems, J = I8 ? 1 : E / 8;
+  using Acc = typename std::conditional<I8, i32x4, f32x4>::type;
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int S = a.S, tile_in_wg = wave / S, slice = wave - tile_in_wg * S;
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const int tile_raw = blockIdx.x * a.tiles_per_wg + tile_in_wg;
+  const int n0 = min(tile_raw, n_tiles - 1) * kTileRows;  // a tile past the last repeats it and writes nothing
+  const int valid = min(kTileRows, a.N - n0);
+  const int g = lane >> 4, i = lane & 15;
+  uint8_t* const lds_bytes = reinterpret_cast<uint8_t*>(lds4);
+  uint8_t* const tile_lds = lds_bytes + tile_in_wg * S * kStageBytes;
+  uint8_t* const stage = tile_lds + slice * kStageBytes;
+  uint8_t* const ximg = lds_bytes + (blockDim.x / kWave) * kStageBytes;
+
+  // One 16-byte piece of the image per thread is asked for before the weights; the rest after them.
+  const char* const xsrc = I8 ? reinterpret_cast<const char*>(a.xq) : static_cast<const char*>(a.xs.x);
+  const int64_t x_ld_bytes = I8 ? a.K : a.xs.ld * (XF32 ? 4 : 2);
+  auto x_piece = [&](int m, int v, u32x4 (&r)[XF32 ? 2 : 1]) {
+    const char* src = xsrc + min(m, a.M - 1) * x_ld_bytes + min(v, a.x_vecs - 1) * (XF32 ? 32 : 16);
+    r[0] = *reinterpret_cast<const u32x4*>(src);
+    if constexpr (XF32) r[1] = *reinterpret_cast<const u32x4*>(src + 16);
+  };
+  auto x_store = [&](int m, int v, const u32x4 (&r)[XF32 ? 2 : 1]) {
+    u32x4 val = r[0];
+    if constexpr (XF32) {
+      bf16x2 q[4] = {pack_bf16(__uint_as_float(r[0].x), __uint_as_float(r[0].y)), pack_bf16(__uint_as_float(r[0].z), __uint_as_float(r[0].w)),
+                     pack_bf16(__uint_as_float(r[1].x), __uint_as_float(r[1].y)), pack_bf16(__uint_as_float(r[1].z), __uint_as_float(r[1].w))};
+      val = __builtin_bit_cast(u32x4, q);
+    }
+    if (v >= a.x_vecs) val = u32x4{0u, 0u, 0u, 0u};
+    // No branch around the store (a piece that belongs nowhere goes to a spare slot behind the image): a branch here
+    // makes the wait for x a wait for every load, the weights included.
+    const bool placed = m < a.M && v < a.x_row_vecs;
+    *reinterpret_cast<u32x4*>(placed ? ximg + m * a.x_pitch + v * 16 : ximg + a.M * a.x_pitch) = val;
+  };
+  // Pieces are numbered row by row: piece p is vector p % x_row_vecs of row p / x_row_vecs.
+  u32x4 xr[XF32 ? 2 : 1];
+  const int first_m = threadIdx.x / a.x_row_vecs, first_v = threadIdx.x - first_m * a.x_row_vecs;
+  x_piece(first_m, first_v, xr);
+
+  // This lane's loads: rows 4 q + g of the tile, chunk i of each 4-step group (256 contiguous bytes per 16 lanes).
+  const uint8_t* const tile_w = a.w + static_cast<int64_t>(n0) * a.row_bytes;
+  uint32_t row_off[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) row_off[q] = static_cast<uint32_t>(min(4 * q + g, valid - 1)) * static_cast<uint32_t>(a.row_bytes);
+  const uint8_t* const own_scale = a.scale + (static_cast<int64_t>(n0) + min(i, valid - 1)) * a.scale_row_bytes;  // NVFP4 only
+  const int t_begin = min(a.steps, slice * a.steps_per_wave), t_end = min(a.steps, t_begin + a.steps_per_wave);
+  u32x4 raw[2][4];
+  uint32_t sc[8];
+  auto issue = [&](int tb) {
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp) {
+      const uint32_t c = static_cast<uint32_t>(min(4 * (tb + 4 * grp) + i, a.chunks - 1)) * 16u;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const uint32_t off = row_off[q] + c;  // one 32-bit offset from the tile's (uniform) base
+        raw[grp][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tile_w + off));
+      }
+    }
+    if constexpr (F == LX_W_NVFP4) {
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        sc[u] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale) + min(4 * (tb + u) + g, a.chunks - 1));
+    }
+  };
+  issue(t_begin);  // unconditionally (an empty slice reads clamped addresses): the wait for x can then count past these loads
+
+  x_store(first_m, first_v, xr);
+  for (int v = threadIdx.x + blockDim.x; v < a.M * a.x_row_vecs; v += blockDim.x) {  // the other pieces, if any
+    const int m = v / a.x_row_vecs, vv = v - m * a.x_row_vecs;
+    u32x4 r[XF32 ? 2 : 1];
+    x_piece(m, vv, r);
+    x_store(m, vv, r);
+  }
+  __syncthreads();
+
+  u32x4* const put = reinterpret_cast<u32x4*>(stage + g * kStagePitch + i * 16);
+  const u32x4* const get = reinterpret_cast<const u32x4*>(stage + i * kStagePitch + g * 16);
+  const uint8_t* const xrow = ximg + min(i, a.M - 1) * a.x_pitch + g * (I8 ? 16 : E * 2);  // + step * 4 chunks
+  Acc acc = {0, 0, 0, 0};
+  for (int tb = t_begin; tb < t_end; tb += 8) {
+    if (tb != t_begin) issue(tb);
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) put[q * (4 * kStagePitch / 16)] = raw[grp][q];
+      wave_lds_order();
+      // Two steps' fragments at a time keep the registers of eight wavefronts a SIMD.
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        u32x4 wv[2];
+#pragma unroll
+        for (int st = 0; st < 2; ++st) wv[st] = get[(2 * half + st) * 4];
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          const int step = 4 * grp + 2 * half + st;
+          const uint8_t* xs = xrow + (tb + step) * 4 * (I8 ? 16 : E * 2);
+          if constexpr (I8) {
+            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, wv[st]), *reinterpret_cast<const i32x4*>(xs), acc, 0, 0, 0);
+          } else {
+#pragma unroll
+            for (int j = 0; j < J; ++j)
+              acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(weight_fragment<F>(wv[st], F == LX_W_NVFP4 ? sc[step] : 0u, j),
+                                                            *reinterpret_cast<const bf16x8*>(xs + 16 * j), acc, 0, 0, 0);
+          }
+        }
+      }
+      wave_lds_order();
+    }
+  }
+
+  // The S partial tiles are added in ascending slice order by the tile's first wavefront, which asks for its
+  // epilogue factors before it waits for the others.
+  Acc* const mine = reinterpret_cast<Acc*>(stage);
+  if (S > 1) {
+    wave_lds_order();
+    if (slice != 0) mine[lane] = acc;
+  }
+  float rf[4], bs[4];
+  const int nq = n0 + 4 * g, m = i;
+  const bool bias_f32 = a.bias && a.bias_dtype == LX_F32;
+  if (slice == 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = min(nq + r, a.N - 1);
+      rf[r] = I8 ? reinterpret_cast<const float*>(a.scale)[n] : row_factor(F, a.scale, a.global, n);
+      bs[r] = bias_f32 ? static_cast<const float*>(a.bias)[n] : 0.0f;
+    }
+  }
+  if (S > 1) __syncthreads();
+  if (slice != 0 || m >= a.M || tile_raw >= n_tiles) return;
+  for (int w = 1; w < S; ++w) acc += reinterpret_cast<const Acc*>(tile_lds + w * kStageBytes)[lane];
+  const float xs = I8 ? a.xscale[m] : 1.0f;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    if (nq + r < a.N) {
+      const float b = bias_f32 || !a.bias ? bs[r] : load_as_f32(a.bias, a.bias_dtype, nq + r);
+      if constexpr (I8) write_out(a, m, nq + r, static_cast<float>(acc[r]), rf[r] * xs, b);
+      else write_out(a, m, nq + r, acc[r], rf[r], b);
+    }
+  }
+}
+
+// Launches the lean tile kernel for a.M <= 16 rows when its LDS image fits; false if it does not.
+template <int F, int MATH>
+bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
+  constexpr bool I8 = MATH == LX_MATH_INT8;
+  const int S = a.S;
+  const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
+  // The activation image: rows as long as the last weight batch reaches, zero past K.
+  constexpr int kBatchElems = kLoadsInFlight * 4 * Fmt<F>::kElems;
+  const int row_elems = (a.K + kBatchElems - 1) / kBatchElems * kBatchElems;
+  const int esize = I8 ? 1 : 2;
+  const size_t image = static_cast<size_t>(a.M) * (row_elems * esize + 16) + 16;  // and a spare slot
+  // One or two tiles to a workgroup: whichever lets a compute unit hold more wavefronts.
+  auto waves_per_cu = [&](int tpw) {
+    const size_t need = static_cast<size_t>(tpw) * S * kStageBytes + image;
+    const size_t wgs = need > kLdsMax ? 0 : kLdsMax / need;
+    const size_t by_waves = 32 / (tpw * S);
+    return (wgs < by_waves ? wgs : by_waves) * tpw * S;
+  };
+  int tiles_per_wg = 2 * S <= kMaxSplit && n_tiles >= 512 && waves_per_cu(2) >= waves_per_cu(1) ? 2 : 1;
+  const size_t lds = static_cast<size_t>(tiles_per_wg) * S * kStageBytes + image;
+  if (lds > kLdsMax) return false;
+  a.tiles_per_wg = tiles_per_wg;
+  a.x_vecs = a.K * esize / 16;
+  a.x_row_vecs = row_elems * esize / 16;
+  a.x_pitch = row_elems * esize + 16;
+  const unsigned threads = tiles_per_wg * S * kWave, grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
+  auto launch = [&](auto kernel) {
+    if (lds > 48 * 1024) {
+      static thread_local bool raised = false;
+      if (!raised) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax) != hipSuccess)
+          (void)hipGetLastError();
+        raised = true;
+      }
+    }
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, a);
+    return status_of(hipGetLastError());
+  };
+  if constexpr (I8) *status = launch(tile16_kernel<F, MATH, false>);
+  else *status = a.xs.dtype == LX_F32 ? launch(tile16_kernel<F, MATH, true>) : launch(tile16_kernel<F, MATH, false>);
+  return true;
+}
+
 // ---- the INT8 math: int8 weights times per-token quantised activations, exact int32 sums ---------------
 //
 // The weights go into v_mfma_i32_16x16x64_i8 as they are stored (a lane's 16-byte chunk is one operand), so
@@ -443,8 +646,6 @@ __global__ void __launch_bounds__(256) gemm_plain_kernel(const GemmArgs a, int w
   }
 }
 
-constexpr size_t kLdsMax = 160 * 1024;
-
 template <int F, int MT, bool XF32, bool XL>
 int launch_skinny_x(const GemmArgs& a, size_t lds, unsigned grid, unsigned threads, hipStream_t stream) {
   auto kernel = skinny_kernel<F, MT, XF32, XL>;
@@ -465,6 +666,8 @@ int launch_skinny(GemmArgs a, hipStream_t stream) {
   const int S = a.S;
   const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
   if constexpr (MT == 1) {
+    int st = kOk;
+    if (launch_tile16<F, LX_MATH_BF16>(a, &st, stream)) return st;
     // The activation image: rows as long as the last weight batch reaches, zero past K.
     constexpr int kBatchElems = (kLoadsInFlight / 1) * 4 * Fmt<F>::kElems;
     const int row_elems = (a.K + kBatchElems - 1) / kBatchElems * kBatchElems;
@@ -668,6 +871,7 @@ int gemm_int8_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w,
         return status_of(hipGetLastError());
       };
       const int mt = (a.M + 15) / 16;
+      if (mt == 1 && launch_tile16<LX_W_INT8, LX_MATH_INT8>(a, &st, s)) continue;
       if (mt == 1) {
         // The activation image: rows as long as the last weight batch reaches, zero past K.
         constexpr int kBatchBytes = kLoadsInFlight * 4 * 16;
