@@ -112,6 +112,67 @@ __global__ void __launch_bounds__(kThreads) quantize_act_kernel(const void* __re
   }
 }
 
+// The INT8 / FP8 rules of quantize_act_kernel for rows that can be read 16 bytes at a time and fit a workgroup's
+// registers (K <= 8 * kActVecs * kThreads): every value is read once, eight bf16 or two times four f32 per thread
+// and pass, and eight codes are stored at a time. The same operations on the same values: the same bytes.
+constexpr int kActVecs = 4;
+
+template <bool XF32>
+__global__ void __launch_bounds__(kThreads) quantize_act_rows_kernel(const void* __restrict__ x, int64_t ld_x, int math,
+                                                                     uint8_t* __restrict__ q, int64_t ld_q, float* __restrict__ scale,
+                                                                     int K) {
+  __shared__ float shared[kWaves];
+  const int64_t m = blockIdx.x;
+  const char* const row = static_cast<const char*>(x) + m * ld_x * (XF32 ? 4 : 2);
+  const int vecs = K >> 3;
+  float v[kActVecs][8];
+  float a = 0.0f;
+#pragma unroll
+  for (int u = 0; u < kActVecs; ++u) {
+    const int vi = threadIdx.x + u * kThreads;
+    const int vc = min(vi, vecs - 1);  // clamped: no predicated loads; a piece past the row is not stored
+    if constexpr (XF32) {
+      const f32x4 lo = *reinterpret_cast<const f32x4*>(row + vc * 32), hi = *reinterpret_cast<const f32x4*>(row + vc * 32 + 16);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[u][j] = lo[j];
+        v[u][4 + j] = hi[j];
+      }
+    } else {
+      const u32x4 w = *reinterpret_cast<const u32x4*>(row + vc * 16);
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        v[u][2 * j] = __uint_as_float(w[j] << 16);
+        v[u][2 * j + 1] = __uint_as_float(w[j] & 0xffff0000u);
+      }
+    }
+    if (vi < vecs) {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) a = fmaxf(a, fabsf(v[u][j]));
+    }
+  }
+  a = block_max(a, shared);
+  const float qmax = math == LX_MATH_INT8 ? 127.0f : 448.0f;
+  const float inv = a > 0.0f ? qmax / a : 0.0f;
+  uint8_t* const out = q + m * ld_q;
+#pragma unroll
+  for (int u = 0; u < kActVecs; ++u) {
+    const int vi = threadIdx.x + u * kThreads;
+    if (vi < vecs) {
+      uint32_t packed[2] = {0u, 0u};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float t = v[u][j] * inv;
+        const uint32_t code = math == LX_MATH_INT8 ? static_cast<uint32_t>(static_cast<int>(fminf(fmaxf(rintf(t), -127.0f), 127.0f))) & 0xffu
+                                                   : e4m3_encode(t);
+        packed[j >> 2] |= code << (8 * (j & 3));
+      }
+      *reinterpret_cast<uint2*>(out + vi * 8) = uint2{packed[0], packed[1]};
+    }
+  }
+  if (threadIdx.x == 0) scale[m] = a > 0.0f ? a / qmax : 1.0f;
+}
+
 // One workgroup per row: absmax, then the row's codes. FP8 = false is INT8.
 template <bool FP8>
 __global__ void __launch_bounds__(kThreads) quantize_rows_kernel(const uint16_t* __restrict__ w, uint8_t* __restrict__ q,
@@ -250,8 +311,18 @@ namespace dro {
 // The launch behind lx_quantize_act (arguments already validated), shared with the INT8 math of lx_gemm_w.
 int quantize_act_rows(const void* x, int x_dtype, int64_t ld_x, int math, void* q, int64_t ld_q, float* scale, void* block_scale,
                       int64_t ld_bs, int M, int K, hipStream_t stream) {
-  hipLaunchKernelGGL(quantize_act_kernel, dim3(static_cast<unsigned>(M)), dim3(kThreads), 0, stream, x, x_dtype, ld_x, math,
-                     static_cast<uint8_t*>(q), ld_q, scale, static_cast<uint8_t*>(block_scale), ld_bs, K);
+  const int esize = x_dtype == LX_F32 ? 4 : 2;
+  const bool fast = math != LX_MATH_FP4 && K % 8 == 0 && K <= 8 * kActVecs * kThreads && reinterpret_cast<uintptr_t>(x) % 16 == 0 &&
+                    (ld_x * esize) % 16 == 0 && reinterpret_cast<uintptr_t>(q) % 8 == 0 && ld_q % 8 == 0;
+  if (fast && x_dtype == LX_F32)
+    hipLaunchKernelGGL(quantize_act_rows_kernel<true>, dim3(static_cast<unsigned>(M)), dim3(kThreads), 0, stream, x, ld_x, math,
+                       static_cast<uint8_t*>(q), ld_q, scale, K);
+  else if (fast)
+    hipLaunchKernelGGL(quantize_act_rows_kernel<false>, dim3(static_cast<unsigned>(M)), dim3(kThreads), 0, stream, x, ld_x, math,
+                       static_cast<uint8_t*>(q), ld_q, scale, K);
+  else
+    hipLaunchKernelGGL(quantize_act_kernel, dim3(static_cast<unsigned>(M)), dim3(kThreads), 0, stream, x, x_dtype, ld_x, math,
+                       static_cast<uint8_t*>(q), ld_q, scale, static_cast<uint8_t*>(block_scale), ld_bs, K);
   return status_of(hipGetLastError());
 }
 
