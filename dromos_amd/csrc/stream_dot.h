@@ -204,6 +204,7 @@ __device__ __forceinline__ void stage_x_pairs(uint32_t* xs, const uint16_t* x, i
 struct XRegs {
   static constexpr int kVecs = 4;
   u32x4 v[kVecs];
+  int k_vec;  // vectors that lie inside the row: the rest of the image is zero
   bool ready;
 };
 
@@ -213,14 +214,17 @@ __device__ __forceinline__ void stage_x_load(XRegs& r, const void* x, int x_dtyp
   const int per_row = steps * kWave * E;
   const int vec_shift = x_dtype == LX_BF16 ? 3 : 2;  // elements per 16-byte vector: 8 or 4
   const int n_vec = per_row >> vec_shift, k_vec = static_cast<int>(K) >> vec_shift;
+  r.k_vec = k_vec;
   r.ready = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && ((ld_x << (4 - vec_shift)) & 15) == 0 && (K & 7) == 0 &&
             n_vec <= XRegs::kVecs * static_cast<int>(blockDim.x);
   if (!r.ready) return;
   const u32x4* src = static_cast<const u32x4*>(x);
 #pragma unroll
   for (int u = 0; u < XRegs::kVecs; ++u) {
+    // Clamped, not predicated (a predicated load makes the compiler wait for every load at the next use); what lies
+    // past K is zeroed when it is stored.
     const int v = threadIdx.x + u * blockDim.x;
-    r.v[u] = v < k_vec ? src[v] : u32x4{0u, 0u, 0u, 0u};
+    r.v[u] = src[min(v, k_vec - 1)];
   }
 }
 
@@ -236,14 +240,14 @@ __device__ __forceinline__ void stage_x_store(const XRegs& r, float* xs, int x_d
     if (v < n_vec) {
       const int k = v << vec_shift, s = k / (kWave * E), within = k % (kWave * E);
       float* at = xs + x_slot<F>(s, within / E, within % E);
+      const u32x4 w = v < r.k_vec ? r.v[u] : u32x4{0u, 0u, 0u, 0u};
       if (x_dtype == LX_BF16) {
-        *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(r.v[u].x << 16), __uint_as_float(r.v[u].x & 0xffff0000u),
-                                              __uint_as_float(r.v[u].y << 16), __uint_as_float(r.v[u].y & 0xffff0000u)};
-        *reinterpret_cast<f32x4*>(at + 256) = f32x4{__uint_as_float(r.v[u].z << 16), __uint_as_float(r.v[u].z & 0xffff0000u),
-                                                    __uint_as_float(r.v[u].w << 16), __uint_as_float(r.v[u].w & 0xffff0000u)};
+        *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(w.x << 16), __uint_as_float(w.x & 0xffff0000u),
+                                              __uint_as_float(w.y << 16), __uint_as_float(w.y & 0xffff0000u)};
+        *reinterpret_cast<f32x4*>(at + 256) = f32x4{__uint_as_float(w.z << 16), __uint_as_float(w.z & 0xffff0000u),
+                                                    __uint_as_float(w.w << 16), __uint_as_float(w.w & 0xffff0000u)};
       } else {
-        *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(r.v[u].x), __uint_as_float(r.v[u].y), __uint_as_float(r.v[u].z),
-                                              __uint_as_float(r.v[u].w)};
+        *reinterpret_cast<f32x4*>(at) = f32x4{__uint_as_float(w.x), __uint_as_float(w.y), __uint_as_float(w.z), __uint_as_float(w.w)};
       }
     }
   }
@@ -259,7 +263,7 @@ __device__ __forceinline__ void stage_x_store_pairs(const XRegs& r, uint32_t* xs
     const int v = threadIdx.x + u * blockDim.x;
     if (v < n_vec) {
       const int k = v << 3, st = k / (kWave * E), within = k % (kWave * E);
-      *reinterpret_cast<u32x4*>(xs + x_pair_slot<F>(st, within / E, within % E)) = r.v[u];
+      *reinterpret_cast<u32x4*>(xs + x_pair_slot<F>(st, within / E, within % E)) = v < r.k_vec ? r.v[u] : u32x4{0u, 0u, 0u, 0u};
     }
   }
 }
@@ -321,11 +325,14 @@ struct Chunk {
   uint32_t scales;  // NVFP4: two e4m3 bytes (block of dwords 0-1, block of dwords 2-3)
 };
 
+// The row pointers are the same for every lane of a wavefront; the lane's part is an unsigned 32-bit byte offset, so
+// the load can take the row from scalar registers and the offset from one vector register.
 template <int F>
 __device__ __forceinline__ void load_chunk(Chunk<F>& c, const uint8_t* row, const uint8_t* row_scales, int chunk) {
-  c.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row) + chunk);
+  const uint32_t off = static_cast<uint32_t>(chunk) * 16u;
+  c.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row + off));
   if constexpr (F == LX_W_NVFP4)
-    c.scales = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(row_scales) + chunk);
+    c.scales = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(row_scales + (off >> 3)));
 }
 
 // acc[m] += sum over the chunk's k of x[m, k] * w[k], for MT activation rows; xs points at the LDS image of
