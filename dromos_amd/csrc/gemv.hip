@@ -128,7 +128,10 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs
   };
   if constexpr (MT == 1) {
     // Ask for x, then for the weights, and only then wait for x: loads return in order.
-    XRegs xr;
+    // Vectors of x a thread holds: a one-batch row of U steps is U * kElems / 8 * 64 values / 8 per vector, over at
+    // least 256 threads (a longer row, or f32 activations, may need all four).
+    constexpr int XV = ONE && XB ? (U * Fmt<F>::kElems / 32 < 1 ? 1 : U * Fmt<F>::kElems / 32 > 4 ? 4 : U * Fmt<F>::kElems / 32) : 4;
+    XRegs<XV> xr;
     stage_x_load<F>(xr, a.x, a.x_dtype, a.ld_x, a.K, steps);
     st.prefetch(rows_fn, group, 0, 1);
     if (xr.ready) {

@@ -235,7 +235,7 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
     // Ask for x, then for the weights, and only then wait for x: loads return in order.
     const int token = s_rows ? s_rows[0] : first / a.top_k;
     const uint16_t* xrow = a.latent + static_cast<int64_t>(token) * a.L;
-    XRegs xr;
+    XRegs<4> xr;
     stage_x_load<F>(xr, xrow, LX_BF16, a.L, a.L, steps);
     st.prefetch(rows_fn, i, 0, 1);
     if (xr.ready) stage_x_store_pairs<F>(xr, image, steps);

@@ -201,26 +201,27 @@ __device__ __forceinline__ void stage_x_pairs(uint32_t* xs, const uint16_t* x, i
 // weights, and only then wait for x: XRegs holds a thread's share of the row between the two calls. Usable
 // when the row can be read 16 bytes at a time and a thread's share is at most kVecs vectors; otherwise
 // `ready` is false and the caller falls back to stage_x.
+template <int XV = 4>
 struct XRegs {
-  static constexpr int kVecs = 4;
+  static constexpr int kVecs = XV;  // 16-byte vectors a thread holds: enough for the row, no more (they cost registers)
   u32x4 v[kVecs];
   int k_vec;  // vectors that lie inside the row: the rest of the image is zero
   bool ready;
 };
 
-template <int F>
-__device__ __forceinline__ void stage_x_load(XRegs& r, const void* x, int x_dtype, int64_t ld_x, int64_t K, int steps) {
+template <int F, int XV>
+__device__ __forceinline__ void stage_x_load(XRegs<XV>& r, const void* x, int x_dtype, int64_t ld_x, int64_t K, int steps) {
   constexpr int E = Fmt<F>::kElems;
   const int per_row = steps * kWave * E;
   const int vec_shift = x_dtype == LX_BF16 ? 3 : 2;  // elements per 16-byte vector: 8 or 4
   const int n_vec = per_row >> vec_shift, k_vec = static_cast<int>(K) >> vec_shift;
   r.k_vec = k_vec;
   r.ready = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && ((ld_x << (4 - vec_shift)) & 15) == 0 && (K & 7) == 0 &&
-            n_vec <= XRegs::kVecs * static_cast<int>(blockDim.x);
+            n_vec <= XV * static_cast<int>(blockDim.x);
   if (!r.ready) return;
   const u32x4* src = static_cast<const u32x4*>(x);
 #pragma unroll
-  for (int u = 0; u < XRegs::kVecs; ++u) {
+  for (int u = 0; u < XV; ++u) {
     // Clamped, not predicated (a predicated load makes the compiler wait for every load at the next use); what lies
     // past K is zeroed when it is stored.
     const int v = threadIdx.x + u * blockDim.x;
@@ -228,14 +229,14 @@ __device__ __forceinline__ void stage_x_load(XRegs& r, const void* x, int x_dtyp
   }
 }
 
-template <int F>
-__device__ __forceinline__ void stage_x_store(const XRegs& r, float* xs, int x_dtype, int steps) {
+template <int F, int XV>
+__device__ __forceinline__ void stage_x_store(const XRegs<XV>& r, float* xs, int x_dtype, int steps) {
   constexpr int E = Fmt<F>::kElems;
   const int per_row = steps * kWave * E;
   const int vec_shift = x_dtype == LX_BF16 ? 3 : 2;
   const int n_vec = per_row >> vec_shift;
 #pragma unroll
-  for (int u = 0; u < XRegs::kVecs; ++u) {
+  for (int u = 0; u < XV; ++u) {
     const int v = threadIdx.x + u * blockDim.x;
     if (v < n_vec) {
       const int k = v << vec_shift, s = k / (kWave * E), within = k % (kWave * E);
@@ -254,12 +255,12 @@ __device__ __forceinline__ void stage_x_store(const XRegs& r, float* xs, int x_d
 }
 
 // The second phase for the packed bf16 image (the row is bf16: its vectors go in as they are).
-template <int F>
-__device__ __forceinline__ void stage_x_store_pairs(const XRegs& r, uint32_t* xs, int steps) {
+template <int F, int XV>
+__device__ __forceinline__ void stage_x_store_pairs(const XRegs<XV>& r, uint32_t* xs, int steps) {
   constexpr int E = Fmt<F>::kElems;
   const int n_vec = x_row_words<F, true>(steps) >> 2;
 #pragma unroll
-  for (int u = 0; u < XRegs::kVecs; ++u) {
+  for (int u = 0; u < XV; ++u) {
     const int v = threadIdx.x + u * blockDim.x;
     if (v < n_vec) {
       const int k = v << 3, st = k / (kWave * E), within = k % (kWave * E);
