@@ -235,7 +235,9 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
     // Ask for x, then for the weights, and only then wait for x: loads return in order.
     const int token = s_rows ? s_rows[0] : first / a.top_k;
     const uint16_t* xrow = a.latent + static_cast<int64_t>(token) * a.L;
-    XRegs<4> xr;
+    // Vectors of the latent row a thread holds: what a one-batch row needs over 256 threads, four otherwise.
+    constexpr int XV = ONE ? (U * Fmt<F>::kElems / 32 < 1 ? 1 : U * Fmt<F>::kElems / 32 > 4 ? 4 : U * Fmt<F>::kElems / 32) : 4;
+    XRegs<XV> xr;
     stage_x_load<F>(xr, xrow, LX_BF16, a.L, a.L, steps);
     st.prefetch(rows_fn, i, 0, 1);
     if (xr.ready) stage_x_store_pairs<F>(xr, image, steps);
