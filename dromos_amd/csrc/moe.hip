@@ -254,17 +254,17 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
 // pass's pairs. One token: every slot is its own group and nothing is sorted; more: the groups come from the
 // table decode_sort_kernel wrote.
 // ONE: a row's steps fit one batch of U.
-template <int F, int U, bool ONE>
+// SINGLE: one token (its own kernel: the many-row paths would set the registers of all).
+template <int F, int U, bool ONE, bool SINGLE>
 __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeArgs a, int mt_cap) {
   extern __shared__ __align__(16) float lds[];
-  __shared__ int s_rows[8];
-  const int P = a.T * a.top_k;
-  if (a.T == 1) {
-    if (static_cast<int>(blockIdx.y) >= P) return;
+  if constexpr (SINGLE) {
+    if (static_cast<int>(blockIdx.y) >= a.top_k) return;
     const int e = __builtin_amdgcn_readfirstlane(a.ids[blockIdx.y]);
     gate_up_rows<F, U, 1, ONE>(a, lds, e, blockIdx.y, 1, nullptr, nullptr);
     return;
   }
+  __shared__ int s_rows[8];
   if (static_cast<int>(blockIdx.y) >= a.table[0]) return;
   const int begin = a.table[1 + blockIdx.y], end = a.table[2 + blockIdx.y];
   const int e = a.table[kTableExpert + begin];
@@ -419,7 +419,9 @@ int launch_gate_up_u(const DecodeArgs& a, hipStream_t s) {
     hipLaunchKernelGGL(kernel, dim3((a.I + kWaves - 1) / kWaves, P), dim3(kThreads), lds, s, a, mt_cap);
     return status_of(hipGetLastError());
   };
-  return steps_for<F>(a.L) <= U ? launch(decode_gate_up_kernel<F, U, true>) : launch(decode_gate_up_kernel<F, U, false>);
+  const bool one = steps_for<F>(a.L) <= U;
+  if (a.T == 1) return one ? launch(decode_gate_up_kernel<F, U, true, true>) : launch(decode_gate_up_kernel<F, U, false, true>);
+  return one ? launch(decode_gate_up_kernel<F, U, true, false>) : launch(decode_gate_up_kernel<F, U, false, false>);
 }
 
 template <int F>
