@@ -293,6 +293,33 @@ def main():
         torch.cuda.empty_cache()
         return case
 
+    def run_layer():
+        """C5: the matrix set of one hybrid decode layer at 32 streams in FP8, back to back: four dense products
+        (lx_gemm_w, BF16 math on fp8 weights) and the routed experts (E = 128, top-8, fp8 stacks)."""
+        dense = [("qkv", 6144, 4096), ("o", 4096, 4096), ("in_proj", 16384, 4096), ("out_proj", 4096, 8192)]
+        parts, nbytes, keep = [], 0, []
+        for i, (_, N, K) in enumerate(dense):
+            step, nb, k = make_gemv_case(lx, torch, "fp8", 32, N, K, 5000 + i, "gemm_w")
+            parts.append(step)
+            nbytes += nb
+            keep.append(k)
+        moe_step, moe_bytes, k, distinct = make_moe_case(lx, torch, "fp8", 32, 128, 4096, 1536, 8, 5032, min(K_STEPS + W, 64))
+        keep.append(k)
+        nbytes += moe_bytes
+
+        def step(i):
+            for p in parts:
+                p(i)
+            moe_step(i)
+
+        us = timer.run(step, min(K_STEPS, 50), min(W, 5))
+        gbps = nbytes / us / 1e3
+        cases.append({"case": "C5 fp8 layer, 32 streams", "entry": "4 x lx_gemm_w + lx_moe_route + lx_moe_experts_grouped", "format": "fp8",
+                      "M": 32, "distinct_experts": round(distinct, 2), "us_per_step": round(us, 3), "bytes_per_step": int(nbytes),
+                      "GBps": round(gbps, 1), "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)})
+        del keep
+        torch.cuda.empty_cache()
+
     head = run_gemv("C2 int8 M=1", "int8", 1, 14336, 4096, 1001)
     if args.cases in ("gemv", "all"):
         run_gemv("C1 bf16 M=1", "bf16", 1, 4096, 4096, 0)
@@ -314,6 +341,7 @@ def main():
             run_gemv(f"C2 int8 M={M} INT8 math", "int8", M, 14336, 4096, 1000 + M, entry="gemm_w", math=1)
         for T in (1, 8, 32, 64):
             run_moe(f"C4 moe bf16 T={T}", "bf16", T, 64, 2048, 1024, 8, 3000 + T)
+        run_layer()
     elif args.cases == "headline":
         run_moe("C4 moe bf16 T=1", "bf16", 1, 64, 2048, 1024, 8, 3001)
 
