@@ -14,7 +14,8 @@ ROOT = Path(__file__).resolve().parent.parent
 CSRC = ROOT / "dromos_amd" / "csrc"
 LIB_DIR = ROOT / "dromos_amd" / "lib"
 HIP_LIB = LIB_DIR / "libdromos_hip.so"
-SOURCES = ["runtime.hip", "quant.hip", "gemv.hip", "gemm.hip", "moe.hip", "moe_grouped.hip"]
+SOURCES = ["runtime.hip", "quant.hip", "gemv.hip", "gemv_bf16.hip", "gemv_int8.hip", "gemv_fp8.hip", "gemv_nvfp4.hip", "gemm.hip",
+           "moe.hip", "moe_grouped.hip"]
 
 # -ffp-contract=off: the epilogues and the ordered sums are written as separate multiplies and adds, as the
 # CPU reference computes them; fused operations are spelled __builtin_fmaf where they are meant.
@@ -58,7 +59,7 @@ def build_hip(verbose=False):
         if verbose:
             print(f"compiled {src}", flush=True)
 
-    with ThreadPoolExecutor(max_workers=min(8, len(SOURCES))) as pool:
+    with ThreadPoolExecutor(max_workers=8) as pool:
         list(pool.map(compile_one, zip(SOURCES, objs)))
     _run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", str(HIP_LIB), *map(str, objs)])
     return HIP_LIB
