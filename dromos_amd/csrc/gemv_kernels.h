@@ -229,7 +229,7 @@ int launch_rows(const GemvArgs& a, const Shape& shape, hipStream_t stream) {
   } else {
     switch (shape.depth) {
       case 8: return launch_stream<F, MT, 2, 8, XB>(a, shape, stream);
-      case 4: return launch_stream<F, MT, 4, 4, XB>(a, shape, stream);
+      case 4: return launch_stream<F, MT, 2, 4, XB>(a, shape, stream);
       case 2: return launch_stream<F, MT, 4, 2, XB>(a, shape, stream);
       default: return launch_stream<F, MT, 4, 1, XB>(a, shape, stream);
     }
