@@ -13,7 +13,7 @@ import checks
 import ops
 from conftest import rel_l2
 from dromos_amd.abi import FORMATS, W_BF16, W_INT8, W_NVFP4
-from dromos_amd.formats import master_weight, quantize_with, random_weight
+from dromos_amd.formats import Weight, master_weight, quantize_with, random_weight
 
 pytestmark = pytest.mark.gpu
 FMT = checks.FMT_NAMES
@@ -164,3 +164,24 @@ def test_baseline_configs_against_the_oracle(hip, oracle, fmt, N, K, M):
     # a checksum of checksums against float64 on the decoded values
     ref64 = x.double() @ w_cpu.dense().T
     assert rel_l2(y.cpu(), ref64) <= 1e-4
+
+
+def test_weights_beyond_four_gigabytes(hip):
+    # 70000 x 65536 int8 = 4.59 GB: row offsets past 2^32 bytes. Drawn on the device; checked on rows spread over the
+    # matrix (the last ones lie past the 4 GB mark) against float64 on the same device.
+    N, K = 70000, 65536
+    g = torch.Generator(device="cuda").manual_seed(3)
+    q = torch.randint(-127, 128, (N, K), generator=g, dtype=torch.int8, device="cuda")
+    scale = torch.rand(N, generator=g, device="cuda") * 0.02 + 0.001
+    w = Weight(FORMATS["int8"], q, scale)
+    rows = torch.tensor([0, 1, 32767, 65535, 65536, 69998, 69999], device="cuda")
+    for M, x_dtype in ((1, torch.bfloat16), (3, torch.float32)):
+        x = torch.randn(M, K, generator=g, device="cuda").to(x_dtype)
+        y = ops.gemv_w(hip, x, w)
+        want = (x.double() @ q[rows].double().T) * scale[rows].double()
+        err = (y[:, rows].double() - want).abs().max().item()
+        assert err <= 2e-4 * want.abs().max().item(), (M, err)
+    x16 = torch.randn(16, K, generator=g, device="cuda").to(torch.bfloat16)
+    y16 = ops.gemm_w(hip, x16, w)
+    want = (x16.double() @ q[rows].double().T) * scale[rows].double()
+    assert (y16[:, rows].double() - want).abs().max().item() <= 2e-4 * want.abs().max().item()
