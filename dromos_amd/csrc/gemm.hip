@@ -299,9 +299,9 @@ __global__ void __launch_bounds__(kPanelThreads) panel_kernel(const GemmArgs a) 
 template <int F, int MATH, bool XF32>
 __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_per_eu(8, 8))) tile16_kernel(const GemmArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
-  constexpr bool I8 = MATH == LX_MATH_INT8;
+  constexpr bool I8 = MATH != LX_MATH_BF16;  // byte activations: the INT8 and FP8 maths
   constexpr int E = Fmt<F>::kElems, J = I8 ? 1 : E / 8;
-  using Acc = typename std::conditional<I8, i32x4, f32x4>::type;
+  using Acc = typename std::conditional<MATH == LX_MATH_INT8, i32x4, f32x4>::type;
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int S = a.S, tile_in_wg = wave / S, slice = wave - tile_in_wg * S;
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
@@ -398,7 +398,7 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
           const int step = 4 * grp + 2 * half + st;
           const uint8_t* xs = xrow + (tb + step) * 4 * (I8 ? 16 : E * 2);
           if constexpr (I8) {
-            acc = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, wv[st]), *reinterpret_cast<const i32x4*>(xs), acc, 0, 0, 0);
+            acc = byte_mfma<MATH>(__builtin_bit_cast(i32x4, wv[st]), *reinterpret_cast<const i32x4*>(xs), acc);
           } else {
 #pragma unroll
             for (int j = 0; j < J; ++j)
@@ -437,8 +437,7 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
   for (int r = 0; r < 4; ++r) {
     if (nq + r < a.N) {
       const float b = bias_f32 || !a.bias ? bs[r] : load_as_f32(a.bias, a.bias_dtype, nq + r);
-      if constexpr (I8) write_out(a, m, nq + r, static_cast<float>(acc[r]), rf[r] * xs, b);
-      else write_out(a, m, nq + r, acc[r], rf[r], b);
+      write_out(a, m, nq + r, static_cast<float>(acc[r]), I8 ? rf[r] * xs : rf[r], b);
     }
   }
 }
@@ -446,7 +445,7 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
 // Launches the lean tile kernel for a.M <= 16 rows when its LDS image fits; false if it does not.
 template <int F, int MATH>
 bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
-  constexpr bool I8 = MATH == LX_MATH_INT8;
+  constexpr bool I8 = MATH != LX_MATH_BF16;
   const int S = a.S;
   const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
   // The activation image: rows as long as the last weight batch reaches, zero past K.
@@ -493,8 +492,10 @@ bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
 // (engine/cpu/gemm.cpp:21-34): t = (rowscale * xscale) * f32(sum), + bias, * alpha, + beta * y.
 // XL (MT == 1): the activation rows are staged in LDS (rows x_pitch bytes apart, zero from K to the end of the
 // last weight batch), several tiles to a workgroup; otherwise the fragments are read from global memory.
-template <int MT, bool XL>
+template <int MATH, int MT, bool XL>
 __global__ void __launch_bounds__(kMaxSplit* kWave) skinny_i8_kernel(const GemmArgs a) {
+  constexpr int F = MATH == LX_MATH_INT8 ? LX_W_INT8 : LX_W_FP8;
+  using Acc = typename std::conditional<MATH == LX_MATH_INT8, i32x4, f32x4>::type;
   extern __shared__ __align__(16) f32x4 lds4[];
   static_assert(!XL || MT == 1, "only one activation tile is staged in LDS");
   constexpr int kRegion = wave_region_bytes<1, MT>();
@@ -534,8 +535,8 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) skinny_i8_kernel(const GemmA
       if (++j == a.x_iters) j = 0, ++m;
     }
   }
-  const TileStream<LX_W_INT8, 1> ts(tiles, a.row_bytes, 0, a.chunks, tile_lds + slice * kRegion);
-  WeightBatch<LX_W_INT8, 1> wb;
+  const TileStream<F, 1> ts(tiles, a.row_bytes, 0, a.chunks, tile_lds + slice * kRegion);
+  WeightBatch<F, 1> wb;
   const int t_begin = min(a.steps, slice * a.steps_per_wave), t_end = min(a.steps, t_begin + a.steps_per_wave);
   if (t_begin < t_end) ts.issue(wb, t_begin);
   // The epilogue's factors: a lane always finishes the same four weight rows and, per tile, the same activation row.
@@ -563,15 +564,15 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) skinny_i8_kernel(const GemmA
     }
     __syncthreads();
   }
-  i32x4 acc[1][MT];
+  Acc acc[1][MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) acc[0][mt] = i32x4{0, 0, 0, 0};
+  for (int mt = 0; mt < MT; ++mt) acc[0][mt] = Acc{0, 0, 0, 0};
   const int k_end = min(a.K, 4 * t_end * 16);
   for (int tb = t_begin; tb < t_end; tb += kLoadsInFlight) {
     if (tb != t_begin) ts.issue(wb, tb);
-    ts.template consume_i8<MT, XL>(wb, tb, xrow, a.K, k_end, acc);
+    ts.template consume_bytes<MT, XL, MATH>(wb, tb, xrow, a.K, k_end, acc);
   }
-  auto finish = [&](int mt, int q, const i32x4& sum) {
+  auto finish = [&](int mt, int q, const Acc& sum) {
     const int m = mt * 16 + (q & 15), nq = n0 + 4 * (q >> 4);  // q % 64 == lane: rf and bs are this slot's
     if (m < a.M && tile_live) {
       const float xs = a.xscale[m];
@@ -588,31 +589,42 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) skinny_i8_kernel(const GemmA
     return;
   }
   wave_lds_order();
-  i32x4* const mine = reinterpret_cast<i32x4*>(tile_lds + slice * kRegion);
+  Acc* const mine = reinterpret_cast<Acc*>(tile_lds + slice * kRegion);
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) mine[mt * kWave + lane] = acc[0][mt];
   __syncthreads();
   for (int item = slice * kWave + lane; item < MT * kWave; item += S * kWave) {
     const int mt = item / kWave, q = item % kWave;
-    i32x4 sum = reinterpret_cast<const i32x4*>(tile_lds)[mt * kWave + q];
-    for (int w = 1; w < S; ++w) sum += reinterpret_cast<const i32x4*>(tile_lds + w * kRegion)[mt * kWave + q];
+    Acc sum = reinterpret_cast<const Acc*>(tile_lds)[mt * kWave + q];
+    for (int w = 1; w < S; ++w) sum += reinterpret_cast<const Acc*>(tile_lds + w * kRegion)[mt * kWave + q];
     finish(mt, q, sum);
   }
 }
 
-// Any alignment: one wavefront per output column, lanes striding over k, exact int32 sums.
-__global__ void __launch_bounds__(256) gemm_i8_plain_kernel(const GemmArgs a) {
+// Any alignment: one wavefront per output column, lanes striding over k; exact int32 sums (INT8) or f32 sums of the
+// exact e4m3 products (FP8).
+template <int MATH>
+__global__ void __launch_bounds__(256) gemm_bytes_plain_kernel(const GemmArgs a) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t n = static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave;
   if (n >= a.N) return;
-  const int8_t* wrow = reinterpret_cast<const int8_t*>(a.w) + n * a.K;
+  const uint8_t* wrow = a.w + n * a.K;
   for (int m = 0; m < a.M; ++m) {
-    int acc = 0;
-    for (int k = lane; k < a.K; k += kWave) acc += static_cast<int>(a.xq[static_cast<int64_t>(m) * a.K + k]) * static_cast<int>(wrow[k]);
+    const uint8_t* xrow = reinterpret_cast<const uint8_t*>(a.xq) + static_cast<int64_t>(m) * a.K;
+    float sum;
+    if constexpr (MATH == LX_MATH_INT8) {
+      int acc = 0;
+      for (int k = lane; k < a.K; k += kWave) acc += static_cast<int>(static_cast<int8_t>(xrow[k])) * static_cast<int>(static_cast<int8_t>(wrow[k]));
 #pragma unroll
-    for (int off = 1; off < kWave; off <<= 1) acc += __shfl_xor(acc, off);
+      for (int off = 1; off < kWave; off <<= 1) acc += __shfl_xor(acc, off);
+      sum = static_cast<float>(acc);
+    } else {
+      float acc = 0.0f;
+      for (int k = lane; k < a.K; k += kWave) acc = __builtin_fmaf(e4m3_byte_to_f32<0>(xrow[k]), e4m3_byte_to_f32<0>(wrow[k]), acc);
+      sum = wave_sum(acc);
+    }
     if (lane == 0)
-      write_out(a, m, static_cast<int>(n), static_cast<float>(acc), reinterpret_cast<const float*>(a.scale)[n] * a.xscale[m],
+      write_out(a, m, static_cast<int>(n), sum, reinterpret_cast<const float*>(a.scale)[n] * a.xscale[m],
                 a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f);
   }
 }
@@ -804,16 +816,20 @@ int gemm_bf16_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w,
   }
 }
 
-// The INT8 math of lx_gemm_w (engine/cpu/gemm.cpp:203-206,231-243): int8 weights only; the activations are
-// quantised per token into the workspace (scales first, rows 64 bytes further, as the reference lays it out).
-int gemm_int8_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w, const void* bias, int bias_dtype, void* y,
-                   int y_dtype, int64_t ld_y, int M, int N, int K, float alpha, float beta, void* workspace, void* stream) {
+// The INT8 and FP8 maths of lx_gemm_w (engine/cpu/gemm.cpp:203-209,231-288) on weights of the math's own type (int8,
+// fp8; NVFP4 weights under the FP8 math answer 801 here): the activations are quantised per token into the
+// workspace (scales first, rows 64 bytes further, as the reference lays it out). INT8 sums are exact; FP8 products
+// are exact and summed in f32 (the reference sums them in double: equal to f32 rounding of the sums).
+template <int MATH>
+int gemm_bytes_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w, const void* bias, int bias_dtype, void* y,
+                    int y_dtype, int64_t ld_y, int M, int N, int K, float alpha, float beta, void* workspace, void* stream) {
+  constexpr int F = MATH == LX_MATH_INT8 ? LX_W_INT8 : LX_W_FP8;
   if (M == 0 || N == 0) return kOk;
   if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(kInvalid);
   if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype) || (bias && !valid_dtype(bias_dtype))) return fail(kInvalid);
   if (w.type == LX_W_BF16X) return fail(kNotSupported);
   if (!x || !y || !valid_weight(&w, K)) return fail(kInvalid);
-  if (w.type != LX_W_INT8) return fail(kNotSupported);
+  if (w.type != F) return fail(kNotSupported);
   hipStream_t s = as_stream(stream);
   const size_t ws_bytes = static_cast<size_t>((static_cast<int64_t>(M) * 4 + 63) / 64 * 64 + static_cast<int64_t>(M) * K);
   void* own = nullptr;
@@ -823,7 +839,7 @@ int gemm_int8_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w,
   }
   float* const scales = static_cast<float*>(workspace);
   int8_t* const q = static_cast<int8_t*>(workspace) + (static_cast<int64_t>(M) * 4 + 63) / 64 * 64;
-  int st = quantize_act_rows(x, x_dtype, ld_x, LX_MATH_INT8, q, K, scales, nullptr, 0, M, K, s);
+  int st = quantize_act_rows(x, x_dtype, ld_x, MATH, q, K, scales, nullptr, 0, M, K, s);
   GemmArgs a{};
   a.w = static_cast<const uint8_t*>(w.data);
   a.scale = static_cast<const uint8_t*>(w.scale);
@@ -844,12 +860,12 @@ int gemm_int8_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w,
     a.xq = q;
     a.xscale = scales;
     a.y = y;
-    hipLaunchKernelGGL(gemm_i8_plain_kernel, dim3(static_cast<unsigned>((N + 3) / 4)), dim3(256), 0, s, a);
+    hipLaunchKernelGGL(gemm_bytes_plain_kernel<MATH>, dim3(static_cast<unsigned>((N + 3) / 4)), dim3(256), 0, s, a);
     st = status_of(hipGetLastError());
   } else if (!st) {
     a.chunks = K / 16;
-    a.steps = load_steps_for<LX_W_INT8>(K);
-    const int S = split_for<LX_W_INT8>(K, 1);
+    a.steps = load_steps_for<F>(K);
+    const int S = split_for<F>(K, 1);
     a.S = S;
     a.steps_per_wave = ((a.steps + S - 1) / S + kLoadsInFlight - 1) / kLoadsInFlight * kLoadsInFlight;
     const unsigned n_tiles = static_cast<unsigned>((N + kTileRows - 1) / kTileRows);
@@ -871,7 +887,7 @@ int gemm_int8_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w,
         return status_of(hipGetLastError());
       };
       const int mt = (a.M + 15) / 16;
-      if (mt == 1 && launch_tile16<LX_W_INT8, LX_MATH_INT8>(a, &st, s)) continue;
+      if (mt == 1 && launch_tile16<F, MATH>(a, &st, s)) continue;
       if (mt == 1) {
         // The activation image: rows as long as the last weight batch reaches, zero past K.
         constexpr int kBatchBytes = kLoadsInFlight * 4 * 16;
@@ -887,16 +903,16 @@ int gemm_int8_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w,
           a.x_row_vecs = row_bytes / 16;
           a.x_pitch = row_bytes + 16;
           a.x_iters = (a.x_row_vecs + threads - 1) / threads;
-          st = launch(skinny_i8_kernel<1, true>, lds, (n_tiles + tiles_per_wg - 1) / tiles_per_wg, threads);
+          st = launch(skinny_i8_kernel<MATH, 1, true>, lds, (n_tiles + tiles_per_wg - 1) / tiles_per_wg, threads);
           continue;
         }
       }
       const unsigned threads = S * kWave;
       switch (mt) {
-        case 1: st = launch(skinny_i8_kernel<1, false>, tile_lds_bytes(S, 1, 1), n_tiles, threads); break;
-        case 2: st = launch(skinny_i8_kernel<2, false>, tile_lds_bytes(S, 1, 2), n_tiles, threads); break;
-        case 3: st = launch(skinny_i8_kernel<3, false>, tile_lds_bytes(S, 1, 3), n_tiles, threads); break;
-        default: st = launch(skinny_i8_kernel<4, false>, tile_lds_bytes(S, 1, 4), n_tiles, threads); break;
+        case 1: st = launch(skinny_i8_kernel<MATH, 1, false>, tile_lds_bytes(S, 1, 1), n_tiles, threads); break;
+        case 2: st = launch(skinny_i8_kernel<MATH, 2, false>, tile_lds_bytes(S, 1, 2), n_tiles, threads); break;
+        case 3: st = launch(skinny_i8_kernel<MATH, 3, false>, tile_lds_bytes(S, 1, 3), n_tiles, threads); break;
+        default: st = launch(skinny_i8_kernel<MATH, 4, false>, tile_lds_bytes(S, 1, 4), n_tiles, threads); break;
       }
     }
   }
@@ -925,7 +941,9 @@ int lx_gemm_w(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, lx_
   if (!w) return fail(kInvalid);
   if (math != LX_MATH_BF16 && math != LX_MATH_INT8 && math != LX_MATH_FP8 && math != LX_MATH_FP4) return fail(kInvalid);
   if (math == LX_MATH_INT8)
-    return gemm_int8_math(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, workspace, stream);
+    return gemm_bytes_math<LX_MATH_INT8>(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, workspace, stream);
+  if (math == LX_MATH_FP8)
+    return gemm_bytes_math<LX_MATH_FP8>(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, workspace, stream);
   if (math != LX_MATH_BF16) return fail(kNotSupported);  // the BF16 math needs no workspace
   return gemm_bf16_math(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
 }

@@ -190,6 +190,24 @@ struct WeightBatch {
   uint32_t sc[WU][NT];
 };
 
+// One 16-byte chunk of byte weights against the same 16 k of byte activations, added to acc.
+template <int MATH>
+__device__ __forceinline__ i32x4 byte_mfma(const i32x4& w, const i32x4& x, const i32x4& acc) {
+  static_assert(MATH == LX_MATH_INT8, "int32 sums are the INT8 math's");
+  return __builtin_amdgcn_mfma_i32_16x16x64_i8(w, x, acc, 0, 0, 0);
+}
+
+template <int MATH>
+__device__ __forceinline__ f32x4 byte_mfma(const i32x4& w, const i32x4& x, const f32x4& acc) {
+  static_assert(MATH == LX_MATH_FP8, "f32 sums are the FP8 math's");
+  const long w_lo = (static_cast<long>(static_cast<unsigned>(w.y)) << 32) | static_cast<unsigned>(w.x);
+  const long w_hi = (static_cast<long>(static_cast<unsigned>(w.w)) << 32) | static_cast<unsigned>(w.z);
+  const long x_lo = (static_cast<long>(static_cast<unsigned>(x.y)) << 32) | static_cast<unsigned>(x.x);
+  const long x_hi = (static_cast<long>(static_cast<unsigned>(x.w)) << 32) | static_cast<unsigned>(x.z);
+  const f32x4 half = __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w_lo, x_lo, acc, 0, 0, 0);
+  return __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(w_hi, x_hi, half, 0, 0, 0);
+}
+
 // A wavefront's view of NT tiles of weights: where its loads come from and how they reach fragment order.
 // The weights of a batch are asked for at once, in the order they lie in memory: one load instruction reads 256
 // contiguous bytes of each of four rows (lane -> row 4q + lane / 16, chunk lane % 16 of a 4-step group). They pass
@@ -299,14 +317,16 @@ struct TileStream {
     }
   }
 
-  // The INT8 math on int8 weights: acc[t][mt] += the batch at tb times int8 activation tile mt, exactly, in int32
-  // (v_mfma_i32_16x16x64_i8: a lane's 16-byte chunk of weights against the same 16 k of its activation row).
-  // xrow[mt] points at this lane's int8 activation row; XL says it is an LDS image that is zero past K (and
-  // covers every k asked for), otherwise rows in global memory, clamped and masked at k_end.
-  template <int MT, bool XL>
-  __device__ __forceinline__ void consume_i8(const WeightBatch<F, NT>& wb, int tb, const int8_t* const (&xrow)[MT], int K, int k_end,
-                                             i32x4 (&acc)[NT][MT]) const {
-    static_assert(F == LX_W_INT8, "the INT8 math takes int8 weights");
+  // The quantised maths: weights and per-token quantised activations are one byte a value and go into the matrix
+  // instruction as they are stored. MATH = LX_MATH_INT8 (int8 x int8, exact int32 sums, v_mfma_i32_16x16x64_i8: a
+  // lane's 16-byte chunk against the same 16 k of its activation row) or LX_MATH_FP8 (e4m3 x e4m3, exact products,
+  // f32 sums, v_mfma_f32_16x16x32_fp8_fp8: the chunk's two halves in turn). xrow[mt] points at this lane's activation
+  // row; XL says it is an LDS image that is zero past K (and covers every k asked for), otherwise rows in global
+  // memory, clamped and masked at k_end.
+  template <int MT, bool XL, int MATH, class Acc>
+  __device__ __forceinline__ void consume_bytes(const WeightBatch<F, NT>& wb, int tb, const int8_t* const (&xrow)[MT], int K, int k_end,
+                                                Acc (&acc)[NT][MT]) const {
+    static_assert((MATH == LX_MATH_INT8 && F == LX_W_INT8) || (MATH == LX_MATH_FP8 && F == LX_W_FP8), "one byte a value on both sides");
     constexpr int U = 4;  // one staging group
     i32x4 xf[U][MT];
     auto load_x = [&](int ub) {
@@ -341,7 +361,7 @@ struct TileStream {
           for (int mt = 0; mt < MT; ++mt) {
             i32x4 xv = xf[u][mt];
             if (!XL && k0 >= k_end) xv = i32x4{0, 0, 0, 0};
-            acc[n][mt] = __builtin_amdgcn_mfma_i32_16x16x64_i8(__builtin_bit_cast(i32x4, wv[u][n]), xv, acc[n][mt], 0, 0, 0);
+            acc[n][mt] = byte_mfma<MATH>(__builtin_bit_cast(i32x4, wv[u][n]), xv, acc[n][mt]);
           }
       }
     }

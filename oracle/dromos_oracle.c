@@ -500,6 +500,44 @@ static int gemm_int8_math(const void* x, int x_dtype, int64_t ld_x, const lx_wei
   return ORC_OK;
 }
 
+/* The FP8 math on fp8 weights (engine/cpu/gemm.cpp:207-209,246-288, Epilogue::apply_d :36-50): the activations are
+ * quantised per token to e4m3 (lx_quantize_act's FP8 rule); the products of the two e4m3 values are exact and are
+ * summed in double (exactly: at most 47 significant bits), and t = float(rowscale * xscale * sum) with the product in
+ * double, before bias, alpha and beta in f32. NVFP4 weights under this math answer 801 in this build. Pinned bit for
+ * bit against oracle/_ref (tests/test_oracle_products.py). */
+static int gemm_fp8_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight* w, const void* bias, int bias_dtype,
+                         void* y, int y_dtype, int64_t ld_y, int64_t M, int64_t N, int64_t K, float alpha, float beta) {
+  if (M == 0 || N == 0) return ORC_OK;
+  if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(ORC_INVALID);
+  if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype) || (bias && !dtype_ok(bias_dtype))) return fail(ORC_INVALID);
+  if (!x || !y || !weight_ok(w, K)) return fail(ORC_INVALID);
+  if (w->type != LX_W_FP8) return fail(ORC_UNSUPPORTED);
+  uint8_t* q = (uint8_t*)malloc((size_t)M * (size_t)K);
+  float* xs = (float*)malloc(sizeof(float) * (size_t)M);
+  if (!q || !xs) {
+    free(q);
+    free(xs);
+    return fail(ORC_NOMEM);
+  }
+  for (int64_t m = 0; m < M; ++m) quant_act_row(x, x_dtype, m * ld_x, LX_MATH_FP8, (int)K, q + m * K, xs + m, NULL);
+  const uint8_t* wq = (const uint8_t*)w->data;
+  const float* rs = (const float*)w->scale;
+#pragma omp parallel for schedule(static)
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t m = 0; m < M; ++m) {
+      double sum = 0.0;
+      for (int64_t k = 0; k < K; ++k) sum += (double)orc_e4m3_to_f32(q[m * K + k]) * (double)orc_e4m3_to_f32(wq[n * K + k]);
+      float t = (float)((double)rs[n] * (double)xs[m] * sum);
+      if (bias) t += load_f32(bias, bias_dtype, n);
+      float v = alpha * t;
+      if (beta != 0.0f) v = beta * load_f32(y, y_dtype, m * ld_y + n) + v;
+      store_f32(y, y_dtype, m * ld_y + n, v);
+    }
+  free(q);
+  free(xs);
+  return ORC_OK;
+}
+
 ORC_API int lx_gemm_w(const void* x, int x_dtype, int ld_x, const lx_weight* w, int math, const void* bias, int bias_dtype,
                       void* y, int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* workspace,
                       void* stream) {
@@ -508,6 +546,7 @@ ORC_API int lx_gemm_w(const void* x, int x_dtype, int ld_x, const lx_weight* w, 
   if (!w) return fail(ORC_INVALID);
   if (math < LX_MATH_BF16 || math > LX_MATH_FP4) return fail(ORC_INVALID);
   if (math == LX_MATH_INT8) return gemm_int8_math(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
+  if (math == LX_MATH_FP8) return gemm_fp8_math(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
   if (math != LX_MATH_BF16) return fail(ORC_UNSUPPORTED);
   return gemm_bf16_math(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
 }

@@ -81,7 +81,10 @@ def test_other_maths_and_arguments(hip):
     w = random_weight(FORMATS["int8"], 32, 64, 1).to("cuda")
     x = torch.zeros(4, 64, dtype=torch.bfloat16, device="cuda")
     for math in (MATH_FP8, MATH_FP4):
-        assert ops.gemm_w(hip, x, w, math, status=True) == 801
+        assert ops.gemm_w(hip, x, w, math, status=True) == 801  # int8 weights take the BF16 and INT8 maths
+    w8 = random_weight(FORMATS["fp8"], 32, 64, 1).to("cuda")
+    assert ops.gemm_w(hip, x, w8, MATH_FP8, status=True) == 0
+    assert ops.gemm_w(hip, x, random_weight(FORMATS["nvfp4"], 32, 64, 1).to("cuda"), MATH_FP8, status=True) == 801  # not in this build
     assert ops.gemm_w(hip, x, w, MATH_INT8, status=True) == 0
     assert ops.gemm_w(hip, x, random_weight(FORMATS["fp8"], 32, 64, 1).to("cuda"), MATH_INT8, status=True) == 801  # int8 weights only
     assert ops.gemm_w(hip, x, w, 7, status=True) == 1
@@ -180,3 +183,36 @@ def test_int8_math_baseline_shape(hip, oracle, M):
     if M == 16:
         want = ops.gemm_w(oracle, x[:M].contiguous(), w, MATH_INT8)
         assert torch.equal(part.cpu().view(torch.int32), want.view(torch.int32))
+
+
+# ---- the FP8 math: exact e4m3 products, f32 sums on the device against the oracle's exact sums ------------
+
+
+@pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (5, 300, 4096), (12, 37, 1030), (16, 96, 512), (17, 2048, 1024), (40, 300, 528),
+                                   (64, 1024, 2048), (70, 96, 4096), (130, 50, 1040), (33, 21, 48)])
+def test_fp8_math_against_the_oracle(hip, oracle, M, N, K, x_dtype, y_dtype):
+    g = torch.Generator().manual_seed(M * 7 + K)
+    x = torch.randn(M, K, generator=g).to(x_dtype)
+    x[M // 2] = 0
+    w = random_weight(FORMATS["fp8"], N, K, M + 3)
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g).to(y_dtype)
+    want = ops.gemm_w(oracle, x, w, MATH_FP8, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    got = ops.gemm_w(hip, x.cuda(), w.to("cuda"), MATH_FP8, bias=bias.cuda(), y=y0.clone().cuda(), alpha=1.25, beta=-0.5)
+    # Tolerance of the path: relative L2 of 1e-2 at most; the matrix instruction's f32 sums of the exact products come
+    # out near 1e-5 at K = 4096 (bf16 outputs: one rounding of the result, 2^-9 relative).
+    err = rel_l2(got, want)
+    assert err <= (4e-3 if y_dtype == torch.bfloat16 else 1e-4), err
+
+
+def test_fp8_math_rows_do_not_depend_on_the_batch(hip):
+    N, K = 2048, 4096
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(64, K, generator=g).to(torch.bfloat16).cuda()
+    w = random_weight(FORMATS["fp8"], N, K, 5).to("cuda")
+    full = ops.gemm_w(hip, x, w, MATH_FP8)
+    for M in (1, 7, 16, 33):
+        part = ops.gemm_w(hip, x[:M].contiguous(), w, MATH_FP8)
+        assert torch.equal(part, full[:M]), M

@@ -78,7 +78,8 @@ def test_gemm_w_bf16_math(oracle, fmt, M):
     want = ops.gemv_reference(x.to(torch.bfloat16), w.dense(), bias, 0.5, 0.0, None)
     checks.check_product(y, want)
     assert ops.gemm_w(oracle, x, w, MATH_INT8, status=True) == (0 if fmt == "int8" else 801)  # int8 weights only
-    assert ops.gemm_w(oracle, x, w, 2, status=True) == 801  # the FP8 and FP4 maths are outside this path
+    assert ops.gemm_w(oracle, x, w, 2, status=True) == (0 if fmt == "fp8" else 801)  # fp8 weights only in this build
+    assert ops.gemm_w(oracle, x, w, 3, status=True) == 801  # the FP4 math is outside this path
     ys = ops.gemm_skinny(oracle, x.to(torch.bfloat16), w, bias=bias, alpha=0.5)
     assert torch.equal(ys, y)
 
@@ -157,4 +158,47 @@ def test_int8_math_equals_the_reference_backend(oracle, ref, M, N, K):
     y0 = torch.randn(M, N, generator=g)
     a = ops.gemm_w(oracle, x, w, MATH_INT8, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
     b = ops.gemm_w(ref, x, w, MATH_INT8, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+
+
+def fp8_math_reference(x, w, bias, alpha, beta, y0):
+    """The FP8 math from closed forms: activations by the per-token e4m3 rule, exact products summed in float64 (exactly:
+    the terms span fewer than 53 bits), t = float(rowscale * xscale * sum), then the f32 epilogue."""
+    from dromos_amd.formats import e4m3_table, quantize_act_reference
+
+    q, xs, _ = quantize_act_reference(x, 2)
+    table = e4m3_table()
+    sums = table[q.long()] @ table[w.data.cpu().long()].T
+    t = (w.scale.cpu().double().unsqueeze(0) * xs.double().unsqueeze(1) * sums).float()
+    if bias is not None:
+        t = t + bias.float()
+    v = alpha * t
+    if beta != 0.0:
+        v = beta * y0.float() + v
+    return v
+
+
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (12, 37, 1030), (40, 300, 528)])
+def test_gemm_w_fp8_math(oracle, M, N, K, x_dtype):
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn(M, K, generator=g).to(x_dtype)
+    x[M // 2] = 0
+    w = random_weight(FORMATS["fp8"], N, K, M + 3)
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g)
+    y = ops.gemm_w(oracle, x, w, 2, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    want = fp8_math_reference(x, w, bias, 1.25, -0.5, y0)
+    assert torch.equal(y.view(torch.int32), want.view(torch.int32))
+
+
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (12, 37, 1030), (40, 300, 528)])
+def test_fp8_math_equals_the_reference_backend(oracle, ref, M, N, K):
+    g = torch.Generator().manual_seed(K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = random_weight(FORMATS["fp8"], N, K, K + 1)
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g)
+    a = ops.gemm_w(oracle, x, w, 2, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    b = ops.gemm_w(ref, x, w, 2, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
     assert torch.equal(a.view(torch.int32), b.view(torch.int32))
