@@ -88,6 +88,16 @@ def gemm(lx, fmt):
     return [x, w.data, bias], {"y": y}
 
 
+def gemm_math(lx, fmt, math):
+    M, N, K = 12, 48, 320
+    g = torch.Generator().manual_seed(4550 + math)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = random_weight(FORMATS[fmt], N, K, 4560 + math)
+    bias = torch.randn(N, generator=g)
+    y = ops.gemm_w(lx, x.to(lx.device), w.to(lx.device), math=math, bias=bias.to(lx.device), alpha=1.5)
+    return [x, w.data, bias], {"y_exact" if math == 1 else "y": y}
+
+
 def route(lx):
     T, E, top_k = 5, 64, 8
     g = torch.Generator().manual_seed(4600)
@@ -144,12 +154,14 @@ CASES["gemv_bf16_f32x_f32y"] = (gemv, ("bf16", torch.float32, torch.float32))
 for _m, _n in ((1, "int8"), (2, "fp8"), (3, "fp4")):
     CASES[f"quantize_act_{_n}_bf16"] = (quantize_act, (_m, torch.bfloat16))
 CASES["quantize_act_fp8_f32"] = (quantize_act, (2, torch.float32))
+CASES["gemm_int8_int8math"] = (gemm_math, ("int8", 1))
+CASES["gemm_fp8_fp8math"] = (gemm_math, ("fp8", 2))
 CASES["route"] = (route, ())
 CASES["experts_bf16"] = (experts_bf16, ())
 
 # Outputs whose bits every backend must reproduce (codec and index work); the rest are f32 sums whose last
 # bits depend on the summation order (the reference's own differ between its ISA levels).
-EXACT = {"data", "scale", "global", "dequantized", "ids", "block_scale"}
+EXACT = {"data", "scale", "global", "dequantized", "ids", "block_scale", "y_exact"}  # y_exact: the INT8 math's exact sums
 
 
 def run_case(lx, name):
