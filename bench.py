@@ -339,6 +339,7 @@ def main():
             # Not one of the headline configurations: the low-precision math of the same product (activations quantised per token
             # inside the call, exact int32 sums); the bytes are the weight-only count.
             run_gemv(f"C2 int8 M={M} INT8 math", "int8", M, 14336, 4096, 1000 + M, entry="gemm_w", math=1)
+            run_gemv(f"C2 fp8 M={M} FP8 math", "fp8", M, 14336, 4096, 1000 + M, entry="gemm_w", math=2)
         for T in (1, 8, 32, 64):
             run_moe(f"C4 moe bf16 T={T}", "bf16", T, 64, 2048, 1024, 8, 3000 + T)
         run_layer()
