@@ -296,22 +296,25 @@ __global__ void __launch_bounds__(kPanelThreads) panel_kernel(const GemmArgs a) 
 // compute unit. The activation rows sit in LDS behind the wavefronts' staging regions: bf16 (BF16 math: f32
 // activations are rounded on the way in) or the per-token int8 (INT8 math), rows x_pitch bytes apart, zero from K
 // to the end of the last weight batch. MATH: LX_MATH_BF16 (any weight format) or LX_MATH_INT8 (int8 weights).
-template <int F, int MATH, bool XF32>
-__global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_per_eu(8, 8))) tile16_kernel(const GemmArgs a) {
+// VS: K slices a wavefront takes (1, or 2: the tile then needs half the wavefronts, so a workgroup holds twice the
+// tiles behind one activation image and a compute unit's whole share is in flight at once; both slices' loads are
+// asked for up front and each slice keeps its own sum, so the order of the sums does not change).
+template <int F, int MATH, bool XF32, int VS>
+__global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_per_eu(VS == 1 ? 8 : 4, 8))) tile16_kernel(const GemmArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
   constexpr bool I8 = MATH != LX_MATH_BF16;  // byte activations: the INT8 and FP8 maths
   constexpr int E = Fmt<F>::kElems, J = I8 ? 1 : E / 8;
   using Acc = typename std::conditional<MATH == LX_MATH_INT8, i32x4, f32x4>::type;
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int S = a.S, tile_in_wg = wave / S, slice = wave - tile_in_wg * S;
+  const int S = a.S, waves_per_tile = S / VS, tile_in_wg = wave / waves_per_tile, wave_in_tile = wave - tile_in_wg * waves_per_tile;
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
   const int tile_raw = blockIdx.x * a.tiles_per_wg + tile_in_wg;
   const int n0 = min(tile_raw, n_tiles - 1) * kTileRows;  // a tile past the last repeats it and writes nothing
   const int valid = min(kTileRows, a.N - n0);
   const int g = lane >> 4, i = lane & 15;
   uint8_t* const lds_bytes = reinterpret_cast<uint8_t*>(lds4);
-  uint8_t* const tile_lds = lds_bytes + tile_in_wg * S * kStageBytes;
-  uint8_t* const stage = tile_lds + slice * kStageBytes;
+  uint8_t* const tile_lds = lds_bytes + tile_in_wg * waves_per_tile * kStageBytes;
+  uint8_t* const stage = tile_lds + wave_in_tile * kStageBytes;
   uint8_t* const ximg = lds_bytes + (blockDim.x / kWave) * kStageBytes;
 
   // One 16-byte piece of the image per thread is asked for before the weights; the rest after them.
@@ -346,26 +349,33 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
 #pragma unroll
   for (int q = 0; q < 4; ++q) row_off[q] = static_cast<uint32_t>(min(4 * q + g, valid - 1)) * static_cast<uint32_t>(a.row_bytes);
   const uint8_t* const own_scale = a.scale + (static_cast<int64_t>(n0) + min(i, valid - 1)) * a.scale_row_bytes;  // NVFP4 only
-  const int t_begin = min(a.steps, slice * a.steps_per_wave), t_end = min(a.steps, t_begin + a.steps_per_wave);
-  u32x4 raw[2][4];
-  uint32_t sc[8];
-  auto issue = [&](int tb) {
+  int t_begin[VS], t_end[VS];
+#pragma unroll
+  for (int v = 0; v < VS; ++v) {
+    t_begin[v] = min(a.steps, (wave_in_tile * VS + v) * a.steps_per_wave);
+    t_end[v] = min(a.steps, t_begin[v] + a.steps_per_wave);
+  }
+  u32x4 raw[VS][2][4];
+  uint32_t sc[VS][8];
+  auto issue = [&](int v, int tb) {
 #pragma unroll
     for (int grp = 0; grp < 2; ++grp) {
       const uint32_t c = static_cast<uint32_t>(min(4 * (tb + 4 * grp) + i, a.chunks - 1)) * 16u;
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
         const uint32_t off = row_off[q] + c;  // one 32-bit offset from the tile's (uniform) base
-        raw[grp][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tile_w + off));
+        raw[v][grp][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tile_w + off));
       }
     }
     if constexpr (F == LX_W_NVFP4) {
 #pragma unroll
       for (int u = 0; u < 8; ++u)
-        sc[u] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale) + min(4 * (tb + u) + g, a.chunks - 1));
+        sc[v][u] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale) + min(4 * (tb + u) + g, a.chunks - 1));
     }
   };
-  issue(t_begin);  // unconditionally (an empty slice reads clamped addresses): the wait for x can then count past these loads
+  // Unconditionally (an empty slice reads clamped addresses): the wait for x can then count past these loads.
+#pragma unroll
+  for (int v = 0; v < VS; ++v) issue(v, t_begin[v]);
 
   x_store(first_m, first_v, xr);
   for (int v = threadIdx.x + blockDim.x; v < a.M * a.x_row_vecs; v += blockDim.x) {  // the other pieces, if any
@@ -379,49 +389,54 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
   u32x4* const put = reinterpret_cast<u32x4*>(stage + g * kStagePitch + i * 16);
   const u32x4* const get = reinterpret_cast<const u32x4*>(stage + i * kStagePitch + g * 16);
   const uint8_t* const xrow = ximg + min(i, a.M - 1) * a.x_pitch + g * (I8 ? 16 : E * 2);  // + step * 4 chunks
-  Acc acc = {0, 0, 0, 0};
-  for (int tb = t_begin; tb < t_end; tb += 8) {
-    if (tb != t_begin) issue(tb);
+  Acc acc[VS];
 #pragma unroll
-    for (int grp = 0; grp < 2; ++grp) {
+  for (int v = 0; v < VS; ++v) {
+    acc[v] = Acc{0, 0, 0, 0};
+    for (int tb = t_begin[v]; tb < t_end[v]; tb += 8) {
+      if (tb != t_begin[v]) issue(v, tb);
 #pragma unroll
-      for (int q = 0; q < 4; ++q) put[q * (4 * kStagePitch / 16)] = raw[grp][q];
-      wave_lds_order();
-      // Two steps' fragments at a time keep the registers of eight wavefronts a SIMD.
+      for (int grp = 0; grp < 2; ++grp) {
 #pragma unroll
-      for (int half = 0; half < 2; ++half) {
-        u32x4 wv[2];
+        for (int q = 0; q < 4; ++q) put[q * (4 * kStagePitch / 16)] = raw[v][grp][q];
+        wave_lds_order();
+        // Two steps' fragments at a time keep the registers of eight wavefronts a SIMD.
 #pragma unroll
-        for (int st = 0; st < 2; ++st) wv[st] = get[(2 * half + st) * 4];
+        for (int half = 0; half < 2; ++half) {
+          u32x4 wv[2];
 #pragma unroll
-        for (int st = 0; st < 2; ++st) {
-          const int step = 4 * grp + 2 * half + st;
-          const uint8_t* xs = xrow + (tb + step) * 4 * (I8 ? 16 : E * 2);
-          if constexpr (I8) {
-            acc = byte_mfma<MATH>(__builtin_bit_cast(i32x4, wv[st]), *reinterpret_cast<const i32x4*>(xs), acc);
-          } else {
+          for (int st = 0; st < 2; ++st) wv[st] = get[(2 * half + st) * 4];
 #pragma unroll
-            for (int j = 0; j < J; ++j)
-              acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(weight_fragment<F>(wv[st], F == LX_W_NVFP4 ? sc[step] : 0u, j),
-                                                            *reinterpret_cast<const bf16x8*>(xs + 16 * j), acc, 0, 0, 0);
+          for (int st = 0; st < 2; ++st) {
+            const int step = 4 * grp + 2 * half + st;
+            const uint8_t* xs = xrow + (tb + step) * 4 * (I8 ? 16 : E * 2);
+            if constexpr (I8) {
+              acc[v] = byte_mfma<MATH>(__builtin_bit_cast(i32x4, wv[st]), *reinterpret_cast<const i32x4*>(xs), acc[v]);
+            } else {
+#pragma unroll
+              for (int j = 0; j < J; ++j)
+                acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(weight_fragment<F>(wv[st], F == LX_W_NVFP4 ? sc[v][step] : 0u, j),
+                                                                 *reinterpret_cast<const bf16x8*>(xs + 16 * j), acc[v], 0, 0, 0);
+            }
           }
         }
+        wave_lds_order();
       }
-      wave_lds_order();
     }
   }
 
-  // The S partial tiles are added in ascending slice order by the tile's first wavefront, which asks for its
-  // epilogue factors before it waits for the others.
+  // The S partial tiles (slice s in the region of wavefront s / VS, at s % VS) are added in ascending slice order by
+  // the tile's first wavefront, which asks for its epilogue factors before it waits for the others.
   Acc* const mine = reinterpret_cast<Acc*>(stage);
   if (S > 1) {
     wave_lds_order();
-    if (slice != 0) mine[lane] = acc;
+#pragma unroll
+    for (int v = 0; v < VS; ++v) mine[v * kWave + lane] = acc[v];
   }
   float rf[4], bs[4];
   const int nq = n0 + 4 * g, m = i;
   const bool bias_f32 = a.bias && a.bias_dtype == LX_F32;
-  if (slice == 0) {
+  if (wave_in_tile == 0) {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       const int n = min(nq + r, a.N - 1);
@@ -430,14 +445,15 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
     }
   }
   if (S > 1) __syncthreads();
-  if (slice != 0 || m >= a.M || tile_raw >= n_tiles) return;
-  for (int w = 1; w < S; ++w) acc += reinterpret_cast<const Acc*>(tile_lds + w * kStageBytes)[lane];
+  if (wave_in_tile != 0 || m >= a.M || tile_raw >= n_tiles) return;
+  Acc sum = acc[0];
+  for (int sl = 1; sl < S; ++sl) sum += reinterpret_cast<const Acc*>(tile_lds + (sl / VS) * kStageBytes)[(sl % VS) * kWave + lane];
   const float xs = I8 ? a.xscale[m] : 1.0f;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
     if (nq + r < a.N) {
       const float b = bias_f32 || !a.bias ? bs[r] : load_as_f32(a.bias, a.bias_dtype, nq + r);
-      write_out(a, m, nq + r, static_cast<float>(acc[r]), I8 ? rf[r] * xs : rf[r], b);
+      write_out(a, m, nq + r, static_cast<float>(sum[r]), I8 ? rf[r] * xs : rf[r], b);
     }
   }
 }
@@ -461,13 +477,22 @@ bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
     return (wgs < by_waves ? wgs : by_waves) * tpw * S;
   };
   int tiles_per_wg = 2 * S <= kMaxSplit && n_tiles >= 512 && waves_per_cu(2) >= waves_per_cu(1) ? 2 : 1;
-  const size_t lds = static_cast<size_t>(tiles_per_wg) * S * kStageBytes + image;
+  // Several activation rows: the image takes the LDS a second workgroup would need, so a wavefront takes two slices
+  // (each a single batch) and the workgroup twice the tiles: a compute unit's share is then in flight at once.
+  const bool two_slices = a.M >= 2 && S % 2 == 0 && S >= 4 && a.steps_per_wave == kLoadsInFlight && n_tiles >= 512;
+  if (two_slices) {
+    const int waves_per_tile = S / 2;
+    tiles_per_wg = kMaxSplit / waves_per_tile;
+    while (tiles_per_wg > 1 && static_cast<size_t>(tiles_per_wg) * waves_per_tile * kStageBytes + image > kLdsMax) tiles_per_wg /= 2;
+  }
+  const int waves_per_tile = two_slices ? S / 2 : S;
+  const size_t lds = static_cast<size_t>(tiles_per_wg) * waves_per_tile * kStageBytes + image;
   if (lds > kLdsMax) return false;
   a.tiles_per_wg = tiles_per_wg;
   a.x_vecs = a.K * esize / 16;
   a.x_row_vecs = row_elems * esize / 16;
   a.x_pitch = row_elems * esize + 16;
-  const unsigned threads = tiles_per_wg * S * kWave, grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
+  const unsigned threads = tiles_per_wg * waves_per_tile * kWave, grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
   auto launch = [&](auto kernel) {
     if (lds > 48 * 1024) {
       static thread_local bool raised = false;
@@ -480,8 +505,13 @@ bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, a);
     return status_of(hipGetLastError());
   };
-  if constexpr (I8) *status = launch(tile16_kernel<F, MATH, false>);
-  else *status = a.xs.dtype == LX_F32 ? launch(tile16_kernel<F, MATH, true>) : launch(tile16_kernel<F, MATH, false>);
+  if (two_slices) {
+    if constexpr (I8) *status = launch(tile16_kernel<F, MATH, false, 2>);
+    else *status = a.xs.dtype == LX_F32 ? launch(tile16_kernel<F, MATH, true, 2>) : launch(tile16_kernel<F, MATH, false, 2>);
+    return true;
+  }
+  if constexpr (I8) *status = launch(tile16_kernel<F, MATH, false, 1>);
+  else *status = a.xs.dtype == LX_F32 ? launch(tile16_kernel<F, MATH, true, 1>) : launch(tile16_kernel<F, MATH, false, 1>);
   return true;
 }
 
