@@ -488,6 +488,8 @@ bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
   const int waves_per_tile = two_slices ? S / 2 : S;
   const size_t lds = static_cast<size_t>(tiles_per_wg) * waves_per_tile * kStageBytes + image;
   if (lds > kLdsMax) return false;
+  // Fewer than eight wavefronts on a compute unit cannot keep it fed: the general kernel does better then.
+  if ((kLdsMax / lds) * tiles_per_wg * waves_per_tile < 8) return false;
   a.tiles_per_wg = tiles_per_wg;
   a.x_vecs = a.K * esize / 16;
   a.x_row_vecs = row_elems * esize / 16;
