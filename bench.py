@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Measures the decode matrix-product path on one MI355X: weight-stream GB/s and fraction of the 8 TB/s HBM peak.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cases headline|gemv|all] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cases headline|gemv|all|layer] [--no-cpu]
     python bench.py --pmc-probe      (for rocprofv3 --pmc: a plain copy of known size, then headline launches)
 
 A step is one pass of the hot path over one batch: one lx_gemv_w call (the headline), one skinny GEMM, or one
@@ -230,7 +230,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--cases", default="headline", choices=["headline", "gemv", "all"])
+    ap.add_argument("--cases", default="headline", choices=["headline", "gemv", "all", "layer"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="no timing: one 256 MiB device copy (the counters' yardstick) and 20 eager headline launches")
@@ -345,6 +345,8 @@ def main():
         run_layer()
     elif args.cases == "headline":
         run_moe("C4 moe bf16 T=1", "bf16", 1, 64, 2048, 1024, 8, 3001)
+    elif args.cases == "layer":
+        run_layer()
 
     result = {
         "metric": "weight-stream GB/s and % of HBM peak: M=1 GEMV and top-8 MoE decode",
