@@ -15,7 +15,9 @@
  *   bf16 / e4m3 / e2m1 codecs        pinned: exhaustive tables against torch.float8_e4m3fn and closed forms
  *   lx_quantize_w8 / _weight         pinned: known-answer ties/zero rows + torch IEEE-division references
  *   lx_dequantize_weight             pinned: closed-form dense values from the stored bytes
+ *   lx_quantize_act                  pinned: the per-token rules in torch with IEEE f32 operations, FP4 tie / underflow cases
  *   lx_gemv* / lx_gemm_w / _skinny   pinned: float64 x @ W^T on the decoded values
+ *   lx_gemm_w INT8 / FP8 maths       pinned: exact integer / float64 products of the quantised values, bit for bit
  *   lx_moe_route                     pinned: stable sort of -(logit + bias) + float64 softmax, tie cases
  *   lx_moe_experts*                  pinned: float64 experts with the bf16-rounded intermediate
  */
