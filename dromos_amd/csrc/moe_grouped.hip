@@ -244,7 +244,7 @@ int launch_stage(Kernel kernel, GroupedArgs a, int64_t K, int NT, int out_rows, 
   a.chunks = static_cast<int>(a.row_bytes / 16);
   a.steps = load_steps_for<F>(K);
   int S = split_for<F>(K, NT);
-  if (S > 8) S = 8;  // the partial tiles of eight wavefronts are what LDS holds comfortably at 64 activation rows
+  if (S > 4) S = 4;  // measured: four wavefronts walking a tile in batches beat more wavefronts with one batch each
   a.steps_per_wave = (a.steps + S - 1) / S;
   const int64_t P = static_cast<int64_t>(a.T) * a.top_k;
   const int mt_max = static_cast<int>(((P < kTileTokens ? P : kTileTokens) + 15) / 16);
