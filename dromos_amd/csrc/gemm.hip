@@ -44,6 +44,7 @@ struct GemmArgs {
   int chunks, steps, steps_per_wave, S;
   int64_t row_bytes, scale_row_bytes;
   int tiles_per_wg, x_vecs, x_row_vecs, x_pitch, x_iters;  // the LDS activation image (XL and panel kernels)
+  int x_phased;  // lean kernel with two slices a wavefront: the image holds half of K at a time
   const int8_t* xq;     // the INT8 math: quantised activations [M, K], rows K bytes apart
   const float* xscale;  // and their per-row scales
 };
@@ -296,9 +297,10 @@ __global__ void __launch_bounds__(kPanelThreads) panel_kernel(const GemmArgs a) 
 // compute unit. The activation rows sit in LDS behind the wavefronts' staging regions: bf16 (BF16 math: f32
 // activations are rounded on the way in) or the per-token int8 (INT8 math), rows x_pitch bytes apart, zero from K
 // to the end of the last weight batch. MATH: LX_MATH_BF16 (any weight format) or LX_MATH_INT8 (int8 weights).
-// VS: K slices a wavefront takes (1, or 2: the tile then needs half the wavefronts, so a workgroup holds twice the
-// tiles behind one activation image and a compute unit's whole share is in flight at once; both slices' loads are
-// asked for up front and each slice keeps its own sum, so the order of the sums does not change).
+// VS: K slices a wavefront takes (1, or 2: slice w of the first half of K, then slice w of the second half; the tile
+// then needs half the wavefronts and the image only half of K at a time, so a workgroup holds more tiles behind one
+// image and a compute unit's whole share is in flight at once; both slices' first loads are asked for up front and
+// each slice keeps its own sum, so the order of the sums does not change).
 template <int F, int MATH, bool XF32, int VS>
 __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_per_eu(VS == 1 ? 8 : 4, 8))) tile16_kernel(const GemmArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
@@ -320,19 +322,21 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
   // One 16-byte piece of the image per thread is asked for before the weights; the rest after them.
   const char* const xsrc = I8 ? reinterpret_cast<const char*>(a.xq) : static_cast<const char*>(a.xs.x);
   const int64_t x_ld_bytes = I8 ? a.K : a.xs.ld * (XF32 ? 4 : 2);
-  auto x_piece = [&](int m, int v, u32x4 (&r)[XF32 ? 2 : 1]) {
-    const char* src = xsrc + min(m, a.M - 1) * x_ld_bytes + min(v, a.x_vecs - 1) * (XF32 ? 32 : 16);
+  // The image holds the k range of one phase (VS == 2: the first half of the slices, then the second); `base` is the
+  // phase's first 16-byte piece within a row.
+  auto x_piece = [&](int m, int v, int base, u32x4 (&r)[XF32 ? 2 : 1]) {
+    const char* src = xsrc + min(m, a.M - 1) * x_ld_bytes + min(base + v, a.x_vecs - 1) * (XF32 ? 32 : 16);
     r[0] = *reinterpret_cast<const u32x4*>(src);
     if constexpr (XF32) r[1] = *reinterpret_cast<const u32x4*>(src + 16);
   };
-  auto x_store = [&](int m, int v, const u32x4 (&r)[XF32 ? 2 : 1]) {
+  auto x_store = [&](int m, int v, int base, const u32x4 (&r)[XF32 ? 2 : 1]) {
     u32x4 val = r[0];
     if constexpr (XF32) {
       bf16x2 q[4] = {pack_bf16(__uint_as_float(r[0].x), __uint_as_float(r[0].y)), pack_bf16(__uint_as_float(r[0].z), __uint_as_float(r[0].w)),
                      pack_bf16(__uint_as_float(r[1].x), __uint_as_float(r[1].y)), pack_bf16(__uint_as_float(r[1].z), __uint_as_float(r[1].w))};
       val = __builtin_bit_cast(u32x4, q);
     }
-    if (v >= a.x_vecs) val = u32x4{0u, 0u, 0u, 0u};
+    if (base + v >= a.x_vecs) val = u32x4{0u, 0u, 0u, 0u};
     // No branch around the store (a piece that belongs nowhere goes to a spare slot behind the image): a branch here
     // makes the wait for x a wait for every load, the weights included.
     const bool placed = m < a.M && v < a.x_row_vecs;
@@ -341,7 +345,7 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
   // Pieces are numbered row by row: piece p is vector p % x_row_vecs of row p / x_row_vecs.
   u32x4 xr[XF32 ? 2 : 1];
   const int first_m = threadIdx.x / a.x_row_vecs, first_v = threadIdx.x - first_m * a.x_row_vecs;
-  x_piece(first_m, first_v, xr);
+  x_piece(first_m, first_v, 0, xr);
 
   // This lane's loads: rows 4 q + g of the tile, chunk i of each 4-step group (256 contiguous bytes per 16 lanes).
   const uint8_t* const tile_w = a.w + static_cast<int64_t>(n0) * a.row_bytes;
@@ -352,7 +356,9 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
   int t_begin[VS], t_end[VS];
 #pragma unroll
   for (int v = 0; v < VS; ++v) {
-    t_begin[v] = min(a.steps, (wave_in_tile * VS + v) * a.steps_per_wave);
+    // Phased: slice w of each half of K; otherwise two neighbouring slices.
+    const int slice = a.x_phased ? wave_in_tile + v * waves_per_tile : wave_in_tile * VS + v;
+    t_begin[v] = min(a.steps, slice * a.steps_per_wave);
     t_end[v] = min(a.steps, t_begin[v] + a.steps_per_wave);
   }
   u32x4 raw[VS][2][4];
@@ -377,14 +383,17 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
 #pragma unroll
   for (int v = 0; v < VS; ++v) issue(v, t_begin[v]);
 
-  x_store(first_m, first_v, xr);
-  for (int v = threadIdx.x + blockDim.x; v < a.M * a.x_row_vecs; v += blockDim.x) {  // the other pieces, if any
-    const int m = v / a.x_row_vecs, vv = v - m * a.x_row_vecs;
-    u32x4 r[XF32 ? 2 : 1];
-    x_piece(m, vv, r);
-    x_store(m, vv, r);
-  }
-  __syncthreads();
+  x_store(first_m, first_v, 0, xr);
+  auto stage_image = [&](int base, int first_piece) {
+    for (int v = first_piece; v < a.M * a.x_row_vecs; v += blockDim.x) {
+      const int m = v / a.x_row_vecs, vv = v - m * a.x_row_vecs;
+      u32x4 r[XF32 ? 2 : 1];
+      x_piece(m, vv, base, r);
+      x_store(m, vv, base, r);
+    }
+    __syncthreads();
+  };
+  stage_image(0, threadIdx.x + blockDim.x);  // the other pieces, if any
 
   u32x4* const put = reinterpret_cast<u32x4*>(stage + g * kStagePitch + i * 16);
   const u32x4* const get = reinterpret_cast<const u32x4*>(stage + i * kStagePitch + g * 16);
@@ -393,6 +402,11 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
 #pragma unroll
   for (int v = 0; v < VS; ++v) {
     acc[v] = Acc{0, 0, 0, 0};
+    const int phase_t0 = a.x_phased ? v * waves_per_tile * a.steps_per_wave : 0;  // the image starts at this step's k
+    if (v > 0 && a.x_phased) {
+      __syncthreads();  // every wavefront is done with the first phase's image
+      stage_image(v * a.x_row_vecs, threadIdx.x);
+    }
     for (int tb = t_begin[v]; tb < t_end[v]; tb += 8) {
       if (tb != t_begin[v]) issue(v, tb);
 #pragma unroll
@@ -409,7 +423,7 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
 #pragma unroll
           for (int st = 0; st < 2; ++st) {
             const int step = 4 * grp + 2 * half + st;
-            const uint8_t* xs = xrow + (tb + step) * 4 * (I8 ? 16 : E * 2);
+            const uint8_t* xs = xrow + (tb + step - phase_t0) * 4 * (I8 ? 16 : E * 2);
             if constexpr (I8) {
               acc[v] = byte_mfma<MATH>(__builtin_bit_cast(i32x4, wv[st]), *reinterpret_cast<const i32x4*>(xs), acc[v]);
             } else {
@@ -425,7 +439,7 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
     }
   }
 
-  // The S partial tiles (slice s in the region of wavefront s / VS, at s % VS) are added in ascending slice order by
+  // The S partial tiles (each in the region of the wavefront that made it, at its first or second place) are added in ascending slice order by
   // the tile's first wavefront, which asks for its epilogue factors before it waits for the others.
   Acc* const mine = reinterpret_cast<Acc*>(stage);
   if (S > 1) {
@@ -447,7 +461,10 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
   if (S > 1) __syncthreads();
   if (wave_in_tile != 0 || m >= a.M || tile_raw >= n_tiles) return;
   Acc sum = acc[0];
-  for (int sl = 1; sl < S; ++sl) sum += reinterpret_cast<const Acc*>(tile_lds + (sl / VS) * kStageBytes)[(sl % VS) * kWave + lane];
+  for (int sl = 1; sl < S; ++sl) {
+    const int region = a.x_phased ? sl % waves_per_tile : sl / VS, sub = a.x_phased ? sl / waves_per_tile : sl % VS;
+    sum += reinterpret_cast<const Acc*>(tile_lds + region * kStageBytes)[sub * kWave + lane];
+  }
   const float xs = I8 ? a.xscale[m] : 1.0f;
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
@@ -464,36 +481,41 @@ bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
   constexpr bool I8 = MATH != LX_MATH_BF16;
   const int S = a.S;
   const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
-  // The activation image: rows as long as the last weight batch reaches, zero past K.
-  constexpr int kBatchElems = kLoadsInFlight * 4 * Fmt<F>::kElems;
-  const int row_elems = (a.K + kBatchElems - 1) / kBatchElems * kBatchElems;
+  // The activation image: rows as long as the slices it serves (all of them, or half of them at a time), zero past K.
   const int esize = I8 ? 1 : 2;
-  const size_t image = static_cast<size_t>(a.M) * (row_elems * esize + 16) + 16;  // and a spare slot
-  // One or two tiles to a workgroup: whichever lets a compute unit hold more wavefronts.
-  auto waves_per_cu = [&](int tpw) {
-    const size_t need = static_cast<size_t>(tpw) * S * kStageBytes + image;
-    const size_t wgs = need > kLdsMax ? 0 : kLdsMax / need;
-    const size_t by_waves = 32 / (tpw * S);
-    return (wgs < by_waves ? wgs : by_waves) * tpw * S;
-  };
-  int tiles_per_wg = 2 * S <= kMaxSplit && n_tiles >= 512 && waves_per_cu(2) >= waves_per_cu(1) ? 2 : 1;
-  // Several activation rows: the image takes the LDS a second workgroup would need, so a wavefront takes two slices
-  // (each a single batch) and the workgroup twice the tiles: a compute unit's share is then in flight at once.
-  const bool two_slices = a.M >= 2 && S % 2 == 0 && S >= 4 && a.steps_per_wave == kLoadsInFlight && n_tiles >= 512;
-  if (two_slices) {
-    const int waves_per_tile = S / 2;
-    tiles_per_wg = kMaxSplit / waves_per_tile;
-    while (tiles_per_wg > 1 && static_cast<size_t>(tiles_per_wg) * waves_per_tile * kStageBytes + image > kLdsMax) tiles_per_wg /= 2;
-  }
+  const int step_bytes = 4 * (I8 ? 16 : Fmt<F>::kElems * 2);  // image bytes of one load step
+  // Several activation rows: the image takes the LDS more workgroups would need, so a wavefront takes two slices,
+  // one in each half of K, the image holds half of K at a time and the workgroup more tiles.
+  const bool two_slices = a.M >= 2 && S % 2 == 0 && n_tiles >= 512;
   const int waves_per_tile = two_slices ? S / 2 : S;
-  const size_t lds = static_cast<size_t>(tiles_per_wg) * waves_per_tile * kStageBytes + image;
+  int tiles_per_wg = 1, row_bytes = 0;
+  size_t best = 0, image = 0;
+  auto lds_for = [&](int tpw) { return static_cast<size_t>(tpw) * waves_per_tile * kStageBytes + image; };
+  // The image of all of K if a compute unit then still holds sixteen wavefronts, else (two slices a wavefront) of half
+  // of K at a time, staged twice.
+  for (int phased = 0; phased <= (two_slices ? 1 : 0); ++phased) {
+    row_bytes = (phased ? waves_per_tile : S) * a.steps_per_wave * step_bytes;
+    image = static_cast<size_t>(a.M) * (row_bytes + 16) + 16;  // and a spare slot
+    tiles_per_wg = 1;
+    best = 0;
+    // Tiles to a workgroup: whichever lets a compute unit hold most wavefronts.
+    for (int tpw = 1; tpw * waves_per_tile <= kMaxSplit; tpw *= 2) {
+      if (lds_for(tpw) > kLdsMax || (tpw > 1 && n_tiles < 512)) break;
+      const size_t by_lds = kLdsMax / lds_for(tpw), by_waves = 32 / (tpw * waves_per_tile);
+      const size_t waves = (by_lds < by_waves ? by_lds : by_waves) * tpw * waves_per_tile;
+      if (waves >= best) best = waves, tiles_per_wg = tpw;
+    }
+    a.x_phased = phased;
+    if (best >= 16) break;
+  }
+  const size_t lds = lds_for(tiles_per_wg);
   if (lds > kLdsMax) return false;
   // Fewer than eight wavefronts on a compute unit cannot keep it fed: the general kernel does better then.
-  if ((kLdsMax / lds) * tiles_per_wg * waves_per_tile < 8) return false;
+  if (best < 8) return false;
   a.tiles_per_wg = tiles_per_wg;
   a.x_vecs = a.K * esize / 16;
-  a.x_row_vecs = row_elems * esize / 16;
-  a.x_pitch = row_elems * esize + 16;
+  a.x_row_vecs = row_bytes / 16;
+  a.x_pitch = row_bytes + 16;
   const unsigned threads = tiles_per_wg * waves_per_tile * kWave, grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
   auto launch = [&](auto kernel) {
     if (lds > 48 * 1024) {
