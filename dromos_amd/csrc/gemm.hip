@@ -302,7 +302,7 @@ __global__ void __launch_bounds__(kPanelThreads) panel_kernel(const GemmArgs a) 
 // image and a compute unit's whole share is in flight at once; both slices' first loads are asked for up front and
 // each slice keeps its own sum, so the order of the sums does not change).
 template <int F, int MATH, bool XF32, int VS>
-__global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_per_eu(VS == 1 ? 8 : 4, 8))) tile16_kernel(const GemmArgs a) {
+__global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_per_eu(VS == 2 ? 4 : F == LX_W_NVFP4 ? 6 : 8, 8))) tile16_kernel(const GemmArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
   constexpr bool I8 = MATH != LX_MATH_BF16;  // byte activations: the INT8 and FP8 maths
   constexpr int E = Fmt<F>::kElems, J = I8 ? 1 : E / 8;
@@ -363,21 +363,23 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
   }
   u32x4 raw[VS][2][4];
   uint32_t sc[VS][8];
-  auto issue = [&](int v, int tb) {
+  // Asks for one 4-step group of a batch (grp 0 or 1 of the batch at step tb) of slice v.
+  auto issue_group = [&](int v, int tb, int grp) {
+    const uint32_t c = static_cast<uint32_t>(min(4 * (tb + 4 * grp) + i, a.chunks - 1)) * 16u;
 #pragma unroll
-    for (int grp = 0; grp < 2; ++grp) {
-      const uint32_t c = static_cast<uint32_t>(min(4 * (tb + 4 * grp) + i, a.chunks - 1)) * 16u;
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const uint32_t off = row_off[q] + c;  // one 32-bit offset from the tile's (uniform) base
-        raw[v][grp][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tile_w + off));
-      }
+    for (int q = 0; q < 4; ++q) {
+      const uint32_t off = row_off[q] + c;  // one 32-bit offset from the tile's (uniform) base
+      raw[v][grp][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tile_w + off));
     }
     if constexpr (F == LX_W_NVFP4) {
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        sc[v][u] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale) + min(4 * (tb + u) + g, a.chunks - 1));
+      for (int u = 0; u < 4; ++u)
+        sc[v][4 * grp + u] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale) + min(4 * (tb + 4 * grp + u) + g, a.chunks - 1));
     }
+  };
+  auto issue = [&](int v, int tb) {
+    issue_group(v, tb, 0);
+    issue_group(v, tb, 1);
   };
   // Unconditionally (an empty slice reads clamped addresses): the wait for x can then count past these loads.
 #pragma unroll
@@ -408,11 +410,16 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
       stage_image(v * a.x_row_vecs, threadIdx.x);
     }
     for (int tb = t_begin[v]; tb < t_end[v]; tb += 8) {
-      if (tb != t_begin[v]) issue(v, tb);
 #pragma unroll
       for (int grp = 0; grp < 2; ++grp) {
+        uint32_t scales[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) scales[u] = F == LX_W_NVFP4 ? sc[v][4 * grp + u] : 0u;
 #pragma unroll
         for (int q = 0; q < 4; ++q) put[q * (4 * kStagePitch / 16)] = raw[v][grp][q];
+        // The group's registers are free: ask for the same group of the slice's next batch, so a wavefront that
+        // walks a long slice always has a batch in flight.
+        if (tb + 8 < t_end[v]) issue_group(v, tb + 8, grp);
         wave_lds_order();
         // Two steps' fragments at a time keep the registers of eight wavefronts a SIMD.
 #pragma unroll
@@ -429,7 +436,7 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
             } else {
 #pragma unroll
               for (int j = 0; j < J; ++j)
-                acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(weight_fragment<F>(wv[st], F == LX_W_NVFP4 ? sc[v][step] : 0u, j),
+                acc[v] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(weight_fragment<F>(wv[st], scales[2 * half + st], j),
                                                                  *reinterpret_cast<const bf16x8*>(xs + 16 * j), acc[v], 0, 0, 0);
             }
           }
@@ -486,7 +493,9 @@ bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
   const int step_bytes = 4 * (I8 ? 16 : Fmt<F>::kElems * 2);  // image bytes of one load step
   // Several activation rows: the image takes the LDS more workgroups would need, so a wavefront takes two slices,
   // one in each half of K, the image holds half of K at a time and the workgroup more tiles.
-  const bool two_slices = a.M >= 2 && S % 2 == 0 && n_tiles >= 512;
+  // (With slices of several batches and few rows the image is small and one slice a wavefront keeps more wavefronts
+  // busy.)
+  const bool two_slices = a.M >= 2 && S % 2 == 0 && n_tiles >= 512 && (a.steps_per_wave == kLoadsInFlight || a.M > 4);
   const int waves_per_tile = two_slices ? S / 2 : S;
   int tiles_per_wg = 1, row_bytes = 0;
   size_t best = 0, image = 0;
@@ -800,7 +809,7 @@ int launch_format(GemmArgs a, const char* x0, char* y0, int M, int x_esize, int 
   a.scale_row_bytes = F == LX_W_NVFP4 ? a.K / 16 : 0;
   a.chunks = static_cast<int>(rb / 16);
   a.steps = load_steps_for<F>(a.K);
-  int S = split_for<F>(a.K, 1);
+  int S = split_for_shape<F>(a.K, a.N);
   // Slices are whole weight batches (the row's last one may be cut short by the row's end).
   a.steps_per_wave = ((a.steps + S - 1) / S + kLoadsInFlight - 1) / kLoadsInFlight * kLoadsInFlight;
   a.S = S;
@@ -919,7 +928,7 @@ int gemm_bytes_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w
   } else if (!st) {
     a.chunks = K / 16;
     a.steps = load_steps_for<F>(K);
-    const int S = split_for<F>(K, 1);
+    const int S = split_for_shape<F>(K, N);
     a.S = S;
     a.steps_per_wave = ((a.steps + S - 1) / S + kLoadsInFlight - 1) / kLoadsInFlight * kLoadsInFlight;
     const unsigned n_tiles = static_cast<unsigned>((N + kTileRows - 1) / kTileRows);

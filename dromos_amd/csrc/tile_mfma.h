@@ -46,6 +46,18 @@ inline int split_for(int64_t K, int NT) {
   return S;
 }
 
+// The K split of a dense product of N rows: the split by K alone gives every wavefront one batch; with many tiles
+// fewer, longer slices do better (measured on MI355X: about 2500 wavefronts in all, each walking its slice in
+// batches). A function of (F, K, N) only, never of M, so a row's bits do not depend on the batch.
+template <int F>
+inline int split_for_shape(int64_t K, int64_t N) {
+  const int by_k = split_for<F>(K, 1);
+  const double want = 2560.0 / static_cast<double>((N + kTileRows - 1) / kTileRows);
+  int S = 1;
+  while (S < kMaxSplit && static_cast<double>(S) * 1.4142135623730951 <= want) S *= 2;  // nearest power of two, ties up
+  return S < by_k ? S : by_k;
+}
+
 // Eight consecutive values of a lane's 16 bytes as the A operand: instruction j of the load step.
 template <int F>
 __device__ __forceinline__ bf16x8 weight_fragment(const u32x4& w, uint32_t scales, int j);
