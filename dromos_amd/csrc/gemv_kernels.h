@@ -273,7 +273,8 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
     a.x = x0 + m0 * x_row;
     a.y = y0 + m0 * y_row;
     const int mt = a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : 8;
-    const Shape shape = shape_for(F, steps);
+    Shape shape = shape_for(F, steps);
+    if (mt >= 2) shape.threads = 512;  // several activation rows: more wavefronts behind one image
     int st;
     switch (mt) {
       case 1: st = xb ? launch_rows<F, 1, true>(a, shape, stream) : launch_rows<F, 1, false>(a, shape, stream); break;
