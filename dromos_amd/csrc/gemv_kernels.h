@@ -12,7 +12,7 @@ namespace dro {
 constexpr int kThreads = 256;  // the plain kernel's workgroup
 constexpr int kMaxThreads = 512;  // the streaming kernel's workgroup is chosen per launch, up to this
 constexpr int kMaxWaves = kMaxThreads / kWave;
-constexpr int kLdsFloats = 32 * 1024;  // 128 KB of x at most: one workgroup per compute unit then
+constexpr int kLdsFloats = 38 * 1024;  // 152 KB of x at most: one workgroup per compute unit then
 
 struct GemvArgs {
   const void* x;
@@ -37,6 +37,7 @@ struct GemvArgs {
   int chunks;          // 16-byte chunks in a row
   int64_t row_bytes;
   int64_t scale_row_bytes;  // NVFP4: bytes of block scales per row
+  int phase_steps;  // > 0: the activation image holds this many steps at a time (two images in turn), else all
 };
 
 namespace {
@@ -61,7 +62,7 @@ template <int F, int MT, int R, int U, bool XB, bool ONE>
 __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs a) {
   extern __shared__ __align__(16) float lds[];
   const int steps = a.steps;
-  const int per_row = x_row_words<F, XB>(steps);
+  const int per_row = x_row_words<F, XB>(a.phase_steps > 0 ? a.phase_steps : steps);
   float* xs = lds;
   float* partial = lds + MT * per_row;  // [waves][MT * R] when S > 1
 
@@ -136,6 +137,22 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs
     }
   } else {
     st.prefetch(rows_fn, group, 0, 1);
+    if constexpr (XB && ONE) {
+      if (a.phase_steps > 0) {
+        // Long rows and several activation rows: the image holds half of K at a time.
+        const int64_t phase_k = static_cast<int64_t>(a.phase_steps) * kWave * Fmt<F>::kElems;
+        const uint16_t* x16 = static_cast<const uint16_t*>(a.x);
+        uint32_t* image = reinterpret_cast<uint32_t*>(xs);
+        stage_x_pairs<F, MT>(image, x16, a.ld_x, nullptr, a.M, a.K < phase_k ? a.K : phase_k, a.phase_steps);
+        __syncthreads();
+        st.run_two_images(rows_fn, done_fn, group, a.phase_steps, [&] {
+          __syncthreads();
+          stage_x_pairs<F, MT>(image, x16 + phase_k, a.ld_x, nullptr, a.M, a.K > phase_k ? a.K - phase_k : 0, a.phase_steps);
+          __syncthreads();
+        });
+        return;
+      }
+    }
     stage_all();
   }
   __syncthreads();
@@ -192,7 +209,7 @@ Shape shape_for(int wtype, int steps) {
 template <int F, int MT, int R, int U, bool XB>
 int launch_stream(GemvArgs a, const Shape& shape, hipStream_t stream) {
   const int waves = shape.threads / kWave;
-  const size_t lds = sizeof(float) * (static_cast<size_t>(MT) * x_row_words<F, XB>(a.steps) + waves * MT * R);
+  const size_t lds = sizeof(float) * (static_cast<size_t>(MT) * x_row_words<F, XB>(a.phase_steps > 0 ? a.phase_steps : a.steps) + waves * MT * R);
   const int groups_per_wg = waves / a.split;
   const int64_t n_groups = (a.N + R - 1) / R;
   const int64_t grid = (n_groups + groups_per_wg - 1) / groups_per_wg;
@@ -249,6 +266,19 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
   const int64_t row_words = xb ? x_row_words<F, true>(steps) : x_row_words<F, false>(steps);
   int fit = 8;
   while (fit >= 1 && fit * row_words + kMaxWaves * fit * 4 > kLdsFloats) fit /= 2;
+  // Rows too long for the call's activation rows to share one image: two images in turn, each half of K (bf16
+  // activations, a row's steps in one batch, no K split), rather than a second pass over the weights.
+  a.phase_steps = 0;
+  if (xb && vector_rows && fit >= 1 && fit < (a.M <= 8 ? a.M : 8) && steps >= 2 && steps <= 8 && batch_depth(steps, 8) >= steps &&
+      (a.K * 2) % 16 == 0 && reinterpret_cast<uintptr_t>(a.x) % 16 == 0 && (a.ld_x * 2) % 16 == 0) {
+    const int half = (steps + 1) / 2;
+    int fit_half = 8;
+    while (fit_half >= 1 && fit_half * static_cast<int64_t>(x_row_words<F, true>(half)) + kMaxWaves * fit_half * 4 > kLdsFloats) fit_half /= 2;
+    if (fit_half > fit && order_class<F>(a.N, a.K, R) == 1) {
+      fit = fit_half;
+      a.phase_steps = half;
+    }
+  }
   if (!vector_rows || fit < 1) {
     const int waves = kThreads / kWave;
     const unsigned grid = static_cast<unsigned>((a.N + waves - 1) / waves);
@@ -257,7 +287,7 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
   }
   a.split = order_class<F>(a.N, a.K, R);
   const int tuned = tuned_variant(kernel_name, a.M, a.N, static_cast<int>(a.K));
-  if (tuned >= 0 && tuned <= 2) a.split = 1 << tuned;
+  if (tuned >= 0 && tuned <= 2 && a.phase_steps == 0) a.split = 1 << tuned;
   a.split_log2 = a.split == 4 ? 2 : a.split == 2 ? 1 : 0;
   a.steps = steps;
   a.steps_per_part = (steps + a.split - 1) / a.split;

@@ -541,6 +541,49 @@ struct RowStreamer {
     }
   }
 
+  // The steps [lo, hi) of the single batch in `buf`, against an image whose first step is s_off.
+  __device__ __forceinline__ void consume_steps(const Chunk<F> (&buf)[U][R], const float* const (&xs)[R], int lo, int hi, int s_off,
+                                                float (&acc)[MT][R]) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s_begin + u;
+      if (s >= lo && s < hi && s < s_end) {
+        const int slot = x_chunk_word<F, XB>(s - s_off, lane);
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+          float a[MT];
+#pragma unroll
+          for (int m = 0; m < MT; ++m) a[m] = acc[m][r];
+          if constexpr (XB) chunk_dot2<F, MT>(buf[u][r], reinterpret_cast<const uint32_t*>(xs[r]) + slot, per_row, a);
+          else chunk_fma<F, MT>(buf[u][r], xs[r] + slot, per_row, a);
+#pragma unroll
+          for (int m = 0; m < MT; ++m) acc[m][r] = a[m];
+        }
+      }
+    }
+  }
+
+  // ONE only: the group's batch against two images in turn, the first holding steps [0, split), the second the
+  // rest; restage() swaps them (the whole workgroup calls this: restage holds barriers). The sums see the steps
+  // in the same ascending order as with one image.
+  template <class RowsFn, class DoneFn, class Restage>
+  __device__ __forceinline__ void run_two_images(RowsFn& rows_fn, DoneFn& done_fn, int group, int split, Restage&& restage) {
+    static_assert(ONE, "one batch");
+    float acc[MT][R];
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+      for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+    const uint8_t* rows[R];
+    const uint8_t* scales[R];
+    const float* xs[R];
+    rows_fn(group, rows, scales, xs);
+    consume_steps(buf_a, xs, 0, split, 0, acc);
+    restage();
+    consume_steps(buf_a, xs, split, s_end, split, acc);
+    done_fn(group, acc);
+  }
+
   // Asks for the first two batches of a stream of n_groups groups (the second one only if there is one).
   template <class RowsFn>
   __device__ __forceinline__ void prefetch(RowsFn& rows_fn, int first_group, int stride, int n_groups) {

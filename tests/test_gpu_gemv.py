@@ -185,3 +185,10 @@ def test_weights_beyond_four_gigabytes(hip):
     y16 = ops.gemm_w(hip, x16, w)
     want = (x16.double() @ q[rows].double().T) * scale[rows].double()
     assert (y16[:, rows].double() - want).abs().max().item() <= 2e-4 * want.abs().max().item()
+
+
+@pytest.mark.parametrize("fmt,N,K", [("nvfp4", 512, 14336), ("nvfp4", 4096, 14336), ("bf16", 300, 4096), ("int8", 256, 8192)])
+def test_rows_do_not_depend_on_the_batch_long_rows(hip, fmt, N, K):
+    # Rows long enough that eight activation rows do not fit one LDS image: the image then holds half of K at a time
+    # (or the weights are passed over twice), and a row's bits must still be those of the row alone.
+    checks.gemv_rows_do_not_depend_on_batch(hip, fmt, N, K, seed=N + K)
