@@ -23,6 +23,9 @@ bool batch_invariant();
 inline hipStream_t as_stream(void* s) { return static_cast<hipStream_t>(s); }
 // Compute units of the current device (cached per device).
 int compute_units();
+// Lets `kernel` take up to `limit` bytes of dynamic LDS on the current device. The runtime is asked once per
+// (device, kernel) and thread; later calls cost a table lookup.
+void allow_lds(const void* kernel, int limit);
 
 // The variant table (runtime.hip): the K split registered for (kernel, M bucket, N, K), or -1.
 int tuned_variant(const char* kernel, int M, int N, int K);

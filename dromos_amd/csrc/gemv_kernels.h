@@ -294,7 +294,7 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
   a.chunks = static_cast<int>(rb / 16);
   a.row_bytes = rb;
   a.scale_row_bytes = F == LX_W_NVFP4 ? a.K / 16 : 0;
-  const int M = a.M;
+  const int M = a.M, phase_steps = a.phase_steps;
   const char* x0 = static_cast<const char*>(a.x);
   char* y0 = static_cast<char*>(a.y);
   const int64_t x_row = a.ld_x * (a.x_dtype == LX_BF16 ? 2 : 4), y_row = a.ld_y * (a.y_dtype == LX_BF16 ? 2 : 4);
@@ -303,6 +303,8 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
     a.x = x0 + m0 * x_row;
     a.y = y0 + m0 * y_row;
     const int mt = a.M <= 1 ? 1 : a.M <= 2 ? 2 : a.M <= 4 ? 4 : 8;
+    // A pass of one row stages its whole row (the single-row kernel has no phases; one row of any streamed K fits).
+    a.phase_steps = mt >= 2 ? phase_steps : 0;
     Shape shape = shape_for(F, steps);
     if (mt >= 2) shape.threads = 512;  // several activation rows: more wavefronts behind one image
     int st;

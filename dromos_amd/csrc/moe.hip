@@ -101,13 +101,17 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
       picked_logit[wave][lane] = NAN;
     }
   } else {
+    // A picked element is struck from the candidates by its bit in `taken` (bit j: this lane's element j), not by
+    // its value: an element whose logit is -inf can still be picked, once, lowest index first, as the reference's
+    // search over the indices not yet picked does (engine/cpu/moe.cpp:367-381).
+    uint64_t taken = 0;
     for (int r = 0; r < top_k; ++r) {
       float best = -INFINITY;
       int best_i = E;
 #pragma unroll
       for (int j = 0; j < NPL; ++j) {
         const int i = lane + j * kWave;
-        if (biased[j] > best || (biased[j] == best && i < best_i && i < E)) {
+        if (i < E && !((taken >> j) & 1) && (biased[j] > best || (biased[j] == best && i < best_i))) {
           best = biased[j];
           best_i = i;
         }
@@ -126,7 +130,7 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
         if (lane + j * kWave == best_i) {
           ids[t * top_k + r] = best_i;
           picked_logit[wave][r] = v[j];
-          biased[j] = -INFINITY;
+          taken |= 1ull << j;
         }
       }
       if (best_i >= E && lane == 0) {
@@ -402,10 +406,7 @@ bool streamable(const Stack& s, int64_t K, int max_rows) {
 
 template <class Kernel>
 void allow_big_lds(Kernel kernel, size_t lds) {
-  if (lds > 48 * 1024)
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,
-                            160 * 1024 - 1024) != hipSuccess)
-      (void)hipGetLastError();
+  if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), 160 * 1024 - 1024);
 }
 
 template <int F, int U>

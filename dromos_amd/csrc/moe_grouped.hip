@@ -13,6 +13,10 @@
 // Every pair's row is computed by the same arithmetic wherever it lands (the matrix instruction keeps rows
 // apart, the K split depends on the shapes only), and the sum runs in slot order, so a token's bits depend on
 // nothing but the token: not on the batch, the placement or the run.
+#include <stdio.h>
+
+#include <mutex>
+
 #include "common.h"
 #include "moe_common.h"
 #include "tile_mfma.h"
@@ -249,10 +253,7 @@ int launch_stage(Kernel kernel, GroupedArgs a, int64_t K, int NT, int out_rows, 
   const int64_t P = static_cast<int64_t>(a.T) * a.top_k;
   const int mt_max = static_cast<int>(((P < kTileTokens ? P : kTileTokens) + 15) / 16);
   const size_t lds = tile_lds_bytes(S, NT, mt_max);
-  if (lds > 48 * 1024)
-    if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024) !=
-        hipSuccess)
-      (void)hipGetLastError();
+  if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), 144 * 1024);
   hipLaunchKernelGGL(kernel, dim3((out_rows + kTileRows - 1) / kTileRows, tiles), dim3(S * kWave), lds, s, a);
   return status_of(hipGetLastError());
 }

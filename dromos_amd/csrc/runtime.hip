@@ -47,6 +47,16 @@ int compute_units() {
   return cached;
 }
 
+void allow_lds(const void* kernel, int limit) {
+  static thread_local std::vector<std::tuple<int, const void*, int>> raised;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) (void)hipGetLastError();
+  for (const auto& r : raised)
+    if (std::get<0>(r) == dev && std::get<1>(r) == kernel && std::get<2>(r) >= limit) return;
+  if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, limit) != hipSuccess) (void)hipGetLastError();
+  raised.emplace_back(dev, kernel, limit);
+}
+
 // Admission rule of the GEMV's variants (gemv.hip).
 bool gemv_admits(int wtype, int variant, int N, int K);
 
@@ -284,7 +294,9 @@ int lx_rt_device_props(int ordinal, lx_device_props* props) {
   if (hipDriverGetVersion(&v) == hipSuccess) props->driver_version = v;
   if (hipRuntimeGetVersion(&v) == hipSuccess) props->runtime_version = v;
   snprintf(props->isa, sizeof(props->isa), "%s", p.gcnArchName);
-  props->native_math = 1 << LX_MATH_BF16;
+  // The maths lx_gemm_w and lx_moe_experts_grouped run on the matrix cores' own types (engine/runtime/plan.cpp:79,358
+  // reads these bits): bf16, int8 (v_mfma_i32_16x16x64_i8) and e4m3 (v_mfma_f32_16x16x32_fp8_fp8) operands.
+  props->native_math = (1 << LX_MATH_BF16) | (1 << LX_MATH_INT8) | (1 << LX_MATH_FP8);
   return kOk;
 }
 

@@ -75,9 +75,16 @@ LX_API int lx_gemv_decode_bf16(const void* x, lx_dtype x_dtype, int ld_x, const 
                                float alpha, float beta, void* stream);
 
 /* ---- batched decode products (replaces engine/cuda/kernels.h:440-451 and 453-477) ----------------
- * lx_gemm_w: any M, the same product with `math`. This library runs LX_MATH_BF16 (activations rounded
- * to bf16, weights of any format expanded exactly to bf16, f32 sums on the matrix cores); the
- * low-precision maths answer 801. The workspace is not used by LX_MATH_BF16 (may be null).
+ * lx_gemm_w: any M, the same product with `math` (engine/cpu/gemm.cpp:189-296):
+ *   LX_MATH_BF16  any weight format: activations rounded to bf16, weights expanded exactly to bf16, f32 sums on
+ *                 the matrix cores; the workspace is not used (may be null)
+ *   LX_MATH_INT8  int8 weights: activations quantised per token to int8 inside the call (lx_quantize_act's rule),
+ *                 exact int32 sums; other weight formats answer 801
+ *   LX_MATH_FP8   fp8 weights: activations quantised per token to e4m3, exact products, f32 sums
+ *   LX_MATH_FP4 and LX_MATH_FP8 on NVFP4 weights answer 801.
+ * The quantised maths keep the activations' scales and bytes in the workspace (lx_gemm_workspace_bytes); with a
+ * null workspace they take scratch from the stream's memory pool instead (hipMallocAsync / hipFreeAsync, as the
+ * reference's kernels do: such a call allocates and cannot be captured in a graph).
  * lx_gemm_skinny: bf16 x, up to 64 rows per pass, every format, with the reduction-order contract of
  * engine/cuda/kernels.h:457-474: the K split depends on (N, K) only, never on M, so a row's bits do not
  * depend on the batch. With the environment variable LX_BATCH_INVARIANT set (non-empty, not starting
@@ -104,8 +111,8 @@ LX_API int lx_dequantize_weight(const lx_weight* w, void* out, int64_t rows, int
  * scale[m] = a / 127; FP8 q = e4m3(x * (448 / a)), scale[m] = a / 448; FP4 (K % 16 == 0) two e2m1 per byte,
  * block_scale e4m3 [M, ld_bs] one per 16 k, scale[m] = g = a / 2688, s_b = e4m3(a_b / (6 g)),
  * q = e2m1(x * (1 / (s_b g))), 0 where s_b = 0. A zero row: scale 1, q = 0. ld_q and ld_bs are in bytes.
- * Bytes identical to engine/cpu/quant.cpp:159-203. (The low-precision maths that consume it are not on this
- * path yet: lx_gemm_w and lx_moe_experts_grouped answer 801 for them.) */
+ * Bytes identical to engine/cpu/quant.cpp:159-203. lx_gemm_w's INT8 and FP8 maths quantise their activations by
+ * these rules. */
 LX_API int lx_quantize_act(const void* x, lx_dtype x_dtype, int ld_x, lx_math math, void* q, int ld_q, float* scale,
                            void* block_scale, int ld_bs, int M, int K, void* stream);
 
