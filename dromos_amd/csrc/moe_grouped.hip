@@ -367,3 +367,61 @@ int lx_moe_experts(const void* latent, const int32_t* ids, const float* weights,
 }
 
 }  // extern "C"
+
+// ---- lx_moe_experts for callers that cannot allocate ------------------------------------------------------
+//
+// The same kernels with their workspace (tables, intermediate rows, per-pair output rows) in a fixed array in device
+// memory instead of the stream's pool. Every device the library runs on holds its own copy of the array at its own
+// address until the process ends; the address is asked for once per device, on the first call there, with that
+// device current, and only that address (never the array's name, which in host code is a stand-in and no device
+// address) is handed to the kernels.
+constexpr int64_t kScratchBytes = 8ll << 20;
+static __device__ __align__(256) unsigned char scratch[kScratchBytes];
+
+namespace dro {
+namespace {
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_lock;
+void* g_scratch_of[kMaxDevices];  // the array's address on each device, once asked for
+
+// The array's address on the current device; null (and a recorded status) when the runtime cannot say.
+void* scratch_of_current_device(int* status) {
+  int dev = 0;
+  if ((*status = status_of(hipGetDevice(&dev)))) return nullptr;
+  if (dev < 0 || dev >= kMaxDevices) {
+    *status = fail(kInvalid);
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> g(g_scratch_lock);
+  if (!g_scratch_of[dev]) {
+    void* ptr = nullptr;
+    if ((*status = status_of(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch))))) return nullptr;
+    g_scratch_of[dev] = ptr;
+  }
+  return g_scratch_of[dev];
+}
+
+}  // namespace
+}  // namespace dro
+
+extern "C" {
+
+int lx_moe_experts_noalloc(const void* latent, const int32_t* ids, const float* weights, const void* gate_up, const void* down,
+                           float* out, int T, int L, int I, int top_k, void* stream) {
+  if (T <= 0) return kOk;
+  if (!latent || !ids || !weights || !out || L <= 0 || I <= 0 || top_k < 1 || !gate_up || !down) return fail(kInvalid);
+  const int64_t bytes = grouped_workspace_bytes(T, L, I, kMaxExperts, top_k);
+  if (bytes > kScratchBytes) {
+    fprintf(stderr, "lx_moe_experts_noalloc: T=%d L=%d I=%d top_k=%d needs %lld bytes of scratch, the fixed array holds %lld\n", T, L,
+            I, top_k, static_cast<long long>(bytes), static_cast<long long>(kScratchBytes));
+    return fail(kInvalid);
+  }
+  int st = kOk;
+  void* const ws = scratch_of_current_device(&st);
+  if (!ws) return st;
+  const lx_weight gu{LX_W_BF16, gate_up, nullptr, 1.0f, nullptr}, dn{LX_W_BF16, down, nullptr, 1.0f, nullptr};
+  return experts_grouped(latent, ids, weights, gu, dn, out, ws, T, L, I, kMaxExperts, top_k, as_stream(stream));
+}
+
+}  // extern "C"

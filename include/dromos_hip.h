@@ -142,6 +142,16 @@ LX_API int lx_moe_experts_grouped(const void* latent, const int32_t* ids, const 
                                   const lx_weight* gate_up, const lx_weight* down, lx_math math, float* out,
                                   void* workspace, int T, int L, int I, int E, int top_k, void* stream);
 LX_API int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int top_k, lx_math math);
+/* lx_moe_experts for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc. It has no counterpart in the reference (whose lx_moe_experts takes its scratch from the
+ * stream's memory pool, as lx_moe_experts here does). Same arguments, same kernels, same bits; the workspace is a
+ * fixed 8 MiB array in device memory that each device the library runs on holds until the process ends. A call
+ * whose lx_moe_grouped_workspace_bytes(T, L, I, 1024, top_k, LX_MATH_BF16) exceeds 8 MiB answers 1 (and says so on
+ * stderr) with nothing launched. Every call on a device shares that device's array: calls that overlap on one
+ * device (two streams, two threads) race; calls in stream order do not. The array's address is looked up on the
+ * first call on a device (no allocation; make that call outside a capture). */
+LX_API int lx_moe_experts_noalloc(const void* latent, const int32_t* ids, const float* weights, const void* gate_up,
+                                  const void* down, float* out, int T, int L, int I, int top_k, void* stream);
 
 /* ---- runtime (replaces engine/cuda/kernels.h:308-381 on the HIP runtime) --------------------------- */
 typedef struct {
