@@ -45,6 +45,8 @@ struct GemmArgs {
   int64_t row_bytes, scale_row_bytes;
   int tiles_per_wg, x_vecs, x_row_vecs, x_pitch, x_iters;  // the LDS activation image (XL and panel kernels)
   int x_phased;  // lean kernel with two slices a wavefront: the image holds half of K at a time
+  int win;       // windowed kernel: load steps of every slice the image holds at a time (2, 4 or 8)
+  int win_steps_shift, win_shift, row_shift;  // log2 of win, of the 16-byte pieces in a window, and in an image row
   const int8_t* xq;     // the INT8 math: quantised activations [M, K], rows K bytes apart
   const float* xscale;  // and their per-row scales
 };
@@ -482,6 +484,259 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) __attribute__((amdgpu_waves_
   }
 }
 
+// ---- up to 64 activation rows: the windowed tile kernel --------------------------------------------------------
+//
+// The arithmetic of the kernels above (one 16-row weight tile per S wavefronts, wavefront w taking the contiguous K
+// slice of steps_per_wave load steps [w * spw, (w + 1) * spw) as one ascending chain from zero, the S partial tiles
+// added in ascending order through LDS) for MT tiles of 16 activation rows at once, with an activation image that is
+// small whatever M and K are: it holds, for every slice, only a window of WIN load steps (2, 4, or 8 = one weight
+// batch), and moves along the slices with the wavefronts. A workgroup is `tiles_per_wg` tiles (their wavefronts share
+// the image); the window is restaged between two barriers whenever the wavefronts cross into the next one (they all
+// do so at the same step of their own slices). Neither the window nor the number of tiles per workgroup enters a
+// sum, so a row's bits are those of every other kernel here.
+//
+// Loads return in the order they were asked for, so what a wavefront waits for decides what stays in flight behind
+// it. The order here: a window's activations are asked for one window ahead and wait in registers; the next batch's
+// weights are asked for two loads at a time right before each place where a window may be crossed, so the wait for
+// the activations at a crossing always leaves weight loads in flight; between the two barriers of a crossing there
+// are only LDS writes. The loops are peeled (first batch: no crossing at its start; last batch: nothing to ask for)
+// so that every wait is a fixed count.
+// MATH as in tile16_kernel; a step past the end of the row is skipped (its clamped loads are not multiplied).
+template <int F, int MATH, bool XF32, int MT>
+__global__ void __launch_bounds__(kMaxSplit* kWave) window_kernel(const GemmArgs a) {
+  extern __shared__ __align__(16) f32x4 lds4[];
+  constexpr bool I8 = MATH != LX_MATH_BF16;
+  constexpr int E = Fmt<F>::kElems, J = I8 ? 1 : E / 8;
+  constexpr int CB = I8 ? 16 : E * 2;  // image bytes under one lane's 16-byte weight chunk
+  constexpr int SB = 4 * CB;           // image bytes of one load step
+  constexpr int SP = SB / 16;          // and its 16-byte pieces
+  using Acc = typename std::conditional<MATH == LX_MATH_INT8, i32x4, f32x4>::type;
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int S = a.S, tile_in_wg = wave / S, w = wave - tile_in_wg * S;
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const int tile_raw = blockIdx.x * a.tiles_per_wg + tile_in_wg;
+  const int n0 = min(tile_raw, n_tiles - 1) * kTileRows;  // a tile past the last repeats it and writes nothing
+  const int valid = min(kTileRows, a.N - n0);
+  const int g = lane >> 4, i = lane & 15;
+  uint8_t* const lds_bytes = reinterpret_cast<uint8_t*>(lds4);
+  uint8_t* const tile_lds = lds_bytes + tile_in_wg * S * kStageBytes;
+  uint8_t* const stage = tile_lds + w * kStageBytes;
+  uint8_t* const ximg = lds_bytes + (blockDim.x / kWave) * kStageBytes;
+  const int spw = a.steps_per_wave, WIN = a.win, kWinShift = a.win_steps_shift;
+
+  // The image of window p: row m holds, slice after slice, the activations under steps [ws * spw + p * WIN, + WIN) of
+  // slice ws; zero from K on. Pieces of 16 image bytes, numbered row by row; S is a power of two, so a piece's row,
+  // slice and place in the window are shifts and masks of its number. A thread holds kAhead pieces (the launcher
+  // sizes the window so that this covers the image).
+  constexpr int kAhead = XF32 ? 2 : 4;
+  const char* const xsrc = I8 ? reinterpret_cast<const char*>(a.xq) : static_cast<const char*>(a.xs.x);
+  const int64_t x_ld_bytes = I8 ? a.K : a.xs.ld * (XF32 ? 4 : 2);
+  const int win_shift = a.win_shift, row_shift = a.row_shift;  // log2 of the pieces in a window, in an image row
+  const int pieces = a.M << row_shift;
+  u32x4 xr[kAhead][XF32 ? 2 : 1];
+  auto window_load = [&](int p) {
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int v = min(static_cast<int>(threadIdx.x) + u * static_cast<int>(blockDim.x), pieces - 1);
+      const int m = v >> row_shift, c = v & ((1 << row_shift) - 1);
+      const int ws = c >> win_shift, cc = c & ((1 << win_shift) - 1);
+      const int piece = min((ws * spw + p * WIN) * SP + cc, a.x_vecs - 1);  // of the activation row; clamped, zeroed when stored
+      const char* src = xsrc + m * x_ld_bytes + static_cast<int64_t>(piece) * (XF32 ? 32 : 16);
+      xr[u][0] = *reinterpret_cast<const u32x4*>(src);
+      if constexpr (XF32) xr[u][1] = *reinterpret_cast<const u32x4*>(src + 16);
+    }
+  };
+  auto window_store = [&](int p) {
+#pragma unroll
+    for (int u = 0; u < kAhead; ++u) {
+      const int v = threadIdx.x + u * blockDim.x;
+      const int m = v >> row_shift, c = v & ((1 << row_shift) - 1);
+      const int ws = c >> win_shift, cc = c & ((1 << win_shift) - 1);
+      const int piece = (ws * spw + p * WIN) * SP + cc;
+      u32x4 val = xr[u][0];
+      if constexpr (XF32) {
+        bf16x2 q[4] = {pack_bf16(__uint_as_float(xr[u][0].x), __uint_as_float(xr[u][0].y)),
+                       pack_bf16(__uint_as_float(xr[u][0].z), __uint_as_float(xr[u][0].w)),
+                       pack_bf16(__uint_as_float(xr[u][1].x), __uint_as_float(xr[u][1].y)),
+                       pack_bf16(__uint_as_float(xr[u][1].z), __uint_as_float(xr[u][1].w))};
+        val = __builtin_bit_cast(u32x4, q);
+      }
+      if (piece >= a.x_vecs) val = u32x4{0u, 0u, 0u, 0u};
+      // No branch around the store (a piece past the image goes to a spare slot behind it): a branch would make the
+      // wait for these pieces a wait for every load in flight, the weights included.
+      *reinterpret_cast<u32x4*>(ximg + (v < pieces ? m * a.x_pitch + c * 16 : a.M * a.x_pitch)) = val;
+    }
+  };
+  const int n_windows = (spw + WIN - 1) >> kWinShift;
+  window_load(0);
+
+  // This lane's loads: rows 4 q + g of the tile, chunk i of each 4-step group (256 contiguous bytes per 16 lanes).
+  const uint8_t* const tile_w = a.w + static_cast<int64_t>(n0) * a.row_bytes;
+  uint32_t row_off[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) row_off[q] = static_cast<uint32_t>(min(4 * q + g, valid - 1)) * static_cast<uint32_t>(a.row_bytes);
+  const uint8_t* const own_scale = a.scale + (static_cast<int64_t>(n0) + min(i, valid - 1)) * a.scale_row_bytes;  // NVFP4 only
+  const int t_begin = w * spw;
+  u32x4 raw[2][4];
+  uint32_t sc[8];
+  auto issue_group = [&](int tb, int grp) {
+    const uint32_t c = static_cast<uint32_t>(min(4 * (tb + 4 * grp) + i, a.chunks - 1)) * 16u;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) raw[grp][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tile_w + (row_off[q] + c)));
+    if constexpr (F == LX_W_NVFP4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        sc[4 * grp + u] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale) + min(4 * (tb + 4 * grp + u) + g, a.chunks - 1));
+    }
+  };
+  issue_group(t_begin, 0);
+  issue_group(t_begin, 1);
+  window_store(0);
+  if (n_windows > 1) window_load(1);
+  __syncthreads();
+
+  u32x4* const put = reinterpret_cast<u32x4*>(stage + g * kStagePitch + i * 16);
+  const u32x4* const get = reinterpret_cast<const u32x4*>(stage + i * kStagePitch + g * 16);
+  const uint8_t* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = ximg + min(mt * 16 + i, a.M - 1) * a.x_pitch + w * WIN * SB + g * CB;
+  Acc acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = Acc{0, 0, 0, 0};
+  for (int off = 0; off < spw; off += 8) {  // the same trip count for every wavefront: the loop holds barriers
+#pragma unroll
+    for (int grp = 0; grp < 2; ++grp) {
+      uint32_t scales[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) scales[u] = F == LX_W_NVFP4 ? sc[4 * grp + u] : 0u;
+#pragma unroll
+      for (int q = 0; q < 4; ++q) put[q * (4 * kStagePitch / 16)] = raw[grp][q];
+      if (off + 8 < spw) issue_group(t_begin + off + 8, grp);  // the same group of the next batch
+      wave_lds_order();
+#pragma unroll
+      for (int half = 0; half < 2; ++half) {
+        const int so = off + 4 * grp + 2 * half;  // step within the slice
+        const int in_window = so & (WIN - 1);
+        if (so > 0 && in_window == 0) {
+          const int p = so >> kWinShift;
+          __syncthreads();  // every wavefront is done with the window before
+          window_store(p);
+          if (p + 1 < n_windows) window_load(p + 1);
+          __syncthreads();
+        }
+        u32x4 wv[2];
+#pragma unroll
+        for (int st = 0; st < 2; ++st) wv[st] = get[(2 * half + st) * 4];
+#pragma unroll
+        for (int st = 0; st < 2; ++st) {
+          if (t_begin + so + st < a.steps) {
+#pragma unroll
+            for (int mt = 0; mt < MT; ++mt) {
+              const uint8_t* xs = xrow[mt] + (in_window + st) * SB;
+              if constexpr (I8) {
+                acc[mt] = byte_mfma<MATH>(__builtin_bit_cast(i32x4, wv[st]), *reinterpret_cast<const i32x4*>(xs), acc[mt]);
+              } else {
+#pragma unroll
+                for (int j = 0; j < J; ++j)
+                  acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(weight_fragment<F>(wv[st], scales[2 * half + st], j),
+                                                                    *reinterpret_cast<const bf16x8*>(xs + 16 * j), acc[mt], 0, 0, 0);
+              }
+            }
+          }
+        }
+      }
+      wave_lds_order();
+    }
+  }
+
+  // The S partial tiles, added in ascending slice order by the tile's first wavefront.
+  Acc* const mine = reinterpret_cast<Acc*>(stage);
+  if (S > 1) {
+    wave_lds_order();
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) mine[mt * kWave + lane] = acc[mt];
+  }
+  float rf[4], bs[4];
+  const int nq = n0 + 4 * g;
+  const bool bias_f32 = a.bias && a.bias_dtype == LX_F32;
+  if (w == 0) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      const int n = min(nq + r, a.N - 1);
+      rf[r] = I8 ? reinterpret_cast<const float*>(a.scale)[n] : row_factor(F, a.scale, a.global, n);
+      bs[r] = bias_f32 ? static_cast<const float*>(a.bias)[n] : 0.0f;
+    }
+  }
+  if (S > 1) __syncthreads();
+  if (w != 0 || tile_raw >= n_tiles) return;
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + i;
+    if (m >= a.M) continue;
+    Acc sum = acc[mt];
+    for (int sl = 1; sl < S; ++sl) sum += reinterpret_cast<const Acc*>(tile_lds + sl * kStageBytes)[mt * kWave + lane];
+    const float xscale = I8 ? a.xscale[m] : 1.0f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      if (nq + r < a.N) {
+        const float b = bias_f32 || !a.bias ? bs[r] : load_as_f32(a.bias, a.bias_dtype, nq + r);
+        write_out(a, m, nq + r, static_cast<float>(sum[r]), I8 ? rf[r] * xscale : rf[r], b);
+      }
+    }
+  }
+}
+
+// Launches the windowed kernel for a.M <= 64 rows; false when no window fits (K slices too many for one workgroup).
+template <int F, int MATH>
+bool launch_window(GemmArgs a, int* status, hipStream_t stream) {
+  constexpr bool I8 = MATH != LX_MATH_BF16;
+  constexpr int SB = 4 * (I8 ? 16 : Fmt<F>::kElems * 2);
+  const int S = a.S, spw = a.steps_per_wave;
+  if (S > kMaxSplit || (S & (S - 1)) != 0 || spw % 8 != 0) return false;
+  const bool xf32 = !I8 && a.xs.dtype == LX_F32;
+  const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
+  auto image = [&](int win) { return static_cast<size_t>(a.M) * (static_cast<size_t>(S) * win * SB + 16) + 16; };
+  auto lds_for = [&](int tpw, int win) { return static_cast<size_t>(tpw) * S * kStageBytes + image(win); };
+  // Tiles to a workgroup: sixteen wavefronts' worth (the more tiles share an image, the less the activations cost).
+  const int tpw = kMaxSplit / S;
+  // The window: the largest of 8, 4, 2 steps whose image fits LDS and whose pieces its threads can hold.
+  const size_t held = (xf32 ? 2u : 4u) * tpw * S * kWave;
+  int win = 8;
+  while (win > 2 && (lds_for(tpw, win) > kLdsMax - 1024 || static_cast<size_t>(a.M) * S * win * (SB / 16) > held)) win /= 2;
+  if (lds_for(tpw, win) > kLdsMax - 1024 || static_cast<size_t>(a.M) * S * win * (SB / 16) > held) return false;
+  auto log2i = [](int v) { int l = 0; while ((1 << l) < v) ++l; return l; };
+  a.tiles_per_wg = tpw;
+  a.win = win;
+  a.win_steps_shift = log2i(win);
+  a.win_shift = log2i(win * (SB / 16));
+  a.row_shift = log2i(S * win * (SB / 16));
+  a.x_vecs = a.K * (I8 ? 1 : 2) / 16;
+  a.x_pitch = S * win * SB + 16;
+  const size_t lds = lds_for(tpw, win);
+  const unsigned threads = tpw * S * kWave, grid = (n_tiles + tpw - 1) / tpw;
+  auto launch = [&](auto kernel) {
+    if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), kLdsMax);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(threads), lds, stream, a);
+    return status_of(hipGetLastError());
+  };
+  auto with_mt = [&](auto mt_tag) {
+    constexpr int MT = decltype(mt_tag)::value;
+    auto with_x = [&](auto x_tag) {
+      constexpr bool XF = decltype(x_tag)::value;
+      return launch(window_kernel<F, MATH, XF, MT>);
+    };
+    if constexpr (I8) return with_x(std::false_type{});
+    else return xf32 ? with_x(std::true_type{}) : with_x(std::false_type{});
+  };
+  switch ((a.M + 15) / 16) {
+    case 1: *status = with_mt(std::integral_constant<int, 1>{}); break;
+    case 2: *status = with_mt(std::integral_constant<int, 2>{}); break;
+    case 3: *status = with_mt(std::integral_constant<int, 3>{}); break;
+    default: *status = with_mt(std::integral_constant<int, 4>{}); break;
+  }
+  return true;
+}
+
 // Launches the lean tile kernel for a.M <= 16 rows when its LDS image fits; false if it does not.
 template <int F, int MATH>
 bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
@@ -740,6 +995,12 @@ template <int F, int MT>
 int launch_skinny(GemmArgs a, hipStream_t stream) {
   const int S = a.S;
   const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
+  // More than eight rows: the windowed kernel (for 9 .. 16 rows where the matrix has the tiles to fill its
+  // sixteen-wavefront workgroups; the lean kernel's image of all of K leaves too few of them resident there).
+  if (MT > 1 || (a.M > 8 && n_tiles >= 320)) {
+    int st = kOk;
+    if (launch_window<F, LX_MATH_BF16>(a, &st, stream)) return st;
+  }
   if constexpr (MT == 1) {
     int st = kOk;
     if (launch_tile16<F, LX_MATH_BF16>(a, &st, stream)) return st;
@@ -950,6 +1211,7 @@ int gemm_bytes_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w
         return status_of(hipGetLastError());
       };
       const int mt = (a.M + 15) / 16;
+      if ((mt > 1 || (a.M > 8 && n_tiles >= 320)) && launch_window<F, MATH>(a, &st, s)) continue;
       if (mt == 1 && launch_tile16<F, MATH>(a, &st, s)) continue;
       if (mt == 1) {
         // The activation image: rows as long as the last weight batch reaches, zero past K.
