@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Measures the decode matrix-product path on one MI355X: weight-stream GB/s and fraction of the 8 TB/s HBM peak.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cases headline|gemv|all|layer] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--cases all|headline|gemv|layer] [--no-cpu]
     python bench.py --pmc-probe      (for rocprofv3 --pmc: a plain copy of known size, then headline launches)
 
 A step is one pass of the hot path over one batch: one lx_gemv_w call (the headline), one skinny GEMM, or one
@@ -11,8 +11,12 @@ once into a HIP graph through the library's own lx_rt_capture_* entry points (as
 steps) and the graph is launched between two HIP events on its stream; W untimed steps run first.
 
 Prints one JSON line. `value` is the headline case (INT8 weight-only GEMV, W 14336 x 4096, M = 1, bf16 x);
-`cases` lists every measured case with its own time, GB/s and fraction of peak. Bytes per step are the
+`cases` lists every measured case (by default one per benchmark configuration: C1, C2 int8 / fp8 at M = 1, 4, 16, 64 in
+both modes, C3 M = 1, 8, C4 T = 1, 8, 32, 64, C5) with its own time, GB/s and fraction of peak. Bytes per step are the
 algorithmic bytes: weights + scales + x + y (bench/bench_gemv.py:51-56 of the reference uses the same count).
+`floor` states what the memory system allows at these sizes, measured the same way in the same run: an empty launch,
+and a plain read of the same weight copies (lx_probe_read: the GEMV's access pattern without the product); a GEMV case
+carries `floor_us` (the plain read of its bytes) and `vs_floor` (its time over that).
 """
 
 import argparse
@@ -97,6 +101,14 @@ def make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, invariant=False, math=0
     nbytes = algorithmic_bytes_gemv(fmt, M, N, K)
     ws_buf = torch.empty(max(int(lx.size("gemm_workspace_bytes", M, K, math)), 256), dtype=torch.uint8, device="cuda")
 
+    def floor_step(i, flat=[]):
+        # A plain read of the same number of bytes (weights + scales) from a flat buffer of rotating copies.
+        if not flat:
+            flat.append(torch.empty(copies * ((per_copy + 255) // 256 * 256), dtype=torch.uint8, device="cuda"))
+        at = (i % copies) * ((per_copy + 255) // 256 * 256)
+        st = lx.status("probe_read", flat[0][at:], ctypes.c_int64(per_copy // 16 * 16))
+        assert st == 0, st
+
     def step(i):
         p = ptrs[i % copies]
         if entry == "gemv_w":
@@ -107,6 +119,7 @@ def make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, invariant=False, math=0
             st = lx.status("gemm_w", x, DTYPE[x.dtype], K, p, math, None, F32, y, F32, N, M, N, K, 1.0, 0.0, ws_buf)
         assert st == 0, st
 
+    step.floor = floor_step
     return step, nbytes, (ws, structs, ptrs, x, y, ws_buf)
 
 
@@ -230,7 +243,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--cases", default="headline", choices=["headline", "gemv", "all", "layer"])
+    ap.add_argument("--cases", default="all", choices=["headline", "gemv", "all", "layer"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="no timing: one 256 MiB device copy (the counters' yardstick) and 20 eager headline launches")
@@ -261,6 +274,12 @@ def main():
     K_STEPS, W = args.steps, args.warmup
 
     cases = []
+    floors = {}
+
+    def empty_step(i):
+        assert lx.status("probe_empty") == 0
+
+    floors["empty_launch_us"] = round(timer.run(empty_step, K_STEPS, W), 3)
 
     def run_gemv(name, fmt, M, N, K, seed, entry="gemv_w", invariant=False, math=0):
         if invariant:
@@ -270,11 +289,14 @@ def main():
         step, nbytes, keep = make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, math=math)
         us = timer.run(step, K_STEPS, W)
         os.environ.pop("LX_BATCH_INVARIANT", None)
+        key = f"read_{fmt}_{N}x{K}_us"
+        if key not in floors:
+            floors[key] = round(timer.run(step.floor, K_STEPS, W), 3)
         gbps = nbytes / us / 1e3
         case = {"case": name, "entry": "lx_" + entry, "format": fmt, "math": ["bf16", "int8", "fp8", "fp4"][math], "M": M, "N": N, "K": K,
                 "batch_invariant": invariant,
                 "us_per_step": round(us, 3), "bytes_per_step": int(nbytes), "GBps": round(gbps, 1),
-                "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4)}
+                "frac_of_hbm_peak": round(gbps / HBM_PEAK_GBPS, 4), "floor_us": floors[key], "vs_floor": round(us / floors[key], 3)}
         cases.append(case)
         del keep
         torch.cuda.empty_cache()
@@ -365,6 +387,7 @@ def main():
                                "lx_gemv_w on rotated weight copies (> 512 MB)"},
         "roofline": {"bound": "hbm", "achieved": head["GBps"], "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(head["GBps"] / HBM_PEAK_GBPS, 4), "traffic": load_traffic()},
+        "floor": floors,
         "cases": cases,
     }
     if not args.no_cpu:

@@ -519,6 +519,21 @@ int experts_decode(const void* latent, const int32_t* ids, const float* weights,
   }
 }
 
+// lx_moe_route behind its validation (engine/cpu/moe.cpp:343-348).
+int route(const float* logits, const float* selection_bias, int32_t* ids, float* weights, float* entropy, float* confidence, int T,
+          int E, int top_k, hipStream_t s) {
+  if (T <= 0) return kOk;
+  if (top_k < 1 || top_k > 64 || top_k > E || !logits || !ids || !weights || !entropy || !confidence) return fail(kInvalid);
+  if (E > 4096) return fail(kNotSupported);
+  const dim3 grid((T + kWaves - 1) / kWaves), block(kThreads);
+  if (E <= 64) hipLaunchKernelGGL(route_kernel<1>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  else if (E <= 128) hipLaunchKernelGGL(route_kernel<2>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  else if (E <= 256) hipLaunchKernelGGL(route_kernel<4>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  else if (E <= 1024) hipLaunchKernelGGL(route_kernel<16>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  else hipLaunchKernelGGL(route_kernel<64>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
+  return status_of(hipGetLastError());
+}
+
 int experts_plain(const DecodeArgs& a, int gu_type, int dn_type, hipStream_t s) {
   if (int st = gate_up_plain(a, gu_type, s)) return st;
   return down_plain(a, dn_type, s);
@@ -532,17 +547,7 @@ extern "C" {
 
 int lx_moe_route(const float* logits, const float* selection_bias, int32_t* ids, float* weights, float* entropy,
                  float* confidence, int T, int E, int top_k, void* stream) {
-  if (T <= 0) return kOk;
-  if (top_k < 1 || top_k > 64 || top_k > E || !logits || !ids || !weights || !entropy || !confidence) return fail(kInvalid);
-  if (E > 4096) return fail(kNotSupported);
-  const dim3 grid((T + kWaves - 1) / kWaves), block(kThreads);
-  hipStream_t s = as_stream(stream);
-  if (E <= 64) hipLaunchKernelGGL(route_kernel<1>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
-  else if (E <= 128) hipLaunchKernelGGL(route_kernel<2>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
-  else if (E <= 256) hipLaunchKernelGGL(route_kernel<4>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
-  else if (E <= 1024) hipLaunchKernelGGL(route_kernel<16>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
-  else hipLaunchKernelGGL(route_kernel<64>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
-  return status_of(hipGetLastError());
+  return route(logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k, as_stream(stream));
 }
 
 int lx_moe_experts_decode(const void* latent, const int32_t* ids, const float* weights, const lx_weight* gate_up,

@@ -45,6 +45,13 @@ inline bool valid_stack(const lx_weight& w, int64_t K) {
   }
 }
 
+// moe.hip: routing behind lx_moe_route, and the decode experts (T <= 8, top_k <= 8) on two stacks of any formats with
+// the intermediate rows and the sort table in `inter` (lx_moe_decode_workspace_bytes).
+int route(const float* logits, const float* selection_bias, int32_t* ids, float* weights, float* entropy, float* confidence, int T,
+          int E, int top_k, hipStream_t s);
+int experts_decode(const void* latent, const int32_t* ids, const float* weights, const lx_weight& gate_up, const lx_weight& down,
+                   float* out, void* inter, int T, int L, int I, int top_k, hipStream_t s);
+
 // Element-wise experts for any T and any shape or alignment (one wavefront per output, pairs independent):
 // gate/up into a.inter (by pair), then down and the ordered sum into a.out.
 int experts_plain(const DecodeArgs& a, int gu_type, int dn_type, hipStream_t s);

@@ -129,6 +129,24 @@ __global__ void __launch_bounds__(256) read_probe_kernel(const u32x4* __restrict
   if (acc == 0x9e3779b9u) *sink = acc;  // keeps the loads alive; pseudo-random data never matches
 }
 
+// The measurement floor of a streamed product: 16-byte non-temporal loads, eight in flight per lane, every wavefront's
+// loads asked for at once, 1 KB contiguous per instruction: what the decode GEMV does, without the product.
+__global__ void __launch_bounds__(256) stream_read_kernel(const u32x4* __restrict__ p, int64_t n16, unsigned* sink) {
+  const int64_t base = (static_cast<int64_t>(blockIdx.x) * 4 + threadIdx.x / kWave) * (8 * kWave) + (threadIdx.x & (kWave - 1));
+  u32x4 v[8];
+#pragma unroll
+  for (int u = 0; u < 8; ++u) {
+    const int64_t i = base + u * kWave;
+    v[u] = __builtin_nontemporal_load(p + (i < n16 ? i : n16 - 1));
+  }
+  unsigned acc = 0;
+#pragma unroll
+  for (int u = 0; u < 8; ++u) acc ^= v[u].x ^ v[u].y ^ v[u].z ^ v[u].w;
+  if (acc == 0x9e3779b9u && sink) *sink = acc;
+}
+
+__global__ void empty_kernel() {}
+
 __global__ void fill_random_kernel(unsigned* p, int64_t n) {
   const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
   if (i < n) {
@@ -353,6 +371,19 @@ int lx_bandwidth_probe(int64_t bytes, int reps, double* read_gbps, double* spec_
   (void)hipFree(sink);
   (void)hipFree(buf);
   return st;
+}
+
+int lx_probe_read(const void* data, int64_t bytes, void* stream) {
+  if (!data || bytes < 16 || reinterpret_cast<uintptr_t>(data) % 16 != 0) return fail(kInvalid);
+  const int64_t n16 = bytes / 16, per_wg = 4 * 8 * kWave;
+  hipLaunchKernelGGL(stream_read_kernel, dim3(static_cast<unsigned>((n16 + per_wg - 1) / per_wg)), dim3(256), 0, as_stream(stream),
+                     static_cast<const u32x4*>(data), n16, static_cast<unsigned*>(nullptr));
+  return status_of(hipGetLastError());
+}
+
+int lx_probe_empty(void* stream) {
+  hipLaunchKernelGGL(empty_kernel, dim3(1), dim3(kWave), 0, as_stream(stream));
+  return status_of(hipGetLastError());
 }
 
 // ---- architecture and variants ------------------------------------------------------------------------

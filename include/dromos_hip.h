@@ -142,6 +142,34 @@ LX_API int lx_moe_experts_grouped(const void* latent, const int32_t* ids, const 
                                   const lx_weight* gate_up, const lx_weight* down, lx_math math, float* out,
                                   void* workspace, int T, int L, int I, int E, int top_k, void* stream);
 LX_API int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int top_k, lx_math math);
+/* ---- the calls either side of the experts in a decode layer (replaces engine/cuda/kernels.h:211-233, 253-261,
+ * 814-819; the model calls them at engine/model/metis.cpp:2086-2096) and the legacy product forms (:66-70) ------
+ *   lx_spec_gemv_f32        y[M, N] = x[M, K] @ w[N, K]^T + bias[N], all f32, M <= 8, a row's bits independent of M
+ *   lx_router_route         that product on the router's weights w [E, K] into logits [M, E], then lx_moe_route on
+ *                           them: every output has the bits of the two calls (it is the two calls, in two launches);
+ *                           M <= 8, E <= 1024, K <= 2048, top_k <= 32; `ticket` (one zeroed int32 the fused CUDA
+ *                           kernel counts in) must be given and is left untouched
+ *   lx_moe_summary          summary[t, :] = sum_k weights[t, k] * expert_emb[ids[t, k], :], expert_emb bf16 [E, R],
+ *                           summary f32 [T, R]; _history also history = a * history + b * summary in place
+ *   lx_moe_experts_w8       lx_moe_experts on int8 stacks with per-row scales (gate_up_scale [E, 2I], down_scale
+ *                           [E, L]), any T, top_k <= 8, workspace of lx_moe_workspace_bytes(T, I, top_k)
+ *   lx_gemm_bf16            y = alpha * (x @ w^T + bias) + beta * y, x and w bf16, bias bf16 or null, any M */
+LX_API int lx_spec_gemv_f32(const float* x, int ld_x, const float* w, const float* bias, float* y, int ld_y, int M, int N,
+                            int K, void* stream);
+LX_API int lx_router_route(const float* x, int ld_x, const float* w, const float* bias, float* logits,
+                           const float* selection_bias, int32_t* ids, float* weights, float* entropy, float* confidence,
+                           int32_t* ticket, int M, int E, int K, int top_k, void* stream);
+LX_API int lx_moe_summary(const int32_t* ids, const float* weights, const void* expert_emb, float* summary, int T, int R,
+                          int top_k, void* stream);
+LX_API int lx_moe_summary_history(const int32_t* ids, const float* weights, const void* expert_emb, float* summary,
+                                  float* history, float a, float b, int T, int R, int top_k, void* stream);
+LX_API int lx_moe_experts_w8(const void* latent, const int32_t* ids, const float* weights, const int8_t* gate_up,
+                             const float* gate_up_scale, const int8_t* down, const float* down_scale, float* out,
+                             void* workspace, int T, int L, int I, int top_k, void* stream);
+LX_API int64_t lx_moe_workspace_bytes(int T, int I, int top_k);
+LX_API int lx_gemm_bf16(const void* x, int ld_x, const void* w, const void* bias, void* y, lx_dtype y_dtype, int ld_y,
+                        int M, int N, int K, float alpha, float beta, void* stream);
+
 /* lx_moe_experts for callers that cannot allocate: code under HIP graph capture, tight serving loops, harnesses
  * that forbid hipMalloc. It has no counterpart in the reference (whose lx_moe_experts takes its scratch from the
  * stream's memory pool, as lx_moe_experts here does). Same arguments, same kernels, same bits; the workspace is a
@@ -197,6 +225,15 @@ LX_API int lx_rt_is_host_memory(const void* ptr);
 LX_API int lx_rt_device_props(int ordinal, lx_device_props* props);
 LX_API int lx_rt_mem_info(int64_t* free_bytes, int64_t* total_bytes);
 LX_API int lx_bandwidth_probe(int64_t bytes, int reps, double* read_gbps, double* spec_gbps, void* stream);
+
+/* ---- measurement floors (no counterpart in the reference: for benches that state how far a product is from a
+ * plain read of the same bytes). Both are asynchronous and capturable.
+ *   lx_probe_read   reads `bytes` bytes at `data` (16-byte aligned) once, as the decode GEMV streams a weight: 16-byte
+ *                   non-temporal loads, 1 KB contiguous per wavefront instruction, eight in flight per lane, nothing
+ *                   computed or written
+ *   lx_probe_empty  one empty kernel launch */
+LX_API int lx_probe_read(const void* data, int64_t bytes, void* stream);
+LX_API int lx_probe_empty(void* stream);
 
 /* ---- architecture and kernel variants (replaces engine/cuda/tunable.h:37-55) -----------------------
  * lx_arch is 95 on gfx950. The GEMV registers its variants under gemv_w_<format>; a variant's name starts

@@ -811,6 +811,111 @@ ORC_API int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int t
   return round256(2 * (int64_t)T * top_k * I);
 }
 
+/* ---- the calls either side of the experts in a decode layer, and the legacy product forms ------------ */
+
+/* engine/cpu/gemm.cpp:304-314: bf16 x and weights under the BF16 math, bias bf16 or null. */
+ORC_API int lx_gemm_bf16(const void* x, int ld_x, const void* w, const void* bias, void* y, int y_dtype, int ld_y, int M, int N,
+                         int K, float alpha, float beta, void* stream) {
+  (void)stream;
+  if (y_dtype != LX_F32 && y_dtype != LX_BF16) return fail(ORC_INVALID);
+  if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(ORC_INVALID);
+  if (M == 0 || N == 0) return ORC_OK;
+  if (!x || !w || !y) return fail(ORC_INVALID);
+  lx_weight wt = {LX_W_BF16, w, NULL, 1.0f, NULL};
+  return gemm_bf16_math(x, LX_BF16, ld_x, &wt, bias, LX_BF16, y, y_dtype, ld_y, M, N, K, alpha, beta);
+}
+
+/* engine/cpu/gemm.cpp:316-337: f32 x and weights, the same dot and epilogue (row factor 1, alpha 1, beta 0). */
+ORC_API int lx_gemm_f32(const float* x, int ld_x, const float* w, const float* bias, float* y, int ld_y, int M, int N, int K,
+                        void* stream) {
+  (void)stream;
+  if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(ORC_INVALID);
+  if (M == 0 || N == 0) return ORC_OK;
+  if (!x || !w || !y) return fail(ORC_INVALID);
+#pragma omp parallel for schedule(static)
+  for (int64_t n = 0; n < N; ++n)
+    for (int64_t m = 0; m < M; ++m)
+      epilogue(dot_f32(x + m * (int64_t)ld_x, w + n * (int64_t)K, K), 1.0f, bias, LX_F32, y, LX_F32, m * (int64_t)ld_y + n, n, 1.0f, 0.0f);
+  return ORC_OK;
+}
+
+/* engine/cpu/spec.cpp:21-28: lx_gemm_f32 limited to decode-sized steps. */
+ORC_API int lx_spec_gemv_f32(const float* x, int ld_x, const float* w, const float* bias, float* y, int ld_y, int M, int N, int K,
+                             void* stream) {
+  if (M == 0 || N == 0) return ORC_OK;
+  if (M < 0 || M > 8 || K <= 0 || ld_x < K || ld_y < N || !x || !w || !y) return fail(ORC_INVALID);
+  return lx_gemm_f32(x, ld_x, w, bias, y, ld_y, M, N, K, stream);
+}
+
+ORC_API int lx_moe_route(const float* logits, const float* selection_bias, int32_t* ids, float* weights, float* entropy,
+                         float* confidence, int T, int E, int top_k, void* stream);
+
+/* engine/cuda/kernels.h:211-219: the two calls in one (the reference's CPU backend leaves it out; by its contract every
+ * output has the bits of lx_spec_gemv_f32 followed by lx_moe_route, which is what this is). */
+ORC_API int lx_router_route(const float* x, int ld_x, const float* w, const float* bias, float* logits, const float* selection_bias,
+                            int32_t* ids, float* weights, float* entropy, float* confidence, int32_t* ticket, int M, int E, int K,
+                            int top_k, void* stream) {
+  if (M <= 0) return ORC_OK;
+  if (M > 8 || E <= 0 || E > 1024 || K <= 0 || K > 2048 || ld_x < K || top_k < 1 || top_k > 32 || top_k > E || !x || !w || !logits ||
+      !ids || !weights || !entropy || !confidence || !ticket)
+    return fail(ORC_INVALID);
+  int st = lx_spec_gemv_f32(x, ld_x, w, bias, logits, E, M, E, K, stream);
+  if (st) return st;
+  return lx_moe_route(logits, selection_bias, ids, weights, entropy, confidence, M, E, top_k, stream);
+}
+
+/* engine/cpu/moe.cpp:399-418 (history == NULL) and :420-442. */
+static int summary(const int32_t* ids, const float* weights, const void* expert_emb, float* sum, float* history, float a, float b,
+                   int T, int R, int top_k, int with_history) {
+  if (T <= 0 || R <= 0) return ORC_OK;
+  if (!ids || !weights || !expert_emb || !sum || top_k < 1 || (with_history && !history)) return fail(ORC_INVALID);
+  const uint16_t* emb = (const uint16_t*)expert_emb;
+  for (int64_t t = 0; t < T; ++t) {
+    float* s = sum + t * R;
+    for (int r = 0; r < R; ++r) s[r] = 0.0f;
+    for (int k = 0; k < top_k; ++k) {
+      const float w = weights[t * top_k + k];
+      const uint16_t* row = emb + (int64_t)ids[t * top_k + k] * R;
+      for (int r = 0; r < R; ++r) s[r] += w * bf16_value(row[r]);
+    }
+    if (with_history) {
+      float* h = history + t * R;
+      for (int r = 0; r < R; ++r) h[r] = a * h[r] + b * s[r];
+    }
+  }
+  return ORC_OK;
+}
+ORC_API int lx_moe_summary(const int32_t* ids, const float* weights, const void* expert_emb, float* sum, int T, int R, int top_k,
+                           void* stream) {
+  (void)stream;
+  return summary(ids, weights, expert_emb, sum, NULL, 0.0f, 0.0f, T, R, top_k, 0);
+}
+ORC_API int lx_moe_summary_history(const int32_t* ids, const float* weights, const void* expert_emb, float* sum, float* history,
+                                   float a, float b, int T, int R, int top_k, void* stream) {
+  (void)stream;
+  return summary(ids, weights, expert_emb, sum, history, a, b, T, R, top_k, 1);
+}
+
+/* engine/cpu/moe.cpp:460-476: the weight-only experts on int8 stacks with per-row scales, any T. */
+ORC_API int lx_moe_experts_w8(const void* latent, const int32_t* ids, const float* weights, const int8_t* gate_up,
+                              const float* gate_up_scale, const int8_t* down, const float* down_scale, float* out, void* workspace,
+                              int T, int L, int I, int top_k, void* stream) {
+  (void)stream;
+  (void)workspace;
+  if (T <= 0) return ORC_OK;
+  int st = experts_args(latent, ids, weights, out, L, I, top_k);
+  if (st) return st;
+  if (!gate_up || !gate_up_scale || !down || !down_scale) return fail(ORC_INVALID);
+  lx_weight gu = {LX_W_INT8, gate_up, gate_up_scale, 1.0f, NULL}, dn = {LX_W_INT8, down, down_scale, 1.0f, NULL};
+  return experts((const uint16_t*)latent, ids, weights, &gu, &dn, out, T, L, I, top_k, 0);
+}
+/* engine/cpu/moe.cpp:512-517 */
+ORC_API int64_t lx_moe_workspace_bytes(int T, int I, int top_k) {
+  if (T <= 0 || I <= 0 || top_k <= 0) return 0;
+  const int64_t pairs = (int64_t)T * top_k;
+  return round256((2 * pairs * I + 15) / 16 * 16 + 8 * pairs);
+}
+
 /* ---- the few runtime calls a host-memory harness needs (engine/cuda/kernels.h:308-339) ------------- */
 
 ORC_API int lx_rt_backend(void) { return 3; /* LX_BACKEND_CPU */ }

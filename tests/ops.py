@@ -176,3 +176,66 @@ def experts_reference(latent, ids, weights, gu_dense, dn_dense):
             mid = (F.silu(g) * u).to(torch.bfloat16).double()
             out[t] += weights[t, k].double() * (dn_dense[e] @ mid)
     return out
+
+
+# ---- the calls either side of the experts, and the legacy product forms ----------------------------------------
+
+
+def spec_gemv_f32(lx, x, w, bias=None, M=None, status=False):
+    M = x.shape[0] if M is None else M
+    N, K = w.shape
+    y = torch.full((max(M, 1), N), float("nan"), device=lx.device)
+    args = (x, x.shape[1], w, bias, y, N, M, N, K)
+    if status:
+        return lx.status("spec_gemv_f32", *args)
+    lx("spec_gemv_f32", *args)
+    return y[:M]
+
+
+def router_route(lx, x, w, bias, selection_bias, top_k, status=False):
+    M, K = x.shape
+    E = w.shape[0]
+    logits = torch.full((M, E), float("nan"), device=lx.device)
+    ids = torch.full((M, top_k), -1, dtype=torch.int32, device=lx.device)
+    weights = torch.full((M, top_k), float("nan"), device=lx.device)
+    entropy = torch.full((M,), float("nan"), device=lx.device)
+    confidence = torch.full((M,), float("nan"), device=lx.device)
+    ticket = torch.zeros(1, dtype=torch.int32, device=lx.device)
+    args = (x, K, w, bias, logits, selection_bias, ids, weights, entropy, confidence, ticket, M, E, K, top_k)
+    if status:
+        return lx.status("router_route", *args)
+    lx("router_route", *args)
+    assert ticket.item() == 0
+    return logits, ids, weights, entropy, confidence
+
+
+def moe_summary(lx, ids, weights, emb, history=None, a=0.0, b=0.0):
+    T, top_k = ids.shape
+    R = emb.shape[1]
+    out = torch.full((T, R), float("nan"), device=lx.device)
+    if history is None:
+        lx("moe_summary", ids, weights, emb, out, T, R, top_k)
+    else:
+        lx("moe_summary_history", ids, weights, emb, out, history, float(a), float(b), T, R, top_k)
+    return out
+
+
+def experts_w8(lx, latent, ids, weights, gu, dn, I, top_k, status=False):
+    T, L = latent.shape
+    nbytes = int(lx.size("moe_workspace_bytes", T, I, top_k))
+    ws = torch.full((max(nbytes, 1),), 0xFF, dtype=torch.uint8, device=lx.device)
+    out = torch.full((T, L), float("nan"), device=lx.device)
+    args = (latent, ids, weights, gu.data, gu.scale, dn.data, dn.scale, out, ws, T, L, I, top_k)
+    if status:
+        return lx.status("moe_experts_w8", *args)
+    lx("moe_experts_w8", *args)
+    return out
+
+
+def gemm_bf16(lx, x, w, bias=None, y=None, alpha=1.0, beta=0.0, y_dtype=torch.float32):
+    M, K = x.shape
+    N = w.shape[0]
+    if y is None:
+        y = torch.full((M, N), float("nan"), dtype=y_dtype, device=lx.device)
+    lx("gemm_bf16", x, K, w, bias, y, DTYPE[y.dtype], N, M, N, K, float(alpha), float(beta))
+    return y
