@@ -218,4 +218,9 @@ __device__ __forceinline__ float silu(float v) { return v / (1.0f + expf(-v)); }
 int quantize_act_rows(const void* x, int x_dtype, int64_t ld_x, int math, void* q, int64_t ld_q, float* scale, void* block_scale,
                       int64_t ld_bs, int M, int K, hipStream_t stream);
 
+// quant.hip: the rows of x as a quantised math sees them (quantised per row, their exact values back as bf16 rows
+// xhat [M, K], the per-row scales apart); q is scratch of M * (K + K / 16) bytes.
+int act_images(const void* x, int x_dtype, int64_t ld_x, int math, uint8_t* q, uint16_t* xhat, float* scale, int M, int K,
+               hipStream_t stream);
+
 }  // namespace dro

@@ -49,11 +49,12 @@ struct GemmArgs {
   int win_steps_shift, win_shift, row_shift;  // log2 of win, of the 16-byte pieces in a window, and in an image row
   const int8_t* xq;     // the INT8 math: quantised activations [M, K], rows K bytes apart
   const float* xscale;  // and their per-row scales
+  const float* act_scale;  // BF16-math kernels on a quantised math's activation images: the rows' scales (else null)
 };
 
 // The epilogue's operation order (engine/cpu/gemm.cpp:21-34); rf is the row factor, b the bias (0 without one).
 __device__ __forceinline__ void write_out(const GemmArgs& a, int m, int n, float sum, float rf, float b) {
-  float t = rf * sum;
+  float t = (a.act_scale ? rf * a.act_scale[m] : rf) * sum;
   if (a.bias) t += b;
   float v = a.alpha * t;
   const int64_t at = m * a.ld_y + n;
@@ -1074,11 +1075,13 @@ int launch_format(GemmArgs a, const char* x0, char* y0, int M, int x_esize, int 
   // Slices are whole weight batches (the row's last one may be cut short by the row's end).
   a.steps_per_wave = ((a.steps + S - 1) / S + kLoadsInFlight - 1) / kLoadsInFlight * kLoadsInFlight;
   a.S = S;
+  const float* const act_scale0 = a.act_scale;
   // Up to 64 activation rows a pass; every pass is the same arithmetic per row.
   for (int m0 = 0; m0 < M; m0 += 64) {
     a.M = M - m0 < 64 ? M - m0 : 64;
     a.xs.x = x0 + static_cast<int64_t>(m0) * a.xs.ld * x_esize;
     a.y = y0 + static_cast<int64_t>(m0) * a.ld_y * y_esize;
+    if (act_scale0) a.act_scale = act_scale0 + m0;
     int st;
     switch ((a.M + 15) / 16) {
       case 1: st = launch_skinny<F, 1>(a, stream); break;
@@ -1108,8 +1111,18 @@ bool valid_weight(const lx_weight* w, int64_t K) {
 
 // The matrix-core product of any format: BF16 math (x rounded to bf16), any M. Validation follows
 // engine/cpu/gemm.cpp:189-197.
+int gemm_bf16_scaled(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w, const void* bias, int bias_dtype, void* y,
+                     int y_dtype, int64_t ld_y, int M, int N, int K, float alpha, float beta, const float* act_scale, void* stream);
+
 int gemm_bf16_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w, const void* bias, int bias_dtype, void* y,
                    int y_dtype, int64_t ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
+  return gemm_bf16_scaled(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, nullptr, stream);
+}
+
+// act_scale (or null): one factor per activation row, multiplied into the row factor in the epilogue: the rows are a
+// quantised math's activation images (act_images) and these their scales.
+int gemm_bf16_scaled(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w, const void* bias, int bias_dtype, void* y,
+                     int y_dtype, int64_t ld_y, int M, int N, int K, float alpha, float beta, const float* act_scale, void* stream) {
   if (M == 0 || N == 0) return kOk;
   if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(kInvalid);
   if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype) || (bias && !valid_dtype(bias_dtype))) return fail(kInvalid);
@@ -1130,6 +1143,7 @@ int gemm_bf16_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w,
   a.K = K;
   a.alpha = alpha;
   a.beta = beta;
+  a.act_scale = act_scale;
   const int xe = x_dtype == LX_BF16 ? 2 : 4, ye = y_dtype == LX_BF16 ? 2 : 4;
   hipStream_t s = as_stream(stream);
   switch (w.type) {
@@ -1245,6 +1259,37 @@ int gemm_bytes_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w
   return st;
 }
 
+// The FP8 math on NVFP4 weights and the FP4 math (engine/cpu/gemm.cpp:207-212,246-288): the activations are quantised
+// per token by the math's rule, their exact values go back into bf16 rows (an e4m3 value, or an e2m1 code times its e4m3
+// block scale, fits bf16), and the BF16-math kernels multiply those rows by the exactly expanded weights (exact products,
+// f32 sums; the reference sums them in double) with the rows' scales in the epilogue: t = (rowfactor * xscale) * sum.
+// Workspace as the reference lays it out: the scales first, the rows 64 bytes further (here: the bf16 images, then the
+// quantiser's bytes).
+int gemm_image_math(int math, const void* x, int x_dtype, int64_t ld_x, const lx_weight& w, const void* bias, int bias_dtype, void* y,
+                    int y_dtype, int64_t ld_y, int M, int N, int K, float alpha, float beta, void* workspace, void* stream) {
+  if (M == 0 || N == 0) return kOk;
+  if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(kInvalid);
+  if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype) || (bias && !valid_dtype(bias_dtype))) return fail(kInvalid);
+  if (w.type == LX_W_BF16X) return fail(kNotSupported);
+  if (!x || !y || !valid_weight(&w, K)) return fail(kInvalid);
+  if (math == LX_MATH_FP8 && w.type != LX_W_FP8 && w.type != LX_W_NVFP4) return fail(kNotSupported);
+  if (math == LX_MATH_FP4 && (w.type != LX_W_NVFP4 || K % 16 != 0)) return fail(kNotSupported);
+  hipStream_t s = as_stream(stream);
+  const int64_t head = (static_cast<int64_t>(M) * 4 + 63) / 64 * 64;
+  void* own = nullptr;
+  if (!workspace) {  // the reference falls back to scratch of its own
+    if (hipMallocAsync(&own, static_cast<size_t>(head + static_cast<int64_t>(M) * K * 4), s) != hipSuccess) return fail(kNoMemory);
+    workspace = own;
+  }
+  float* const scales = static_cast<float*>(workspace);
+  uint16_t* const xhat = reinterpret_cast<uint16_t*>(static_cast<char*>(workspace) + head);
+  uint8_t* const q = reinterpret_cast<uint8_t*>(xhat + static_cast<int64_t>(M) * K);
+  int st = act_images(x, x_dtype, ld_x, math, q, xhat, scales, M, K, s);
+  if (!st) st = gemm_bf16_scaled(xhat, LX_BF16, K, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, scales, stream);
+  if (own) (void)hipFreeAsync(own, s);
+  return st;
+}
+
 }  // namespace dro
 
 using namespace dro;
@@ -1267,9 +1312,10 @@ int lx_gemm_w(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, lx_
   if (math != LX_MATH_BF16 && math != LX_MATH_INT8 && math != LX_MATH_FP8 && math != LX_MATH_FP4) return fail(kInvalid);
   if (math == LX_MATH_INT8)
     return gemm_bytes_math<LX_MATH_INT8>(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, workspace, stream);
-  if (math == LX_MATH_FP8)
+  if (math == LX_MATH_FP8 && w->type != LX_W_NVFP4)
     return gemm_bytes_math<LX_MATH_FP8>(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, workspace, stream);
-  if (math != LX_MATH_BF16) return fail(kNotSupported);  // the BF16 math needs no workspace
+  if (math != LX_MATH_BF16)
+    return gemm_image_math(math, x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, workspace, stream);
   return gemm_bf16_math(x, x_dtype, ld_x, *w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
 }
 

@@ -41,16 +41,29 @@ int max_tiles(int P, int E) { return (P < E ? P : E) + P / kTileTokens + 1; }
 
 struct Layout {
   int64_t tables, inter, contrib, total;
+  // The quantised maths: the latent rows' images and scales (by token), the intermediate rows' (by position), and the
+  // quantiser's bytes.
+  int64_t image1, scale1, image2, scale2, qbytes;
 };
 
-Layout layout(int T, int L, int I, int E, int top_k) {
+Layout layout(int T, int L, int I, int E, int top_k, int math) {
   const int64_t P = static_cast<int64_t>(T) * top_k;
   const int64_t ints = (E + 1) + 2 * P + 3 * max_tiles(static_cast<int>(P), E) + 1;
-  Layout l;
+  auto up = [](int64_t b) { return (b + 255) / 256 * 256; };
+  Layout l{};
   l.tables = 0;
-  l.inter = (ints * 4 + 255) / 256 * 256;
-  l.contrib = l.inter + (P * I * 2 + 255) / 256 * 256;
-  l.total = l.contrib + (P * L * 4 + 255) / 256 * 256;
+  l.inter = up(ints * 4);
+  l.contrib = l.inter + up(P * I * 2);
+  l.total = l.contrib + up(P * L * 4);
+  if (math != LX_MATH_BF16) {
+    l.image1 = l.total;
+    l.scale1 = l.image1 + up(static_cast<int64_t>(T) * L * 2);
+    l.image2 = l.scale1 + up(static_cast<int64_t>(T) * 4);
+    l.scale2 = l.image2 + up(P * I * 2);
+    l.qbytes = l.scale2 + up(P * 4);
+    const int64_t q1 = static_cast<int64_t>(T) * (L + L / 16), q2 = P * (I + I / 16);
+    l.total = l.qbytes + up(q1 > q2 ? q1 : q2);
+  }
   return l;
 }
 
@@ -119,7 +132,10 @@ __global__ void __launch_bounds__(kMaxExperts) group_kernel(const int32_t* __res
 }
 
 struct GroupedArgs {
-  const uint16_t* latent;
+  const uint16_t* latent;  // bf16 [T, L]: the latent rows, or their images under a quantised math
+  const float* xs1;        // the latent rows' scales by token under a quantised math, else null
+  const uint16_t* down_in; // bf16 [P, I] by position: the intermediate rows, or their images
+  const float* xs2;        // the intermediate rows' scales by position, else null
   const float* weights;
   Stack gu, dn;
   Tables t;
@@ -150,11 +166,13 @@ __device__ __forceinline__ void gate_up_tile(const GroupedArgs& a, int e, int g0
     const int m = mt * 16 + (q & 15), i = i0 + 4 * (q >> 4);
     if (m >= rows) return;
     const int64_t stack_row = static_cast<int64_t>(e) * 2 * a.I + i;
+    // The activation row's scale under a quantised math (engine/cpu/moe.cpp:254-268: g = s_g * (xs * sum)).
+    const float xs = a.xs1 ? a.xs1[a.t.order[g0 + m] / a.top_k] : 1.0f;
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
       if (i + r < a.I) {
-        const float g = stack_factor(F, a.gu, e, stack_row + r) * sums[0][r];
-        const float u = stack_factor(F, a.gu, e, stack_row + a.I + r) * sums[1][r];
+        const float g = stack_factor(F, a.gu, e, stack_row + r) * (xs * sums[0][r]);
+        const float u = stack_factor(F, a.gu, e, stack_row + a.I + r) * (xs * sums[1][r]);
         a.inter[static_cast<int64_t>(g0 + m) * a.I + i + r] = f32_to_bf16_bits(silu(g) * u);
       }
     }
@@ -183,14 +201,15 @@ __device__ __forceinline__ void down_tile(const GroupedArgs& a, int e, int g0, i
   const TileRows tiles[1] = {{a.dn.data + row * a.row_bytes, a.dn.scale + row * a.scale_row_bytes, min(kTileRows, a.L - l0)}};
   const void* xrow[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xrow[mt] = a.inter + static_cast<int64_t>(g0 + min(mt * 16 + (lane & 15), rows - 1)) * a.I;
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = a.down_in + static_cast<int64_t>(g0 + min(mt * 16 + (lane & 15), rows - 1)) * a.I;
   mfma_tile<F, 1, MT, kXGlobalBf16>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.I, lds, blockDim.x / kWave, __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), [] {}, [&](int mt, int q, f32x4(&sums)[1]) {
     const int m = mt * 16 + (q & 15), l = l0 + 4 * (q >> 4);
     if (m >= rows) return;
     const int64_t stack_row = static_cast<int64_t>(e) * a.L + l;
+    const float xs = a.xs2 ? a.xs2[g0 + m] : 1.0f;  // engine/cpu/moe.cpp:304-309: c = rf * (xs * sum)
 #pragma unroll
     for (int r = 0; r < 4; ++r)
-      if (l + r < a.L) a.contrib[static_cast<int64_t>(g0 + m) * a.L + l + r] = stack_factor(F, a.dn, e, stack_row + r) * sums[0][r];
+      if (l + r < a.L) a.contrib[static_cast<int64_t>(g0 + m) * a.L + l + r] = stack_factor(F, a.dn, e, stack_row + r) * (xs * sums[0][r]);
   });
 }
 
@@ -260,15 +279,19 @@ int launch_stage(Kernel kernel, GroupedArgs a, int64_t K, int NT, int out_rows, 
 
 }  // namespace
 
-int64_t grouped_workspace_bytes(int T, int L, int I, int E, int top_k) {
+int64_t grouped_workspace_bytes(int T, int L, int I, int E, int top_k, int math) {
   if (T <= 0 || L <= 0 || I <= 0 || top_k <= 0 || E <= 0) return 0;
-  return layout(T, L, I, E, top_k).total;
+  return layout(T, L, I, E, top_k, math).total;
 }
 
+// math: LX_MATH_BF16, or a quantised math: then the latent rows are quantised per token and the intermediate rows per
+// pair by lx_quantize_act's rule, their exact values go back into bf16 rows (act_images) for the same matrix-core
+// kernels (exact products, f32 sums), and the rows' scales enter the epilogues as the reference applies them
+// (engine/cpu/moe.cpp:241-312).
 int experts_grouped(const void* latent, const int32_t* ids, const float* weights, const lx_weight& gate_up, const lx_weight& down,
-                    float* out, void* workspace, int T, int L, int I, int E, int top_k, hipStream_t s) {
+                    float* out, void* workspace, int T, int L, int I, int E, int top_k, int math, hipStream_t s) {
   const int P = T * top_k;
-  const Layout lay = layout(T, L, I, E, top_k);
+  const Layout lay = layout(T, L, I, E, top_k, math);
   char* ws = static_cast<char*>(workspace);
   GroupedArgs a{};
   a.latent = static_cast<const uint16_t*>(latent);
@@ -277,7 +300,9 @@ int experts_grouped(const void* latent, const int32_t* ids, const float* weights
   a.dn = as_stack(down);
   a.t = tables_at(ws + lay.tables, P, E);
   a.inter = reinterpret_cast<uint16_t*>(ws + lay.inter);
+  a.down_in = a.inter;
   a.contrib = reinterpret_cast<float*>(ws + lay.contrib);
+  const bool quantised = math != LX_MATH_BF16;
   a.out = out;
   a.T = T;
   a.L = L;
@@ -285,7 +310,9 @@ int experts_grouped(const void* latent, const int32_t* ids, const float* weights
   a.top_k = top_k;
   if (!tileable_any(gate_up.type, a.gu, L) || !tileable_any(down.type, a.dn, I) ||
       reinterpret_cast<uintptr_t>(latent) % 16 != 0) {
-    // Shapes the tiles cannot read 16 bytes at a time: the element-wise experts (pairs independent, any T).
+    // Shapes the tiles cannot read 16 bytes at a time: the element-wise experts (pairs independent, any T); they have
+    // the weight-only and BF16 maths only.
+    if (quantised) return fail(kNotSupported);
     DecodeArgs d{};
     d.latent = a.latent;
     d.ids = ids;
@@ -302,6 +329,13 @@ int experts_grouped(const void* latent, const int32_t* ids, const float* weights
   }
   hipLaunchKernelGGL(group_kernel, dim3(1), dim3(kMaxExperts), 0, s, ids, P, E, a.t);
   if (int st = status_of(hipGetLastError())) return st;
+  if (quantised) {
+    uint16_t* const image1 = reinterpret_cast<uint16_t*>(ws + lay.image1);
+    float* const scale1 = reinterpret_cast<float*>(ws + lay.scale1);
+    if (int st = act_images(latent, LX_BF16, L, math, reinterpret_cast<uint8_t*>(ws + lay.qbytes), image1, scale1, T, L, s)) return st;
+    a.latent = image1;
+    a.xs1 = scale1;
+  }
   const int tiles = max_tiles(P, E);
   int st;
   switch (gate_up.type) {
@@ -311,6 +345,15 @@ int experts_grouped(const void* latent, const int32_t* ids, const float* weights
     default: st = launch_stage<LX_W_NVFP4>(grouped_gate_up_kernel<LX_W_NVFP4>, a, L, 2, I, tiles, s); break;
   }
   if (st) return st;
+  if (quantised) {
+    // Every intermediate row is complete: quantise it again, per row (engine/cpu/moe.cpp:281-286). Positions past the
+    // pairs routed to experts in range hold nothing and are never read.
+    uint16_t* const image2 = reinterpret_cast<uint16_t*>(ws + lay.image2);
+    float* const scale2 = reinterpret_cast<float*>(ws + lay.scale2);
+    if ((st = act_images(a.inter, LX_BF16, I, math, reinterpret_cast<uint8_t*>(ws + lay.qbytes), image2, scale2, P, I, s))) return st;
+    a.down_in = image2;
+    a.xs2 = scale2;
+  }
   switch (down.type) {
     case LX_W_BF16: st = launch_stage<LX_W_BF16>(grouped_down_kernel<LX_W_BF16>, a, I, 1, L, tiles, s); break;
     case LX_W_INT8: st = launch_stage<LX_W_INT8>(grouped_down_kernel<LX_W_INT8>, a, I, 1, L, tiles, s); break;
@@ -337,16 +380,27 @@ int lx_moe_experts_grouped(const void* latent, const int32_t* ids, const float* 
   if (E <= 0 || !gate_up || !down) return fail(kInvalid);
   if (gate_up->type == LX_W_BF16X || down->type == LX_W_BF16X) return fail(kNotSupported);
   if (!valid_stack(*gate_up, L) || !valid_stack(*down, I)) return fail(kInvalid);
-  if (math != LX_MATH_BF16 && math != LX_MATH_INT8 && math != LX_MATH_FP8 && math != LX_MATH_FP4) return fail(kInvalid);
-  if (math != LX_MATH_BF16) return fail(kNotSupported);
+  switch (math) {  // engine/cpu/moe.cpp:555-569
+    case LX_MATH_BF16: break;
+    case LX_MATH_INT8:
+      if (gate_up->type != LX_W_INT8 || down->type != LX_W_INT8) return fail(kNotSupported);
+      break;
+    case LX_MATH_FP8:
+      if ((gate_up->type != LX_W_FP8 && gate_up->type != LX_W_NVFP4) || (down->type != LX_W_FP8 && down->type != LX_W_NVFP4))
+        return fail(kNotSupported);
+      break;
+    case LX_MATH_FP4:
+      if (gate_up->type != LX_W_NVFP4 || down->type != LX_W_NVFP4 || L % 16 || I % 16) return fail(kNotSupported);
+      break;
+    default: return fail(kInvalid);
+  }
   if (E > kMaxExperts) return fail(kNotSupported);
   if (!workspace) return fail(kInvalid);
-  return experts_grouped(latent, ids, weights, *gate_up, *down, out, workspace, T, L, I, E, top_k, as_stream(stream));
+  return experts_grouped(latent, ids, weights, *gate_up, *down, out, workspace, T, L, I, E, top_k, math, as_stream(stream));
 }
 
 int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int top_k, lx_math math) {
-  (void)math;
-  return grouped_workspace_bytes(T, L, I, E, top_k);
+  return grouped_workspace_bytes(T, L, I, E, top_k, math >= LX_MATH_INT8 && math <= LX_MATH_FP4 ? math : LX_MATH_BF16);
 }
 
 // The bf16-stack form without a workspace argument: the scratch is taken from and returned to the stream's
@@ -359,9 +413,9 @@ int lx_moe_experts(const void* latent, const int32_t* ids, const float* weights,
   const lx_weight gu{LX_W_BF16, gate_up, nullptr, 1.0f, nullptr}, dn{LX_W_BF16, down, nullptr, 1.0f, nullptr};
   hipStream_t s = as_stream(stream);
   void* ws = nullptr;
-  const int64_t bytes = grouped_workspace_bytes(T, L, I, kMaxExperts, top_k);
+  const int64_t bytes = grouped_workspace_bytes(T, L, I, kMaxExperts, top_k, LX_MATH_BF16);
   if (int st = status_of(hipMallocAsync(&ws, static_cast<size_t>(bytes), s))) return st;
-  const int st = experts_grouped(latent, ids, weights, gu, dn, out, ws, T, L, I, kMaxExperts, top_k, s);
+  const int st = experts_grouped(latent, ids, weights, gu, dn, out, ws, T, L, I, kMaxExperts, top_k, LX_MATH_BF16, s);
   const int fr = status_of(hipFreeAsync(ws, s));
   return st ? st : fr;
 }
@@ -411,7 +465,7 @@ int lx_moe_experts_noalloc(const void* latent, const int32_t* ids, const float* 
                            float* out, int T, int L, int I, int top_k, void* stream) {
   if (T <= 0) return kOk;
   if (!latent || !ids || !weights || !out || L <= 0 || I <= 0 || top_k < 1 || !gate_up || !down) return fail(kInvalid);
-  const int64_t bytes = grouped_workspace_bytes(T, L, I, kMaxExperts, top_k);
+  const int64_t bytes = grouped_workspace_bytes(T, L, I, kMaxExperts, top_k, LX_MATH_BF16);
   if (bytes > kScratchBytes) {
     fprintf(stderr, "lx_moe_experts_noalloc: T=%d L=%d I=%d top_k=%d needs %lld bytes of scratch, the fixed array holds %lld\n", T, L,
             I, top_k, static_cast<long long>(bytes), static_cast<long long>(kScratchBytes));
@@ -421,7 +475,7 @@ int lx_moe_experts_noalloc(const void* latent, const int32_t* ids, const float* 
   void* const ws = scratch_of_current_device(&st);
   if (!ws) return st;
   const lx_weight gu{LX_W_BF16, gate_up, nullptr, 1.0f, nullptr}, dn{LX_W_BF16, down, nullptr, 1.0f, nullptr};
-  return experts_grouped(latent, ids, weights, gu, dn, out, ws, T, L, I, kMaxExperts, top_k, as_stream(stream));
+  return experts_grouped(latent, ids, weights, gu, dn, out, ws, T, L, I, kMaxExperts, top_k, LX_MATH_BF16, as_stream(stream));
 }
 
 }  // extern "C"

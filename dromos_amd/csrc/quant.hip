@@ -326,6 +326,52 @@ int quantize_act_rows(const void* x, int x_dtype, int64_t ld_x, int math, void* 
   return status_of(hipGetLastError());
 }
 
+namespace {
+
+// xhat[m, k] = the value row m holds at k after its quantisation: the int8, the e4m3 value, or the e2m1 code times its
+// block's e4m3 scale, as bf16 (exact: eight, four and six significant bits). One thread per eight values.
+__global__ void __launch_bounds__(kThreads) act_values_kernel(const uint8_t* __restrict__ q, int64_t ld_q, const uint8_t* __restrict__ bs,
+                                                              int64_t ld_bs, int math, uint16_t* __restrict__ xhat, int64_t ld_o, int M,
+                                                              int K) {
+  const int per_row = (K + 7) / 8;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * kThreads + threadIdx.x;
+  if (item >= static_cast<int64_t>(M) * per_row) return;
+  const int64_t m = item / per_row;
+  const int k0 = static_cast<int>(item - m * per_row) * 8;
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    const int k = k0 + j;
+    if (k >= K) break;
+    float v;
+    if (math == LX_MATH_INT8) {
+      v = static_cast<float>(static_cast<int8_t>(q[m * ld_q + k]));
+    } else if (math == LX_MATH_FP8) {
+      v = e4m3_decode(q[m * ld_q + k]);
+    } else {
+      const uint32_t byte = q[m * ld_q + (k >> 1)];
+      v = e2m1_to_f32((k & 1) ? (byte >> 4) : (byte & 15u)) * e4m3_decode(bs[m * ld_bs + (k >> 4)]);
+    }
+    xhat[m * ld_o + k] = f32_to_bf16_bits(v);
+  }
+}
+
+}  // namespace
+
+// The rows of x [M, K] as a quantised math sees them: quantised per row by lx_quantize_act's rule for `math` (bytes into
+// `q`, M * (K + K / 16) of them at most; scales into scale [M]) and their values written back as bf16 rows xhat [M, K]
+// (exact). The matrix-core kernels then multiply xhat as they multiply any bf16 activations and apply the scales in
+// their epilogues.
+int act_images(const void* x, int x_dtype, int64_t ld_x, int math, uint8_t* q, uint16_t* xhat, float* scale, int M, int K,
+               hipStream_t stream) {
+  const int64_t ld_q = math == LX_MATH_FP4 ? K / 2 : K, ld_bs = K / 16;
+  uint8_t* const bs = q + static_cast<int64_t>(M) * ld_q;
+  if (int st = quantize_act_rows(x, x_dtype, ld_x, math, q, ld_q, scale, bs, ld_bs, M, K, stream)) return st;
+  const int64_t items = static_cast<int64_t>(M) * ((K + 7) / 8);
+  hipLaunchKernelGGL(act_values_kernel, dim3(static_cast<unsigned>((items + kThreads - 1) / kThreads)), dim3(kThreads), 0, stream, q, ld_q,
+                     bs, ld_bs, math, xhat, static_cast<int64_t>(K), M, K);
+  return status_of(hipGetLastError());
+}
+
 }  // namespace dro
 
 using namespace dro;

@@ -80,8 +80,10 @@ LX_API int lx_gemv_decode_bf16(const void* x, lx_dtype x_dtype, int ld_x, const 
  *                 the matrix cores; the workspace is not used (may be null)
  *   LX_MATH_INT8  int8 weights: activations quantised per token to int8 inside the call (lx_quantize_act's rule),
  *                 exact int32 sums; other weight formats answer 801
- *   LX_MATH_FP8   fp8 weights: activations quantised per token to e4m3, exact products, f32 sums
- *   LX_MATH_FP4 and LX_MATH_FP8 on NVFP4 weights answer 801.
+ *   LX_MATH_FP8   fp8 or NVFP4 weights: activations quantised per token to e4m3, exact products, f32 sums
+ *   LX_MATH_FP4   NVFP4 weights (K % 16 == 0): activations quantised per token to e2m1 with e4m3 block scales,
+ *                 exact products, f32 sums
+ * Any other pair of math and weight format answers 801 (engine/cpu/gemm.cpp:195-212).
  * The quantised maths keep the activations' scales and bytes in the workspace (lx_gemm_workspace_bytes); with a
  * null workspace they take scratch from the stream's memory pool instead (hipMallocAsync / hipFreeAsync, as the
  * reference's kernels do: such a call allocates and cannot be captured in a graph).
@@ -124,7 +126,10 @@ LX_API int lx_quantize_act(const void* x, lx_dtype x_dtype, int ld_x, lx_math ma
  * written once; the k terms are added in slot order. The pairs are grouped by expert on the device
  * (counting sort + prefix-summed offset table in the workspace): no host round trip.
  *   lx_moe_experts_decode   T <= 8, top_k <= 8, weight-only f32 math
- *   lx_moe_experts_grouped  any T, LX_MATH_BF16 on the matrix cores (other maths: 801), E <= 1024
+ *   lx_moe_experts_grouped  any T, on the matrix cores, E <= 1024; LX_MATH_BF16 on any stacks, LX_MATH_INT8 on int8
+ *                           stacks, LX_MATH_FP8 on fp8 or NVFP4 stacks, LX_MATH_FP4 on NVFP4 stacks (the latent rows are
+ *                           quantised per token and the intermediate rows per pair by lx_quantize_act's rule; other
+ *                           pairs answer 801, engine/cpu/moe.cpp:555-569)
  *   lx_moe_experts / lx_moe_experts_decode_bf16   the bf16-stack forms of the two */
 LX_API int lx_moe_route(const float* logits, const float* selection_bias, int32_t* ids, float* weights,
                         float* entropy, float* confidence, int T, int E, int top_k, void* stream);

@@ -502,42 +502,69 @@ static int gemm_int8_math(const void* x, int x_dtype, int64_t ld_x, const lx_wei
   return ORC_OK;
 }
 
-/* The FP8 math on fp8 weights (engine/cpu/gemm.cpp:207-209,246-288, Epilogue::apply_d :36-50): the activations are
- * quantised per token to e4m3 (lx_quantize_act's FP8 rule); the products of the two e4m3 values are exact and are
- * summed in double (exactly: at most 47 significant bits), and t = float(rowscale * xscale * sum) with the product in
- * double, before bias, alpha and beta in f32. NVFP4 weights under this math answer 801 in this build. Pinned bit for
+/* The value an activation row holds under the FP8 or FP4 math at element k: the e4m3 value, or the e2m1 code times
+ * its block's e4m3 scale (engine/cpu/gemm.cpp:270-277; exact in f32). */
+static float act_value(int math, const uint8_t* q, const uint8_t* bs, int64_t k) {
+  if (math == LX_MATH_FP8) return orc_e4m3_to_f32(q[k]);
+  const uint8_t b = q[k >> 1];
+  return orc_e2m1_to_f32((k & 1) ? (uint32_t)(b >> 4) : (uint32_t)(b & 15u)) * orc_e4m3_to_f32(bs[k >> 4]);
+}
+
+/* The FP8 math (fp8 or NVFP4 weights) and the FP4 math (NVFP4 weights) (engine/cpu/gemm.cpp:207-212,246-288,
+ * Epilogue::apply_d :36-50): the activations are quantised per token (lx_quantize_act's rule for the math); the
+ * products of the quantised activation values and the exact weight elements are summed in double (exactly), and
+ * t = float(rowfactor * xscale * sum) with the products in double, before bias, alpha and beta in f32. Pinned bit for
  * bit against oracle/_ref (tests/test_oracle_products.py). */
-static int gemm_fp8_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight* w, const void* bias, int bias_dtype,
-                         void* y, int y_dtype, int64_t ld_y, int64_t M, int64_t N, int64_t K, float alpha, float beta) {
+static int gemm_exact_math(int math, const void* x, int x_dtype, int64_t ld_x, const lx_weight* w, const void* bias, int bias_dtype,
+                           void* y, int y_dtype, int64_t ld_y, int64_t M, int64_t N, int64_t K, float alpha, float beta) {
   if (M == 0 || N == 0) return ORC_OK;
   if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(ORC_INVALID);
   if (!dtype_ok(x_dtype) || !dtype_ok(y_dtype) || (bias && !dtype_ok(bias_dtype))) return fail(ORC_INVALID);
   if (!x || !y || !weight_ok(w, K)) return fail(ORC_INVALID);
-  if (w->type != LX_W_FP8) return fail(ORC_UNSUPPORTED);
-  uint8_t* q = (uint8_t*)malloc((size_t)M * (size_t)K);
+  if (math == LX_MATH_FP8 && w->type != LX_W_FP8 && w->type != LX_W_NVFP4) return fail(ORC_UNSUPPORTED);
+  if (math == LX_MATH_FP4 && (w->type != LX_W_NVFP4 || K % 16 != 0)) return fail(ORC_UNSUPPORTED);
+  float* xv = (float*)malloc(sizeof(float) * (size_t)M * (size_t)K);
   float* xs = (float*)malloc(sizeof(float) * (size_t)M);
-  if (!q || !xs) {
-    free(q);
+  uint8_t* q = (uint8_t*)malloc((size_t)K + (size_t)K / 16 + 64);
+  if (!xv || !xs || !q) {
+    free(xv);
     free(xs);
+    free(q);
     return fail(ORC_NOMEM);
   }
-  for (int64_t m = 0; m < M; ++m) quant_act_row(x, x_dtype, m * ld_x, LX_MATH_FP8, (int)K, q + m * K, xs + m, NULL);
-  const uint8_t* wq = (const uint8_t*)w->data;
-  const float* rs = (const float*)w->scale;
-#pragma omp parallel for schedule(static)
-  for (int64_t n = 0; n < N; ++n)
-    for (int64_t m = 0; m < M; ++m) {
-      double sum = 0.0;
-      for (int64_t k = 0; k < K; ++k) sum += (double)orc_e4m3_to_f32(q[m * K + k]) * (double)orc_e4m3_to_f32(wq[n * K + k]);
-      float t = (float)((double)rs[n] * (double)xs[m] * sum);
-      if (bias) t += load_f32(bias, bias_dtype, n);
-      float v = alpha * t;
-      if (beta != 0.0f) v = beta * load_f32(y, y_dtype, m * ld_y + n) + v;
-      store_f32(y, y_dtype, m * ld_y + n, v);
+  for (int64_t m = 0; m < M; ++m) {
+    quant_act_row(x, x_dtype, m * ld_x, math, (int)K, q, xs + m, q + K);
+    for (int64_t k = 0; k < K; ++k) xv[m * K + k] = act_value(math, q, q + K, k);
+  }
+  int err = 0;
+#pragma omp parallel
+  {
+    float* row = (float*)malloc(sizeof(float) * (size_t)K);
+    if (!row) {
+#pragma omp atomic write
+      err = 1;
+    } else {
+#pragma omp for schedule(static)
+      for (int64_t n = 0; n < N; ++n) {
+        decode_row(w->type, w->data, w->scale, n, K, row);
+        const double rf = w->type == LX_W_NVFP4 ? (double)w->global : (double)((const float*)w->scale)[n];
+        for (int64_t m = 0; m < M; ++m) {
+          double sum = 0.0;
+          for (int64_t k = 0; k < K; ++k) sum += (double)xv[m * K + k] * (double)row[k];
+          float t = (float)(rf * (double)xs[m] * sum);
+          if (bias) t += load_f32(bias, bias_dtype, n);
+          float v = alpha * t;
+          if (beta != 0.0f) v = beta * load_f32(y, y_dtype, m * ld_y + n) + v;
+          store_f32(y, y_dtype, m * ld_y + n, v);
+        }
+      }
+      free(row);
     }
-  free(q);
+  }
+  free(xv);
   free(xs);
-  return ORC_OK;
+  free(q);
+  return err ? fail(ORC_NOMEM) : ORC_OK;
 }
 
 ORC_API int lx_gemm_w(const void* x, int x_dtype, int ld_x, const lx_weight* w, int math, const void* bias, int bias_dtype,
@@ -548,8 +575,8 @@ ORC_API int lx_gemm_w(const void* x, int x_dtype, int ld_x, const lx_weight* w, 
   if (!w) return fail(ORC_INVALID);
   if (math < LX_MATH_BF16 || math > LX_MATH_FP4) return fail(ORC_INVALID);
   if (math == LX_MATH_INT8) return gemm_int8_math(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
-  if (math == LX_MATH_FP8) return gemm_fp8_math(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
-  if (math != LX_MATH_BF16) return fail(ORC_UNSUPPORTED);
+  if (math == LX_MATH_FP8 || math == LX_MATH_FP4)
+    return gemm_exact_math(math, x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
   return gemm_bf16_math(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
 }
 
@@ -657,12 +684,57 @@ static float row_factor(const lx_weight* w, int64_t n) {
   return 1.0f;
 }
 
-/* Weight-only experts: for each (token, slot) pair, inter = bf16(silu(s_g * g) * (s_u * u)) with
- * g = gate_e . x, u = up_e . x (engine/cpu/moe.cpp:241-279, rounding point :267-270), contribution =
- * s_l * down_e . inter (:292-312), and out[t] = w0 * c0 + sum_{k >= 1} w_k * c_k in slot order
- * (:315-327). BF16 math on bf16 operands is the same arithmetic (exact products, f32 sums). */
+#define ORC_WEIGHT_ONLY (-1) /* the decode and legacy entries: f32 math on the activations as given */
+
+/* One pass's activation rows under a math (engine/cpu/moe.cpp:82-121): weight-only and BF16: the bf16 values; INT8:
+ * per-row int8 and a scale; FP8 / FP4: the quantised rows' exact values as f32 and a scale. */
+typedef struct {
+  float* f;     /* [rows, K] values (all maths but INT8) */
+  int8_t* i;    /* [rows, K] (INT8) */
+  float* scale; /* [rows], or NULL */
+  int64_t K;
+} orc_acts;
+
+static void acts_fill(orc_acts* a, int64_t r, const uint16_t* src, int math, uint8_t* tmp) {
+  const int64_t K = a->K;
+  if (math == ORC_WEIGHT_ONLY || math == LX_MATH_BF16) {
+    for (int64_t k = 0; k < K; ++k) a->f[r * K + k] = bf16_value(src[k]);
+    return;
+  }
+  if (math == LX_MATH_INT8) {
+    quant_act_row(src, LX_BF16, 0, LX_MATH_INT8, (int)K, (uint8_t*)(a->i + r * K), a->scale + r, NULL);
+    return;
+  }
+  quant_act_row(src, LX_BF16, 0, math, (int)K, tmp, a->scale + r, tmp + K);
+  for (int64_t k = 0; k < K; ++k) a->f[r * K + k] = act_value(math, tmp, tmp + K, k);
+}
+
+/* The dot of activation row r with a decoded weight row (wrow: f32 values; wq: the int8 bytes under the INT8 math):
+ * f32 lanes (weight-only, BF16), an exact int32 sum as f32 (INT8), or an exact double sum (FP8 / FP4)
+ * (engine/cpu/moe.cpp:125-154). */
+static double acts_dot(const orc_acts* a, int64_t r, const float* wrow, const int8_t* wq, int math) {
+  const int64_t K = a->K;
+  if (math == LX_MATH_INT8) {
+    int32_t sum = 0;
+    for (int64_t k = 0; k < K; ++k) sum += (int32_t)a->i[r * K + k] * (int32_t)wq[k];
+    return (double)(float)sum;
+  }
+  if (math == LX_MATH_FP8 || math == LX_MATH_FP4) {
+    double sum = 0.0;
+    for (int64_t k = 0; k < K; ++k) sum += (double)a->f[r * K + k] * (double)wrow[k];
+    return sum;
+  }
+  return (double)dot_f32(a->f + r * K, wrow, K);
+}
+
+/* The routed experts under a math (engine/cpu/moe.cpp:163-329): for each (token, slot) pair, inter =
+ * bf16(silu(s_g * (xs * g)) * (s_u * (xs * u))) with g = gate_e . x, u = up_e . x on the pair's activation row (the
+ * token's latent row, quantised per row under the INT8 / FP8 / FP4 maths: xs is its scale; :241-279, rounding point
+ * :267-270; under the FP8 / FP4 maths the whole SwiGLU is in double on the exact dots, :259-265); the intermediate row
+ * is quantised again per row once it is complete (:281-286); contribution = s_l * (xs2 * down_e . inter) (:292-312),
+ * and out[t] = w0 * c0 + sum_{k >= 1} w_k * c_k in slot order (:315-327). */
 static int experts(const uint16_t* latent, const int32_t* ids, const float* weights, const lx_weight* gu,
-                   const lx_weight* dn, float* out, int64_t T, int64_t L, int64_t I, int64_t top_k, int64_t E) {
+                   const lx_weight* dn, float* out, int64_t T, int64_t L, int64_t I, int64_t top_k, int64_t E, int math) {
   const int64_t P = T * top_k;
   if (E <= 0) {
     for (int64_t p = 0; p < P; ++p)
@@ -670,55 +742,88 @@ static int experts(const uint16_t* latent, const int32_t* ids, const float* weig
   }
   for (int64_t p = 0; p < P; ++p)
     if (ids[p] < 0 || ids[p] >= E) return fail(ORC_INVALID);
+  const int quantised = math == LX_MATH_INT8 || math == LX_MATH_FP8 || math == LX_MATH_FP4;
+  const int exact = math == LX_MATH_FP8 || math == LX_MATH_FP4;
+  const int int8 = math == LX_MATH_INT8;
   float* contrib = (float*)malloc(sizeof(float) * (size_t)P * (size_t)L);
-  float* xf = (float*)malloc(sizeof(float) * (size_t)T * (size_t)L);
-  if (!contrib || !xf) {
-    free(contrib);
-    free(xf);
-    return fail(ORC_NOMEM);
-  }
-  for (int64_t i = 0; i < T * L; ++i) xf[i] = bf16_value(latent[i]);
-  int err = 0;
-  /* Experts in turn; each expert's rows are decoded once for all the pairs that chose it. */
+  orc_acts x1 = {NULL, NULL, NULL, L}, x2 = {NULL, NULL, NULL, I};
+  x1.f = int8 ? NULL : (float*)malloc(sizeof(float) * (size_t)P * (size_t)L);
+  x1.i = int8 ? (int8_t*)malloc((size_t)P * (size_t)L) : NULL;
+  x2.f = int8 ? NULL : (float*)malloc(sizeof(float) * (size_t)P * (size_t)I);
+  x2.i = int8 ? (int8_t*)malloc((size_t)P * (size_t)I) : NULL;
+  x1.scale = quantised ? (float*)malloc(sizeof(float) * (size_t)P) : NULL;
+  x2.scale = quantised ? (float*)malloc(sizeof(float) * (size_t)P) : NULL;
+  uint16_t* staged = (uint16_t*)malloc(sizeof(uint16_t) * (size_t)P * (size_t)I); /* the bf16 intermediate, by pair */
+  const int64_t kmax = L > I ? L : I;
+  uint8_t* tmp = (uint8_t*)malloc((size_t)kmax + (size_t)kmax / 16 + 64);
+  int err = !contrib || !staged || !tmp || (int8 ? !x1.i || !x2.i : !x1.f || !x2.f) || (quantised && (!x1.scale || !x2.scale));
+  if (!err) {
+    /* Rows are kept by pair (the reference keeps them in grouped order; a row's content is the same). */
+    for (int64_t p = 0; p < P; ++p) acts_fill(&x1, p, latent + (p / top_k) * L, math, tmp);
+    /* Gate/up: experts in turn; each expert's rows are decoded once for all the pairs that chose it. */
 #pragma omp parallel for schedule(dynamic, 1)
-  for (int64_t e = 0; e < E; ++e) {
-    int64_t cnt = 0;
-    for (int64_t p = 0; p < P; ++p) cnt += ids[p] == e;
-    if (!cnt) continue;
-    lx_weight g = expert_slice(gu, e, 2 * I, L), d = expert_slice(dn, e, L, I);
-    float* wrow = (float*)malloc(sizeof(float) * (size_t)(L > I ? L : I));
-    float* gate = (float*)malloc(sizeof(float) * (size_t)cnt * (size_t)I * 2);
-    float* inter = (float*)malloc(sizeof(float) * (size_t)cnt * (size_t)I);
-    int64_t* pair = (int64_t*)malloc(sizeof(int64_t) * (size_t)cnt);
-    if (!wrow || !gate || !inter || !pair) {
+    for (int64_t e = 0; e < E; ++e) {
+      int64_t cnt = 0;
+      for (int64_t p = 0; p < P; ++p) cnt += ids[p] == e;
+      if (!cnt) continue;
+      lx_weight g = expert_slice(gu, e, 2 * I, L);
+      float* wg = (float*)malloc(sizeof(float) * (size_t)L);
+      float* wu = (float*)malloc(sizeof(float) * (size_t)L);
+      if (!wg || !wu) {
 #pragma omp atomic write
-      err = 1;
-    } else {
-      int64_t c = 0;
-      for (int64_t p = 0; p < P; ++p)
-        if (ids[p] == e) pair[c++] = p;
-      float* up = gate + cnt * I;
-      for (int64_t i = 0; i < 2 * I; ++i) {
-        decode_row(g.type, g.data, g.scale, i, L, wrow);
-        float rf = row_factor(&g, i);
-        for (int64_t r = 0; r < cnt; ++r) {
-          float s = rf * (1.0f * dot_f32(xf + (pair[r] / top_k) * L, wrow, L));
-          if (i < I) gate[r * I + i] = s;
-          else up[r * I + (i - I)] = s;
+        err = 1;
+      } else {
+        for (int64_t i = 0; i < I; ++i) {
+          decode_row(g.type, g.data, g.scale, i, L, wg);
+          decode_row(g.type, g.data, g.scale, I + i, L, wu);
+          const int8_t* qg = int8 ? (const int8_t*)g.data + i * L : NULL;
+          const int8_t* qu = int8 ? (const int8_t*)g.data + (I + i) * L : NULL;
+          const float sg = row_factor(&g, i), su = row_factor(&g, I + i);
+          for (int64_t p = 0; p < P; ++p) {
+            if (ids[p] != e) continue;
+            const float xs = x1.scale ? x1.scale[p] : 1.0f;
+            const double dg = acts_dot(&x1, p, wg, qg, math), du = acts_dot(&x1, p, wu, qu, math);
+            if (exact) {
+              const double gg = sg * ((double)xs * dg), uu = su * ((double)xs * du);
+              staged[p * I + i] = bf16_round((float)(gg / (1.0 + exp(-gg)) * uu));
+            } else {
+              const float gg = sg * (xs * (float)dg), uu = su * (xs * (float)du);
+              staged[p * I + i] = bf16_round(silu(gg) * uu);
+            }
+          }
         }
       }
-      for (int64_t r = 0; r < cnt; ++r)
-        for (int64_t i = 0; i < I; ++i) inter[r * I + i] = bf16_value(bf16_round(silu(gate[r * I + i]) * up[r * I + i]));
-      for (int64_t l = 0; l < L; ++l) {
-        decode_row(d.type, d.data, d.scale, l, I, wrow);
-        float rf = row_factor(&d, l);
-        for (int64_t r = 0; r < cnt; ++r) contrib[pair[r] * L + l] = rf * (1.0f * dot_f32(inter + r * I, wrow, I));
-      }
+      free(wg);
+      free(wu);
     }
-    free(wrow);
-    free(gate);
-    free(inter);
-    free(pair);
+  }
+  if (!err) {
+    for (int64_t p = 0; p < P; ++p) acts_fill(&x2, p, staged + p * I, math, tmp);
+#pragma omp parallel for schedule(dynamic, 1)
+    for (int64_t e = 0; e < E; ++e) {
+      int64_t cnt = 0;
+      for (int64_t p = 0; p < P; ++p) cnt += ids[p] == e;
+      if (!cnt) continue;
+      lx_weight d = expert_slice(dn, e, L, I);
+      float* wrow = (float*)malloc(sizeof(float) * (size_t)I);
+      if (!wrow) {
+#pragma omp atomic write
+        err = 1;
+      } else {
+        for (int64_t l = 0; l < L; ++l) {
+          decode_row(d.type, d.data, d.scale, l, I, wrow);
+          const int8_t* qd = int8 ? (const int8_t*)d.data + l * I : NULL;
+          const float rf = row_factor(&d, l);
+          for (int64_t p = 0; p < P; ++p) {
+            if (ids[p] != e) continue;
+            const float xs = x2.scale ? x2.scale[p] : 1.0f;
+            const double dd = acts_dot(&x2, p, wrow, qd, math);
+            contrib[p * L + l] = exact ? (float)(rf * ((double)xs * dd)) : rf * (xs * (float)dd);
+          }
+        }
+      }
+      free(wrow);
+    }
   }
   if (!err) {
     for (int64_t t = 0; t < T; ++t) {
@@ -732,7 +837,14 @@ static int experts(const uint16_t* latent, const int32_t* ids, const float* weig
     }
   }
   free(contrib);
-  free(xf);
+  free(x1.f);
+  free(x1.i);
+  free(x2.f);
+  free(x2.i);
+  free(x1.scale);
+  free(x2.scale);
+  free(staged);
+  free(tmp);
   return err ? fail(ORC_NOMEM) : ORC_OK;
 }
 
@@ -752,7 +864,7 @@ ORC_API int lx_moe_experts(const void* latent, const int32_t* ids, const float* 
   if (st) return st;
   if (!gate_up || !down) return fail(ORC_INVALID);
   lx_weight gu = {LX_W_BF16, gate_up, NULL, 1.0f, NULL}, dn = {LX_W_BF16, down, NULL, 1.0f, NULL};
-  return experts((const uint16_t*)latent, ids, weights, &gu, &dn, out, T, L, I, top_k, 0);
+  return experts((const uint16_t*)latent, ids, weights, &gu, &dn, out, T, L, I, top_k, 0, ORC_WEIGHT_ONLY);
 }
 
 /* engine/cpu/moe.cpp:496-503 */
@@ -776,10 +888,10 @@ ORC_API int lx_moe_experts_decode(const void* latent, const int32_t* ids, const 
   if (st) return st;
   if (!gate_up || !down) return fail(ORC_INVALID);
   if (!stack_ok(gate_up, L) || !stack_ok(down, I)) return fail(ORC_INVALID);
-  return experts((const uint16_t*)latent, ids, weights, gate_up, down, out, T, L, I, top_k, 0);
+  return experts((const uint16_t*)latent, ids, weights, gate_up, down, out, T, L, I, top_k, 0, ORC_WEIGHT_ONLY);
 }
 
-/* engine/cpu/moe.cpp:546-572; only the weight-only BF16 math is on this build's path. */
+/* engine/cpu/moe.cpp:546-572 */
 ORC_API int lx_moe_experts_grouped(const void* latent, const int32_t* ids, const float* weights, const lx_weight* gate_up,
                                    const lx_weight* down, int math, float* out, void* workspace, int T, int L, int I, int E,
                                    int top_k, void* stream) {
@@ -789,9 +901,21 @@ ORC_API int lx_moe_experts_grouped(const void* latent, const int32_t* ids, const
   int st = experts_args(latent, ids, weights, out, L, I, top_k);
   if (st) return st;
   if (E <= 0 || !gate_up || !down || !stack_ok(gate_up, L) || !stack_ok(down, I)) return fail(ORC_INVALID);
-  if (math < LX_MATH_BF16 || math > LX_MATH_FP4) return fail(ORC_INVALID);
-  if (math != LX_MATH_BF16) return fail(ORC_UNSUPPORTED);
-  return experts((const uint16_t*)latent, ids, weights, gate_up, down, out, T, L, I, top_k, E);
+  switch (math) {
+    case LX_MATH_BF16: break;
+    case LX_MATH_INT8:
+      if (gate_up->type != LX_W_INT8 || down->type != LX_W_INT8) return fail(ORC_UNSUPPORTED);
+      break;
+    case LX_MATH_FP8:
+      if ((gate_up->type != LX_W_FP8 && gate_up->type != LX_W_NVFP4) || (down->type != LX_W_FP8 && down->type != LX_W_NVFP4))
+        return fail(ORC_UNSUPPORTED);
+      break;
+    case LX_MATH_FP4:
+      if (gate_up->type != LX_W_NVFP4 || down->type != LX_W_NVFP4 || L % 16 || I % 16) return fail(ORC_UNSUPPORTED);
+      break;
+    default: return fail(ORC_INVALID);
+  }
+  return experts((const uint16_t*)latent, ids, weights, gate_up, down, out, T, L, I, top_k, E, math);
 }
 
 static int64_t round256(int64_t b) { return (b + 255) / 256 * 256; }
@@ -907,7 +1031,7 @@ ORC_API int lx_moe_experts_w8(const void* latent, const int32_t* ids, const floa
   if (st) return st;
   if (!gate_up || !gate_up_scale || !down || !down_scale) return fail(ORC_INVALID);
   lx_weight gu = {LX_W_INT8, gate_up, gate_up_scale, 1.0f, NULL}, dn = {LX_W_INT8, down, down_scale, 1.0f, NULL};
-  return experts((const uint16_t*)latent, ids, weights, &gu, &dn, out, T, L, I, top_k, 0);
+  return experts((const uint16_t*)latent, ids, weights, &gu, &dn, out, T, L, I, top_k, 0, ORC_WEIGHT_ONLY);
 }
 /* engine/cpu/moe.cpp:512-517 */
 ORC_API int64_t lx_moe_workspace_bytes(int T, int I, int top_k) {

@@ -127,11 +127,43 @@ def experts_decode(lx, fmt):
     return [latent, ids, weights, gu.data, dn.data], {"out": out}
 
 
-def experts_grouped(lx, fmt):
+def experts_grouped(lx, fmt, math=0):
     E, L, I, top_k, latent, ids, weights, gu, dn = _expert_inputs(fmt, 12)
     d = lx.device
-    out = ops.experts_grouped(lx, latent.to(d), ids.to(d), weights.to(d), gu.to(d), dn.to(d), I, E, top_k)
+    out = ops.experts_grouped(lx, latent.to(d), ids.to(d), weights.to(d), gu.to(d), dn.to(d), I, E, top_k, math=math)
     return [latent, ids, weights, gu.data, dn.data], {"out": out}
+
+
+def experts_w8(lx):
+    E, L, I, top_k, latent, ids, weights, gu, dn = _expert_inputs("int8", 11)
+    d = lx.device
+    out = ops.experts_w8(lx, latent.to(d), ids.to(d), weights.to(d), gu.to(d), dn.to(d), I, top_k)
+    return [latent, ids, weights, gu.data, dn.data], {"out": out}
+
+
+def router(lx):
+    M, E, K, top_k = 5, 48, 200, 6
+    g = torch.Generator().manual_seed(4800)
+    x = torch.randn(M, K, generator=g)
+    w = torch.randn(E, K, generator=g) / K**0.5
+    bias = torch.randn(E, generator=g) * 0.1
+    d = lx.device
+    logits = ops.spec_gemv_f32(lx, x.to(d), w.to(d), bias.to(d))
+    ids, weights, _, _ = ops.route(lx, logits, None, top_k)
+    emb = torch.randn(E, 40, generator=g).to(torch.bfloat16)
+    hist = torch.randn(M, 40, generator=g).to(d)
+    summary = ops.moe_summary(lx, ids, weights, emb.to(d), history=hist, a=0.75, b=0.25)
+    return [x, w, bias, emb], {"logits": logits, "ids": ids, "summary": summary, "history": hist}
+
+
+def gemm_bf16(lx):
+    M, N, K = 12, 48, 320
+    g = torch.Generator().manual_seed(4900)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) * 0.05).to(torch.bfloat16)
+    bias = torch.randn(N, generator=g).to(torch.bfloat16)
+    d = lx.device
+    return [x, w, bias], {"y": ops.gemm_bf16(lx, x.to(d), w.to(d), bias.to(d), alpha=1.5)}
 
 
 def experts_bf16(lx):
@@ -156,6 +188,13 @@ for _m, _n in ((1, "int8"), (2, "fp8"), (3, "fp4")):
 CASES["quantize_act_fp8_f32"] = (quantize_act, (2, torch.float32))
 CASES["gemm_int8_int8math"] = (gemm_math, ("int8", 1))
 CASES["gemm_fp8_fp8math"] = (gemm_math, ("fp8", 2))
+CASES["gemm_nvfp4_fp8math"] = (gemm_math, ("nvfp4", 2))
+CASES["gemm_nvfp4_fp4math"] = (gemm_math, ("nvfp4", 3))
+for _f, _m, _n in (("int8", 1, "int8"), ("fp8", 2, "fp8"), ("nvfp4", 2, "fp8"), ("nvfp4", 3, "fp4")):
+    CASES[f"experts_grouped_{_f}_{_n}math"] = (experts_grouped, (_f, _m))
+CASES["experts_w8"] = (experts_w8, ())
+CASES["router"] = (router, ())
+CASES["gemm_bf16"] = (gemm_bf16, ())
 CASES["route"] = (route, ())
 CASES["experts_bf16"] = (experts_bf16, ())
 

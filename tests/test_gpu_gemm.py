@@ -84,7 +84,11 @@ def test_other_maths_and_arguments(hip):
         assert ops.gemm_w(hip, x, w, math, status=True) == 801  # int8 weights take the BF16 and INT8 maths
     w8 = random_weight(FORMATS["fp8"], 32, 64, 1).to("cuda")
     assert ops.gemm_w(hip, x, w8, MATH_FP8, status=True) == 0
-    assert ops.gemm_w(hip, x, random_weight(FORMATS["nvfp4"], 32, 64, 1).to("cuda"), MATH_FP8, status=True) == 801  # not in this build
+    assert ops.gemm_w(hip, x, w8, MATH_FP4, status=True) == 801  # the FP4 math takes NVFP4 weights only
+    w4 = random_weight(FORMATS["nvfp4"], 32, 64, 1).to("cuda")
+    assert ops.gemm_w(hip, x, w4, MATH_FP8, status=True) == 0 and ops.gemm_w(hip, x, w4, MATH_FP4, status=True) == 0
+    assert ops.gemm_w(hip, x, w4, MATH_INT8, status=True) == 801
+    assert ops.gemm_w(hip, x, random_weight(FORMATS["bf16"], 32, 64, 1).to("cuda"), MATH_FP8, status=True) == 801
     assert ops.gemm_w(hip, x, w, MATH_INT8, status=True) == 0
     assert ops.gemm_w(hip, x, random_weight(FORMATS["fp8"], 32, 64, 1).to("cuda"), MATH_INT8, status=True) == 801  # int8 weights only
     assert ops.gemm_w(hip, x, w, 7, status=True) == 1
@@ -216,3 +220,51 @@ def test_fp8_math_rows_do_not_depend_on_the_batch(hip):
     for M in (1, 7, 16, 33):
         part = ops.gemm_w(hip, x[:M].contiguous(), w, MATH_FP8)
         assert torch.equal(part, full[:M]), M
+
+
+# ---- the FP8 math on NVFP4 weights and the FP4 math: quantised activations times exact weight values ----------
+
+
+@pytest.mark.parametrize("math", [MATH_FP8, MATH_FP4])
+@pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (5, 300, 4096), (12, 37, 1040), (16, 96, 512), (17, 2048, 1024), (40, 300, 528),
+                                   (64, 1024, 2048), (130, 50, 1040), (33, 21, 48)])
+def test_nvfp4_under_the_fp8_and_fp4_maths(hip, oracle, math, M, N, K, x_dtype, y_dtype):
+    g = torch.Generator().manual_seed(M * 7 + K + math)
+    x = torch.randn(M, K, generator=g).to(x_dtype)
+    x[M // 2] = 0
+    w = random_weight(FORMATS["nvfp4"], N, K, M + 3)
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g).to(y_dtype)
+    want = ops.gemm_w(oracle, x, w, math, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    got = ops.gemm_w(hip, x.cuda(), w.to("cuda"), math, bias=bias.cuda(), y=y0.clone().cuda(), alpha=1.25, beta=-0.5)
+    # The activations' quantised bytes are the oracle's bit for bit (tests/test_gpu_quant.py), the products are exact; the
+    # device sums them in f32 where the oracle sums in double: near 1e-6 (bf16 outputs: one rounding of the result).
+    err = rel_l2(got, want)
+    assert err <= (4e-3 if y_dtype == torch.bfloat16 else 1e-4), err
+
+
+@pytest.mark.parametrize("math", [MATH_FP8, MATH_FP4])
+def test_nvfp4_maths_rows_do_not_depend_on_the_batch(hip, math):
+    N, K = 2048, 4096
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(64, K, generator=g).to(torch.bfloat16).cuda()
+    w = random_weight(FORMATS["nvfp4"], N, K, 5).to("cuda")
+    full = ops.gemm_w(hip, x, w, math)
+    for M in (1, 7, 16, 33):
+        part = ops.gemm_w(hip, x[:M].contiguous(), w, math)
+        assert torch.equal(part, full[:M]), M
+
+
+def test_c3_shape_under_the_fp4_math(hip, oracle):
+    # W 4096 x 14336 NVFP4 (the NVFP4 GEMV configuration's weight), 8 rows, under the FP4 math against the oracle.
+    N, K, M = 4096, 14336, 8
+    g = torch.Generator().manual_seed(2008)
+    master = master_weight(N, K, g)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = quantize_with(hip, master.cuda(), FORMATS["nvfp4"])
+    got = ops.gemm_w(hip, x.cuda(), w, MATH_FP4)
+    want = ops.gemm_w(oracle, x, w.to("cpu"), MATH_FP4)
+    err = rel_l2(got, want)
+    assert err <= 1e-2 and err <= 1e-4, err

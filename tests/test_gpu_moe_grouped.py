@@ -114,3 +114,46 @@ def test_baseline_config_against_the_oracle(hip, oracle, T):
     want = ops.experts_grouped(oracle, latent, ids_o, weights_o, gu, dn, I, E, top_k)
     err = rel_l2(out.cpu(), want)
     assert err <= 1e-2 and err <= 2e-3, err
+
+
+# ---- the quantised maths: latent rows quantised per token, the intermediate per pair, both by lx_quantize_act's rule --
+
+GROUPED_MATHS = [("int8", MATH_INT8), ("fp8", MATH_FP8), ("nvfp4", MATH_FP8), ("nvfp4", MATH_FP4)]
+
+
+@pytest.mark.parametrize("fmt,math", GROUPED_MATHS)
+@pytest.mark.parametrize("T,L,I,E,top_k", [(5, 256, 256, 8, 2), (37, 512, 256, 16, 3), (96, 1024, 768, 64, 4)])
+def test_grouped_under_a_math_against_the_oracle(hip, oracle, fmt, math, T, L, I, E, top_k):
+    g = torch.Generator().manual_seed(T * 31 + E + math)
+    gu = checks.quantize_reference_stack(torch.randn(E, 2 * I, L, generator=g) / L**0.5, FORMATS[fmt])
+    dn = checks.quantize_reference_stack(torch.randn(E, L, I, generator=g) / I**0.5, FORMATS[fmt])
+    latent, ids, weights = checks.make_routing(T, E, L, top_k, T + 1)
+    want = ops.experts_grouped(oracle, latent, ids, weights, gu, dn, I, E, top_k, math=math)
+    got = ops.experts_grouped(hip, latent.cuda(), ids.cuda(), weights.cuda(), gu.to("cuda"), dn.to("cuda"), I, E, top_k, math=math)
+    # The device's exp and f32 sums differ from the oracle's in last bits; where that moves a bf16 intermediate value it
+    # can move its quantised code too (the coarser the math, the further): a tolerance, not bits.
+    err = rel_l2(got, want)
+    assert err <= 1e-2 and err <= (1e-2 if math == MATH_FP4 else 3e-3), err
+
+
+@pytest.mark.parametrize("fmt,math", GROUPED_MATHS)
+def test_grouped_under_a_math_rows_do_not_depend_on_the_batch(hip, fmt, math):
+    L, I, E, top_k = 1024, 512, 32, 4
+    latent, ids, weights, gu, dn = make(fmt, 40, L, I, E, top_k, 77)
+    full = ops.experts_grouped(hip, latent, ids, weights, gu, dn, I, E, top_k, math=math)
+    assert torch.equal(ops.experts_grouped(hip, latent, ids, weights, gu, dn, I, E, top_k, math=math), full)
+    for t in (0, 17, 39):
+        alone = ops.experts_grouped(hip, latent[t : t + 1].contiguous(), ids[t : t + 1].contiguous(),
+                                    weights[t : t + 1].contiguous(), gu, dn, I, E, top_k, math=math)
+        assert torch.equal(alone[0], full[t]), f"token {t} alone differs from the token in a batch of 40"
+
+
+def test_grouped_maths_and_formats_that_do_not_pair(hip):
+    from dromos_amd.formats import random_stack
+
+    T, E, L, I, top_k = 2, 4, 64, 32, 2
+    latent, ids, weights = (t.cuda() for t in checks.make_routing(T, E, L, top_k, 1))
+    for fmt, math, want in [("int8", 2, 801), ("fp8", 1, 801), ("bf16", 3, 801), ("nvfp4", 1, 801), ("fp8", 3, 801), ("nvfp4", 3, 0),
+                            ("int8", 1, 0), ("fp8", 2, 0), ("nvfp4", 2, 0), ("bf16", 7, 1)]:
+        gu, dn = random_stack(FORMATS[fmt], E, 2 * I, L, 3).to("cuda"), random_stack(FORMATS[fmt], E, L, I, 4).to("cuda")
+        assert ops.experts_grouped(hip, latent, ids, weights, gu, dn, I, E, top_k, math=math, status=True) == want, (fmt, math)

@@ -7,7 +7,7 @@ import torch
 
 import checks
 import ops
-from conftest import rel_l2
+from conftest import close, rel_l2
 from dromos_amd.abi import FORMATS
 from dromos_amd.formats import random_stack
 
@@ -79,3 +79,79 @@ def test_experts_equal_the_reference_generic_level(oracle, ref, fmt):
         assert rel_l2(a, b) < 1e-5  # the reference's BF16 math may take its bf16 dot instructions
     finally:
         ref.lib.lx_set_arch_override(0)
+
+
+GROUPED_MATHS = [("int8", 1), ("fp8", 2), ("nvfp4", 2), ("nvfp4", 3), ("bf16", 0)]
+
+
+def grouped_math_reference(latent, ids, weights, gu, dn, math):
+    """The routed experts under a quantised math from closed forms, in float64: per pair, the token's latent row
+    quantised by the per-row rule, gate and up as scale products of exact dots, SwiGLU, the bf16 intermediate quantised
+    again per row, down, and the weighted sum."""
+    import torch.nn.functional as F
+
+    from dromos_amd.formats import e2m1_table, e4m3_table, quantize_act_reference, unpack_codes
+
+    def values(rows):
+        if math == 0:
+            return rows.double(), torch.ones(rows.shape[0], dtype=torch.float64)
+        q, xs, bs = quantize_act_reference(rows, math)
+        if math == 1:
+            return q.view(torch.int8).double(), xs.double()
+        if math == 2:
+            return e4m3_table()[q.long()], xs.double()
+        return e2m1_table()[unpack_codes(q).long()] * e4m3_table()[bs.long()].repeat_interleave(16, dim=-1), xs.double()
+
+    I = gu.data.shape[1] // 2
+    gd, dd = gu.dense(), dn.dense()
+    xv, xs = values(latent)
+    out = torch.zeros(latent.shape, dtype=torch.float64)
+    for t in range(ids.shape[0]):
+        for k in range(ids.shape[1]):
+            e = int(ids[t, k])
+            g, u = xs[t] * (gd[e, :I] @ xv[t]), xs[t] * (gd[e, I:] @ xv[t])
+            mid = (F.silu(g) * u).to(torch.bfloat16)
+            mv, ms = values(mid.unsqueeze(0))
+            out[t] += weights[t, k].double() * ms[0] * (dd[e] @ mv[0])
+    return out
+
+
+@pytest.mark.parametrize("fmt,math", GROUPED_MATHS)
+def test_grouped_experts_under_a_math(oracle, fmt, math):
+    T, E, L, I, top_k = 9, 8, 128, 64, 3
+    g = torch.Generator().manual_seed(5 + math)
+    gu = checks.quantize_reference_stack(torch.randn(E, 2 * I, L, generator=g) / L**0.5, FORMATS[fmt])
+    dn = checks.quantize_reference_stack(torch.randn(E, L, I, generator=g) / I**0.5, FORMATS[fmt])
+    latent, ids, weights = checks.make_routing(T, E, L, top_k, 6)
+    out = ops.experts_grouped(oracle, latent, ids, weights, gu, dn, I, E, top_k, math=math)
+    want = grouped_math_reference(latent, ids, weights, gu, dn, math)
+    # The intermediate is rounded to bf16 and quantised again: a last-bit difference in a sum can move one of its
+    # values by a code, so the comparison with float64 is a tolerance, not bits.
+    close(out, want, atol=(2e-2 if math == 3 else 5e-3) * want.abs().max().item())
+    assert rel_l2(out, want) <= (3e-2 if math == 3 else 1e-2)
+
+
+@pytest.mark.parametrize("fmt,math", GROUPED_MATHS)
+def test_grouped_experts_under_a_math_equal_the_reference_generic_level(oracle, ref, fmt, math):
+    ref.lib.lx_set_arch_override(1)
+    try:
+        T, E, L, I, top_k = 7, 12, 256, 128, 4
+        gu, dn = random_stack(FORMATS[fmt], E, 2 * I, L, 71), random_stack(FORMATS[fmt], E, L, I, 72)
+        latent, ids, weights = checks.make_routing(T, E, L, top_k, 73)
+        a = ops.experts_grouped(oracle, latent, ids, weights, gu, dn, I, E, top_k, math=math)
+        b = ops.experts_grouped(ref, latent, ids, weights, gu, dn, I, E, top_k, math=math)
+        if math == 0:
+            assert rel_l2(a, b) < 1e-5  # the reference's BF16 math may take its bf16 dot instructions
+        else:
+            assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+    finally:
+        ref.lib.lx_set_arch_override(0)
+
+
+def test_grouped_maths_and_formats_that_do_not_pair(oracle):
+    T, E, L, I, top_k = 2, 4, 64, 32, 2
+    latent, ids, weights = checks.make_routing(T, E, L, top_k, 1)
+    for fmt, math, want in [("int8", 2, 801), ("fp8", 1, 801), ("bf16", 3, 801), ("nvfp4", 1, 801), ("fp8", 3, 801), ("nvfp4", 3, 0),
+                            ("int8", 1, 0), ("fp8", 2, 0), ("nvfp4", 2, 0), ("bf16", 7, 1)]:
+        gu, dn = random_stack(FORMATS[fmt], E, 2 * I, L, 3), random_stack(FORMATS[fmt], E, L, I, 4)
+        assert ops.experts_grouped(oracle, latent, ids, weights, gu, dn, I, E, top_k, math=math, status=True) == want, (fmt, math)

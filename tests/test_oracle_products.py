@@ -78,8 +78,8 @@ def test_gemm_w_bf16_math(oracle, fmt, M):
     want = ops.gemv_reference(x.to(torch.bfloat16), w.dense(), bias, 0.5, 0.0, None)
     checks.check_product(y, want)
     assert ops.gemm_w(oracle, x, w, MATH_INT8, status=True) == (0 if fmt == "int8" else 801)  # int8 weights only
-    assert ops.gemm_w(oracle, x, w, 2, status=True) == (0 if fmt == "fp8" else 801)  # fp8 weights only in this build
-    assert ops.gemm_w(oracle, x, w, 3, status=True) == 801  # the FP4 math is outside this path
+    assert ops.gemm_w(oracle, x, w, 2, status=True) == (0 if fmt in ("fp8", "nvfp4") else 801)  # fp8 or NVFP4 weights
+    assert ops.gemm_w(oracle, x, w, 3, status=True) == (0 if fmt == "nvfp4" else 801)  # NVFP4 weights only
     ys = ops.gemm_skinny(oracle, x.to(torch.bfloat16), w, bias=bias, alpha=0.5)
     assert torch.equal(ys, y)
 
@@ -202,3 +202,61 @@ def test_fp8_math_equals_the_reference_backend(oracle, ref, M, N, K):
     a = ops.gemm_w(oracle, x, w, 2, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
     b = ops.gemm_w(ref, x, w, 2, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
     assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+
+
+def exact_math_reference(x, w, math, bias, alpha, beta, y0):
+    """The FP8 math on NVFP4 weights and the FP4 math from closed forms: the activations' quantised values (the
+    per-token rules of quantize_act_reference) times the exact weight elements, summed in float64 (exactly),
+    t = float(global * xscale * sum), then the f32 epilogue."""
+    from dromos_amd.formats import e2m1_table, e4m3_table, quantize_act_reference, unpack_codes
+
+    q, xs, bs = quantize_act_reference(x, math)
+    if math == 2:
+        xv = e4m3_table()[q.long()]
+    else:
+        xv = e2m1_table()[unpack_codes(q).long()] * e4m3_table()[bs.long()].repeat_interleave(16, dim=-1)
+    elems = w.dense() / w.glob if w.fmt == 3 else w.dense() / w.scale.cpu().double().unsqueeze(-1)
+    rf = torch.full((elems.shape[0],), w.glob, dtype=torch.float64) if w.fmt == 3 else w.scale.cpu().double()
+    sums = xv @ elems.T
+    t = (rf.unsqueeze(0) * xs.double().unsqueeze(1) * sums).float()
+    if bias is not None:
+        t = t + bias.float()
+    v = alpha * t
+    if beta != 0.0:
+        v = beta * y0.float() + v
+    return v
+
+
+@pytest.mark.parametrize("fmt,math", [("nvfp4", 2), ("nvfp4", 3), ("fp8", 2)])
+@pytest.mark.parametrize("x_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (12, 37, 1040), (40, 300, 528)])
+def test_gemm_w_exact_maths(oracle, fmt, math, M, N, K, x_dtype):
+    g = torch.Generator().manual_seed(M + K)
+    x = torch.randn(M, K, generator=g).to(x_dtype)
+    x[M // 2] = 0
+    w = random_weight(FORMATS[fmt], N, K, M + 3, glob=0.25)  # a power of two: the element values come back exactly
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g)
+    y = ops.gemm_w(oracle, x, w, math, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    want = exact_math_reference(x, w, math, bias, 1.25, -0.5, y0)
+    assert torch.equal(y.view(torch.int32), want.view(torch.int32))
+
+
+@pytest.mark.parametrize("fmt,math", [("nvfp4", 2), ("nvfp4", 3)])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 1024), (12, 37, 1040), (40, 300, 528)])
+def test_exact_maths_equal_the_reference_backend(oracle, ref, fmt, math, M, N, K):
+    g = torch.Generator().manual_seed(K)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = random_weight(FORMATS[fmt], N, K, K + 1)
+    bias = torch.randn(N, generator=g)
+    y0 = torch.randn(M, N, generator=g)
+    a = ops.gemm_w(oracle, x, w, math, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    b = ops.gemm_w(ref, x, w, math, bias=bias, y=y0.clone(), alpha=1.25, beta=-0.5)
+    assert torch.equal(a.view(torch.int32), b.view(torch.int32))
+
+
+def test_maths_and_formats_that_do_not_pair(oracle):
+    x = torch.zeros(4, 64, dtype=torch.bfloat16)
+    for fmt, math, want in [("int8", 2, 801), ("int8", 3, 801), ("fp8", 1, 801), ("fp8", 3, 801), ("bf16", 1, 801), ("nvfp4", 1, 801),
+                            ("nvfp4", 2, 0), ("nvfp4", 3, 0), ("fp8", 2, 0), ("int8", 1, 0)]:
+        assert ops.gemm_w(oracle, x, random_weight(FORMATS[fmt], 32, 64, 1), math, status=True) == want, (fmt, math)
