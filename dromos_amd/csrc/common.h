@@ -129,6 +129,14 @@ struct Fmt<LX_W_NVFP4> {
   static constexpr int kBitsPerK = 4;
 };
 
+// LX_W_BF16X: eight values a lane and step, as bf16; a row record is a header and 192-byte blocks of 128 values
+// (bf16x.h). A lane's loads are 8 bytes of sign|mantissa, 4 bytes of codes and the block's base exponent.
+template <>
+struct Fmt<LX_W_BF16X> {
+  static constexpr int kElems = 8;
+  static constexpr int kBitsPerK = 16;  // once decoded: the products are bf16's
+};
+
 // A dword as two bf16 (low half first). Taking the dword by value matters: a bit cast written directly on an
 // element of a vector, `__builtin_bit_cast(bf16x2, v[i])`, has compiled to element 0 for every i.
 __device__ __forceinline__ bf16x2 as_bf16x2(uint32_t d) { return __builtin_bit_cast(bf16x2, d); }
@@ -146,6 +154,10 @@ template <>
 __device__ __forceinline__ void decode_dword<LX_W_BF16>(uint32_t d, float* out) {
   out[0] = __uint_as_float(d << 16);
   out[1] = __uint_as_float(d & 0xffff0000u);
+}
+template <>
+__device__ __forceinline__ void decode_dword<LX_W_BF16X>(uint32_t d, float* out) {
+  decode_dword<LX_W_BF16>(d, out);
 }
 template <>
 __device__ __forceinline__ void decode_dword<LX_W_INT8>(uint32_t d, float* out) {
@@ -185,6 +197,16 @@ __device__ __forceinline__ void decode_dword<LX_W_NVFP4>(uint32_t d, float* out)
 template <int F>
 __host__ __device__ inline int64_t row_bytes(int64_t K) {
   return K * Fmt<F>::kBitsPerK / 8;
+}
+template <>
+__host__ __device__ inline int64_t row_bytes<LX_W_BF16X>(int64_t K) {
+  const int64_t blocks = (K + 127) / 128;
+  return (4 * (2 + K / 2048) + blocks + 7) / 8 * 8 + 192 * blocks;
+}
+// The 16-byte (BF16X: eight-value) chunks a lane may take of a row of K values.
+template <int F>
+__host__ __device__ inline int chunks_of(int64_t K) {
+  return static_cast<int>(F == LX_W_BF16X ? K / 8 : row_bytes<F>(K) / 16);
 }
 __host__ __device__ inline int64_t row_bytes_of(int type, int64_t K) {
   return type == LX_W_BF16 ? 2 * K : type == LX_W_NVFP4 ? K / 2 : K;

@@ -1299,6 +1299,8 @@ extern "C" {
 int lx_gemv_w(const void* x, lx_dtype x_dtype, int ld_x, const lx_weight* w, const void* bias, lx_dtype bias_dtype, void* y,
               lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
   if (!w) return fail(kInvalid);
+  // engine/cpu/gemm.cpp:356-357: lossless rows have their own entry point.
+  if (w->type == LX_W_BF16X) return lx_gemv_bf16x(x, x_dtype, ld_x, w->data, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
   // Batch-invariant mode: bf16 activations take the matrix-core kernel, whose sums are the same for every row
   // count from 1 up (lx_gemm_w runs the same kernel). f32 activations keep the exact f32 product.
   if (batch_invariant() && x_dtype == LX_BF16 && M >= 1 && M <= 8 && N > 0)

@@ -16,7 +16,8 @@ namespace dro {
 bool gemv_admits(int wtype, int variant, int N, int K) {
   int S = 1;
   switch (wtype) {
-    case LX_W_BF16: S = order_class<LX_W_BF16>(N, K, 2); break;
+    case LX_W_BF16:
+    case LX_W_BF16X: S = order_class<LX_W_BF16>(N, K, 2); break;
     case LX_W_INT8: S = order_class<LX_W_INT8>(N, K, 2); break;
     case LX_W_FP8: S = order_class<LX_W_FP8>(N, K, 2); break;
     default: S = order_class<LX_W_NVFP4>(N, K, 2); break;
@@ -31,9 +32,12 @@ int gemv_any(const void* x, int x_dtype, int ld_x, const lx_weight& w, const voi
   if (M < 0 || M > 8 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(kInvalid);
   if (!valid_dtype(x_dtype) || !valid_dtype(y_dtype) || !valid_dtype(bias_dtype)) return fail(kInvalid);
   if (!x || !y || !w.data) return fail(kInvalid);
-  if (w.type == LX_W_BF16X) return fail(kNotSupported);
-  if (w.type != LX_W_BF16 && w.type != LX_W_INT8 && w.type != LX_W_FP8 && w.type != LX_W_NVFP4) return fail(kInvalid);
-  if (w.type != LX_W_BF16 && !w.scale) return fail(kInvalid);
+  if (w.type == LX_W_BF16X) {
+    if (K >= bf16x::kMaxK) return fail(kInvalid);
+  } else {
+    if (w.type != LX_W_BF16 && w.type != LX_W_INT8 && w.type != LX_W_FP8 && w.type != LX_W_NVFP4) return fail(kInvalid);
+    if (w.type != LX_W_BF16 && !w.scale) return fail(kInvalid);
+  }
   if (w.type == LX_W_NVFP4 && K % 16 != 0) return fail(kInvalid);
   GemvArgs a{};
   a.x = x;
@@ -58,6 +62,7 @@ int gemv_any(const void* x, int x_dtype, int ld_x, const lx_weight& w, const voi
     case LX_W_BF16: return gemv_launch_bf16(a, s);
     case LX_W_INT8: return gemv_launch_int8(a, s);
     case LX_W_FP8: return gemv_launch_fp8(a, s);
+    case LX_W_BF16X: return gemv_launch_bf16x(a, s);
     default: return gemv_launch_nvfp4(a, s);
   }
 }
@@ -75,6 +80,15 @@ int lx_gemv(const void* x, lx_dtype x_dtype, int ld_x, const void* w, lx_wtype w
   if (w_type != LX_W_BF16 && w_type != LX_W_INT8) return fail(kInvalid);
   if (w_type == LX_W_INT8 && !w_scale && M > 0 && N > 0) return fail(kInvalid);
   const lx_weight wt{w_type, w, w_scale, 1.0f, nullptr};
+  return gemv_any(x, x_dtype, ld_x, wt, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
+}
+
+// engine/cpu/gemm.cpp:364-371: the bf16 product on the encoded rows; the kernel decodes a lane's eight values to the
+// bf16 bits the bf16 kernel loads, in the same lanes and steps, so y is lx_gemv's on the original weights to the bit.
+int lx_gemv_bf16x(const void* x, lx_dtype x_dtype, int ld_x, const void* w, const void* bias, lx_dtype bias_dtype, void* y,
+                  lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
+  if (M != 0 && N != 0 && (reinterpret_cast<uintptr_t>(w) & 7) != 0) return fail(kInvalid);
+  const lx_weight wt{LX_W_BF16X, w, nullptr, 1.0f, nullptr};
   return gemv_any(x, x_dtype, ld_x, wt, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
 }
 

@@ -19,7 +19,7 @@ struct GemvArgs {
   int x_dtype;
   int64_t ld_x;
   const uint8_t* w;
-  const uint8_t* scale;  // f32 [N] (INT8 / FP8) or e4m3 [N, K / 16] (NVFP4)
+  const uint8_t* scale;  // f32 [N] (INT8 / FP8) or e4m3 [N, K / 16] (NVFP4); BF16X streamed: the first row's span tops
   float global;
   const void* bias;
   int bias_dtype;
@@ -34,9 +34,9 @@ struct GemvArgs {
   int split_log2;
   int steps;           // wave steps covering K
   int steps_per_part;  // ceil(steps / S)
-  int chunks;          // 16-byte chunks in a row
+  int chunks;          // 16-byte chunks in a row (BF16X: groups of eight values)
   int64_t row_bytes;
-  int64_t scale_row_bytes;  // NVFP4: bytes of block scales per row
+  int64_t scale_row_bytes;  // NVFP4: bytes of block scales per row; BF16X: a whole record
   int phase_steps;  // > 0: the activation image holds this many steps at a time (two images in turn), else all
 };
 
@@ -117,6 +117,7 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs
   };
 
   RowStreamer<F, MT, R, U, XB, ONE> st(a.chunks, s_begin, s_end, per_row);
+  if constexpr (F == LX_W_BF16X) st.set_bf16x(static_cast<int>(a.K));
   auto stage_all = [&] {
     if constexpr (XB) stage_x_pairs<F, MT>(reinterpret_cast<uint32_t*>(xs), static_cast<const uint16_t*>(a.x), a.ld_x, nullptr, a.M, a.K, steps);
     else stage_x<F, MT>(xs, a.x, a.x_dtype, a.ld_x, nullptr, a.M, a.K, steps);
@@ -170,7 +171,7 @@ __global__ void __launch_bounds__(kThreads) gemv_plain_kernel(const GemvArgs a, 
 #pragma unroll
   for (int m = 0; m < 8; ++m) acc[m] = 0.0f;
   for (int64_t k = lane; k < a.K; k += kWave) {
-    const float w = weight_element(wtype, a.w, a.scale, n, k, a.K);
+    const float w = weight_element_any(wtype, a.w, a.scale, n, k, a.K);
 #pragma unroll
     for (int m = 0; m < 8; ++m)
       if (m < a.M) acc[m] = __builtin_fmaf(load_as_f32(a.x, a.x_dtype, m * a.ld_x + k), w, acc[m]);
@@ -258,8 +259,10 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
   constexpr int R = 2;  // the order class counts row groups of two
   const int64_t rb = row_bytes<F>(a.K);
   const int steps = steps_for<F>(a.K);
-  const bool vector_rows = rb % 16 == 0 && reinterpret_cast<uintptr_t>(a.w) % 16 == 0 &&
-                           (F != LX_W_NVFP4 || reinterpret_cast<uintptr_t>(a.scale) % 2 == 0);
+  // BF16X: a lane's loads are 8 and 4 bytes within 8-byte aligned records, eight values at a time.
+  const bool vector_rows = F == LX_W_BF16X ? a.K % 8 == 0 && reinterpret_cast<uintptr_t>(a.w) % 8 == 0
+                                           : rb % 16 == 0 && reinterpret_cast<uintptr_t>(a.w) % 16 == 0 &&
+                                                 (F != LX_W_NVFP4 || reinterpret_cast<uintptr_t>(a.scale) % 2 == 0);
   // Activation rows a pass can hold in LDS: a function of K only. More rows than that run as several
   // passes over the weights; each row's arithmetic is the same in any pass, so its bits do not change.
   const bool xb = a.x_dtype == LX_BF16;
@@ -291,9 +294,12 @@ int launch_format(GemvArgs& a, const char* kernel_name, hipStream_t stream) {
   a.split_log2 = a.split == 4 ? 2 : a.split == 2 ? 1 : 0;
   a.steps = steps;
   a.steps_per_part = (steps + a.split - 1) / a.split;
-  a.chunks = static_cast<int>(rb / 16);
+  const RowBase<F> base(a.w, a.scale, a.K);
+  a.w = base.data;
+  a.scale = base.scale;
+  a.chunks = base.chunks;
   a.row_bytes = rb;
-  a.scale_row_bytes = F == LX_W_NVFP4 ? a.K / 16 : 0;
+  a.scale_row_bytes = base.scale_row;
   const int M = a.M, phase_steps = a.phase_steps;
   const char* x0 = static_cast<const char*>(a.x);
   char* y0 = static_cast<char*>(a.y);
@@ -328,5 +334,6 @@ int gemv_launch_bf16(GemvArgs& a, hipStream_t stream);
 int gemv_launch_int8(GemvArgs& a, hipStream_t stream);
 int gemv_launch_fp8(GemvArgs& a, hipStream_t stream);
 int gemv_launch_nvfp4(GemvArgs& a, hipStream_t stream);
+int gemv_launch_bf16x(GemvArgs& a, hipStream_t stream);
 
 }  // namespace dro

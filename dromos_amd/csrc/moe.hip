@@ -198,9 +198,9 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
                                              const int* s_rows) {
   const int steps = steps_for<F>(a.L);
   const int per_row = x_row_words<F, true>(steps);  // the packed bf16 image: the latent rows are bf16
-  const int64_t rb = row_bytes<F>(a.L);
-  const int chunks = static_cast<int>(rb / 16);
-  const int64_t scale_row = F == LX_W_NVFP4 ? a.L / 16 : 0;
+  const RowBase<F> base(a.gu.data, a.gu.scale, a.L);
+  const int64_t rb = base.rb, scale_row = base.scale_row;
+  const int chunks = base.chunks;
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int64_t stack_row0 = static_cast<int64_t>(e) * 2 * a.I;
   const int i = blockIdx.x * (blockDim.x / kWave) + wave;
@@ -209,10 +209,10 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
   const float sg = stack_factor(F, a.gu, e, my_gate_row), su = stack_factor(F, a.gu, e, my_gate_row + a.I);
   auto rows_fn = [&](int ii, const uint8_t* (&rows)[2], const uint8_t* (&scales)[2], const float* (&x_image)[2]) {
     const int64_t gate_row = stack_row0 + min(ii, a.I - 1), up_row = gate_row + a.I;
-    rows[0] = a.gu.data + gate_row * rb;
-    rows[1] = a.gu.data + up_row * rb;
-    scales[0] = a.gu.scale + gate_row * scale_row;
-    scales[1] = a.gu.scale + up_row * scale_row;
+    rows[0] = base.data + gate_row * rb;
+    rows[1] = base.data + up_row * rb;
+    scales[0] = base.scale + gate_row * scale_row;
+    scales[1] = base.scale + up_row * scale_row;
     x_image[0] = lds;
     x_image[1] = lds;
   };
@@ -234,6 +234,7 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
     }
   };
   RowStreamer<F, MT, 2, U, true, ONE> st(chunks, 0, steps, per_row);
+  if constexpr (F == LX_W_BF16X) st.set_bf16x(a.L);
   uint32_t* const image = reinterpret_cast<uint32_t*>(lds);
   if constexpr (MT == 1) {
     // Ask for x, then for the weights, and only then wait for x: loads return in order.
@@ -302,9 +303,9 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
   if (lblock >= n_lblocks) return;
   const int steps = steps_for<F>(a.I);
   const int per_row = x_row_words<F, true>(steps);  // the packed bf16 image: the intermediate rows are bf16
-  const int64_t rb = row_bytes<F>(a.I);
-  const int chunks = static_cast<int>(rb / 16);
-  const int64_t scale_row = F == LX_W_NVFP4 ? a.I / 16 : 0;
+  const RowBase<F> base(a.dn.data, a.dn.scale, a.I);
+  const int64_t rb = base.rb, scale_row = base.scale_row;
+  const int chunks = base.chunks;
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int top_k = a.top_k;
   const int l = lblock * (blockDim.x / kWave) + wave;
@@ -323,8 +324,8 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
       const int k = min(c * R + r, top_k - 1);
       const int e = __builtin_amdgcn_readlane(my_e, k);
       const int64_t row = static_cast<int64_t>(e) * a.L + lc;
-      rows[r] = a.dn.data + row * rb;
-      scales[r] = a.dn.scale + row * scale_row;
+      rows[r] = base.data + row * rb;
+      scales[r] = base.scale + row * scale_row;
       x_image[r] = lds + k * per_row;
     }
   };
@@ -343,6 +344,7 @@ __global__ void __launch_bounds__(kThreads) decode_down_kernel(const DecodeArgs 
   };
   const int n_groups = (top_k + R - 1) / R;
   RowStreamer<F, 1, R, U, true> st(chunks, 0, steps, per_row);
+  if constexpr (F == LX_W_BF16X) st.set_bf16x(a.I);
   // Ask for the intermediate rows, then for the weights, and only then wait for the rows: loads return in order.
   const uint16_t* const rows_of_t = a.inter + static_cast<int64_t>(t) * top_k * a.I;  // the token's top_k rows, in slot order
   XRowRegs xr;
@@ -368,8 +370,8 @@ __global__ void __launch_bounds__(kThreads) decode_gate_up_plain_kernel(const De
   float g = 0.0f, u = 0.0f;
   for (int k = lane; k < a.L; k += kWave) {
     const float x = bf16_bits_to_f32(a.latent[static_cast<int64_t>(t) * a.L + k]);
-    g = __builtin_fmaf(x, weight_element(type, a.gu.data, a.gu.scale, gate_row, k, a.L), g);
-    u = __builtin_fmaf(x, weight_element(type, a.gu.data, a.gu.scale, up_row, k, a.L), u);
+    g = __builtin_fmaf(x, weight_element_any(type, a.gu.data, a.gu.scale, gate_row, k, a.L), g);
+    u = __builtin_fmaf(x, weight_element_any(type, a.gu.data, a.gu.scale, up_row, k, a.L), u);
   }
   g = stack_factor(type, a.gu, e, gate_row) * wave_sum(g);
   u = stack_factor(type, a.gu, e, up_row) * wave_sum(u);
@@ -388,7 +390,7 @@ __global__ void __launch_bounds__(kThreads) decode_down_plain_kernel(const Decod
     float s = 0.0f;
     for (int j = lane; j < a.I; j += kWave)
       s = __builtin_fmaf(bf16_bits_to_f32(a.inter[static_cast<int64_t>(pair) * a.I + j]),
-                         weight_element(type, a.dn.data, a.dn.scale, row, j, a.I), s);
+                         weight_element_any(type, a.dn.data, a.dn.scale, row, j, a.I), s);
     const float wc = a.weights[pair] * (stack_factor(type, a.dn, e, row) * wave_sum(s));
     o = k == 0 ? wc : o + wc;
   }
@@ -399,8 +401,10 @@ template <int F>
 bool streamable(const Stack& s, int64_t K, int max_rows) {
   const int64_t rb = row_bytes<F>(K);
   const int steps = steps_for<F>(K);
-  return rb % 16 == 0 && reinterpret_cast<uintptr_t>(s.data) % 16 == 0 &&
-         (F != LX_W_NVFP4 || reinterpret_cast<uintptr_t>(s.scale) % 2 == 0) &&
+  const bool vector_rows = F == LX_W_BF16X ? K % 8 == 0 && reinterpret_cast<uintptr_t>(s.data) % 8 == 0
+                                           : rb % 16 == 0 && reinterpret_cast<uintptr_t>(s.data) % 16 == 0 &&
+                                                 (F != LX_W_NVFP4 || reinterpret_cast<uintptr_t>(s.scale) % 2 == 0);
+  return vector_rows &&
          static_cast<int64_t>(max_rows) * x_row_words<F, true>(steps) * 4 <= 128 * 1024;
 }
 
@@ -489,6 +493,7 @@ int experts_decode(const void* latent, const int32_t* ids, const float* weights,
   auto can_stream = [](int type, const Stack& st, int64_t K) {
     switch (type) {
       case LX_W_BF16: return streamable<LX_W_BF16>(st, K, 8);
+      case LX_W_BF16X: return streamable<LX_W_BF16X>(st, K, 8);
       case LX_W_INT8: return streamable<LX_W_INT8>(st, K, 8);
       case LX_W_FP8: return streamable<LX_W_FP8>(st, K, 8);
       default: return streamable<LX_W_NVFP4>(st, K, 8);
@@ -504,6 +509,7 @@ int experts_decode(const void* latent, const int32_t* ids, const float* weights,
   } else {
     switch (gate_up.type) {
       case LX_W_BF16: st = launch_gate_up<LX_W_BF16>(a, s); break;
+      case LX_W_BF16X: st = launch_gate_up<LX_W_BF16X>(a, s); break;
       case LX_W_INT8: st = launch_gate_up<LX_W_INT8>(a, s); break;
       case LX_W_FP8: st = launch_gate_up<LX_W_FP8>(a, s); break;
       default: st = launch_gate_up<LX_W_NVFP4>(a, s); break;
@@ -513,6 +519,7 @@ int experts_decode(const void* latent, const int32_t* ids, const float* weights,
   if (!can_stream(down.type, a.dn, I)) return down_plain(a, down.type, s);
   switch (down.type) {
     case LX_W_BF16: return launch_down<LX_W_BF16>(a, s);
+    case LX_W_BF16X: return launch_down<LX_W_BF16X>(a, s);
     case LX_W_INT8: return launch_down<LX_W_INT8>(a, s);
     case LX_W_FP8: return launch_down<LX_W_FP8>(a, s);
     default: return launch_down<LX_W_NVFP4>(a, s);
@@ -556,7 +563,11 @@ int lx_moe_experts_decode(const void* latent, const int32_t* ids, const float* w
   if (T > 8 || top_k > 8) return fail(kInvalid);
   if (!latent || !ids || !weights || !out || L <= 0 || I <= 0 || top_k < 1) return fail(kInvalid);
   if (!gate_up || !down || !workspace) return fail(kInvalid);
-  if (gate_up->type == LX_W_BF16X || down->type == LX_W_BF16X) return fail(kNotSupported);
+  if (gate_up->type == LX_W_BF16X || down->type == LX_W_BF16X) {
+    // engine/cpu/moe.cpp:528-533: both stacks encoded, or no kernel.
+    if (gate_up->type != LX_W_BF16X || down->type != LX_W_BF16X) return fail(kNotSupported);
+    return lx_moe_experts_bf16x(latent, ids, weights, gate_up->data, down->data, out, workspace, T, L, I, top_k, stream);
+  }
   if (!valid_stack(*gate_up, L) || !valid_stack(*down, I)) return fail(kInvalid);
   return experts_decode(latent, ids, weights, *gate_up, *down, out, workspace, T, L, I, top_k, as_stream(stream));
 }
@@ -569,12 +580,40 @@ int64_t lx_moe_decode_workspace_bytes(int T, int I, int top_k) {
 
 int64_t lx_moe_bf16x_workspace_bytes(int T, int I, int top_k) { return lx_moe_decode_workspace_bytes(T, I, top_k); }
 
+// The decode kernels on a pair of stacks of one format for any T, eight tokens a step (a token's output depends on
+// nothing but the token, so the steps are independent).
+static int experts_by_eight(const void* latent, const int32_t* ids, const float* weights, const lx_weight& gu, const lx_weight& dn,
+                            float* out, void* workspace, int T, int L, int I, int top_k, void* stream) {
+  hipStream_t s = as_stream(stream);
+  for (int t0 = 0; t0 < T; t0 += 8) {
+    const int n = T - t0 < 8 ? T - t0 : 8;
+    const int st = experts_decode(static_cast<const uint16_t*>(latent) + static_cast<int64_t>(t0) * L, ids + static_cast<int64_t>(t0) * top_k,
+                                  weights + static_cast<int64_t>(t0) * top_k, gu, dn, out + static_cast<int64_t>(t0) * L, workspace, n, L, I,
+                                  top_k, s);
+    if (st) return st;
+  }
+  return kOk;
+}
+
+// engine/cpu/moe.cpp:480-494. The kernels are the bf16 decode kernels with the encoded rows decoded in registers to
+// the bf16 bits those load, so out equals lx_moe_experts_decode_bf16 on the original stacks to the bit.
+int lx_moe_experts_bf16x(const void* latent, const int32_t* ids, const float* weights, const void* gate_up, const void* down,
+                         float* out, void* workspace, int T, int L, int I, int top_k, void* stream) {
+  if (T <= 0) return kOk;
+  if (!latent || !ids || !weights || !out || L <= 0 || I <= 0 || top_k < 1) return fail(kInvalid);
+  if (top_k > 8 || !gate_up || !down || !workspace || L >= bf16x::kMaxK || I >= bf16x::kMaxK) return fail(kInvalid);
+  if ((reinterpret_cast<uintptr_t>(gate_up) | reinterpret_cast<uintptr_t>(down)) & 7) return fail(kInvalid);
+  const lx_weight gu{LX_W_BF16X, gate_up, nullptr, 1.0f, nullptr}, dn{LX_W_BF16X, down, nullptr, 1.0f, nullptr};
+  return experts_by_eight(latent, ids, weights, gu, dn, out, workspace, T, L, I, top_k, stream);
+}
+
 int lx_moe_experts_decode_bf16(const void* latent, const int32_t* ids, const float* weights, const void* gate_up,
                                const void* down, float* out, void* workspace, int T, int L, int I, int top_k, void* stream) {
   if (T <= 0) return kOk;
   if (top_k > 8 || !workspace) return fail(kInvalid);
+  if (!latent || !ids || !weights || !out || !gate_up || !down || L <= 0 || I <= 0 || top_k < 1) return fail(kInvalid);
   const lx_weight gu{LX_W_BF16, gate_up, nullptr, 1.0f, nullptr}, dn{LX_W_BF16, down, nullptr, 1.0f, nullptr};
-  return lx_moe_experts_decode(latent, ids, weights, &gu, &dn, out, workspace, T, L, I, top_k, stream);
+  return experts_by_eight(latent, ids, weights, gu, dn, out, workspace, T, L, I, top_k, stream);
 }
 
 }  // extern "C"

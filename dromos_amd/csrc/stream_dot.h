@@ -23,6 +23,7 @@
 // output's bits depend only on its own x row (and its type), its weight row and the K split.
 #pragma once
 
+#include "bf16x.h"
 #include "common.h"
 
 namespace dro {
@@ -326,10 +327,47 @@ struct Chunk {
   uint32_t scales;  // NVFP4: two e4m3 bytes (block of dwords 0-1, block of dwords 2-3)
 };
 
+// Where the streams of an [N, K] matrix's rows start: row n's chunks at data + n * rb, its second stream (NVFP4 block
+// scales; BF16X span tops) at scale + n * scale_row. For BF16X `data` skips the first record's header, and both streams
+// advance by a whole record.
+template <int F>
+struct RowBase {
+  const uint8_t* data;
+  const uint8_t* scale;
+  int64_t rb, scale_row;
+  int chunks;
+  __host__ __device__ RowBase(const uint8_t* d, const uint8_t* s, int64_t K) {
+    rb = row_bytes<F>(K);
+    chunks = chunks_of<F>(K);
+    if constexpr (F == LX_W_BF16X) {
+      const bf16x::Geometry g(static_cast<int>(K));
+      data = d + g.header;
+      scale = d + g.tops_at();
+      scale_row = rb;
+    } else {
+      data = d;
+      scale = s;
+      scale_row = F == LX_W_NVFP4 ? K / 16 : 0;
+    }
+  }
+};
+
 // The row pointers are the same for every lane of a wavefront; the lane's part is an unsigned 32-bit byte offset, so
 // the load can take the row from scalar registers and the offset from one vector register.
 template <int F>
 __device__ __forceinline__ void load_chunk(Chunk<F>& c, const uint8_t* row, const uint8_t* row_scales, int chunk) {
+  if constexpr (F == LX_W_BF16X) {
+    // `row` points at the record's first block, `row_scales` at its base exponents. The chunk's eight values: 8 bytes
+    // of sign|mantissa (w.x, w.y), their 4 bytes of codes (w.z), the block's base (w.w); finish_chunk makes them bf16.
+    const uint32_t span = static_cast<uint32_t>(chunk) >> 4, within = static_cast<uint32_t>(chunk) & 15u;
+    const uint8_t* p = row + span * static_cast<uint32_t>(bf16x::kSpanBytes);
+    const u32x2 sm = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p + within * 8u));
+    c.w.x = sm.x;
+    c.w.y = sm.y;
+    c.w.z = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p + bf16x::kNibbles + within * 4u));
+    c.w.w = __builtin_nontemporal_load(row_scales + span);
+    return;
+  }
   const uint32_t off = static_cast<uint32_t>(chunk) * 16u;
   c.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row + off));
   if constexpr (F == LX_W_NVFP4)
@@ -403,6 +441,11 @@ __device__ __forceinline__ void dword_pairs(uint32_t d, bf16x2* out);
 
 template <>
 __device__ __forceinline__ void dword_pairs<LX_W_BF16>(uint32_t d, bf16x2* out) {
+  out[0] = as_bf16x2(d);
+}
+
+template <>
+__device__ __forceinline__ void dword_pairs<LX_W_BF16X>(uint32_t d, bf16x2* out) {
   out[0] = as_bf16x2(d);
 }
 
@@ -494,6 +537,15 @@ template <int F, int MT, int R, int U, bool XB = false, bool ONE = false>
 struct RowStreamer {
   Chunk<F> buf_a[U][R], buf_b[ONE ? 1 : U][ONE ? 1 : R];
   int chunks, s_begin, s_end, per_row, batches, lane;
+  // BF16X: the row pointers of rows_fn point at a record's first block (its header lies hdr_bytes before), the scale
+  // pointers at its base exponents; a row with exceptions (its first word says so) takes them from the header.
+  int hdr_bytes = 0, slots = 0;
+
+  __device__ __forceinline__ void set_bf16x(int K) {
+    const bf16x::Geometry g(K);
+    hdr_bytes = g.header;
+    slots = g.slots;
+  }
 
   __device__ __forceinline__ RowStreamer(int chunks_, int s_begin_, int s_end_, int per_row_)
       : chunks(chunks_), s_begin(s_begin_), s_end(s_end_), per_row(per_row_) {
@@ -520,8 +572,24 @@ struct RowStreamer {
     }
   }
 
-  __device__ __forceinline__ void consume(const Chunk<F> (&buf)[U][R], const float* const (&xs)[R], int batch,
-                                          float (&acc)[MT][R]) {
+  // The chunk as the products take it: BF16X is decoded to bf16 bits here (s: the chunk's step).
+  __device__ __forceinline__ Chunk<F> ready(const Chunk<F>& c, const uint8_t* row, int s) const {
+    if constexpr (F == LX_W_BF16X) {
+      const uint8_t* const rec = row - hdr_bytes;
+      // One word, the same for every lane, and vacant in nearly every row.
+      const bool has = bf16x::has_exceptions(rec);
+      const uint32_t k0 = static_cast<uint32_t>(min(s * kWave + lane, chunks - 1)) * 8u;
+      Chunk<F> o;
+      o.w = bf16x::octet_bits(c.w.x, c.w.y, c.w.z, c.w.w, has ? rec : nullptr, slots, k0);
+      o.scales = 0;
+      return o;
+    } else {
+      return c;
+    }
+  }
+
+  __device__ __forceinline__ void consume(const Chunk<F> (&buf)[U][R], const uint8_t* const (&rows)[R], const float* const (&xs)[R],
+                                          int batch, float (&acc)[MT][R]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int s = s_begin + batch * U + u;
@@ -532,8 +600,9 @@ struct RowStreamer {
           float a[MT];
 #pragma unroll
           for (int m = 0; m < MT; ++m) a[m] = acc[m][r];
-          if constexpr (XB) chunk_dot2<F, MT>(buf[u][r], reinterpret_cast<const uint32_t*>(xs[r]) + slot, per_row, a);
-          else chunk_fma<F, MT>(buf[u][r], xs[r] + slot, per_row, a);
+          const Chunk<F> c = ready(buf[u][r], rows[r], s);
+          if constexpr (XB) chunk_dot2<F, MT>(c, reinterpret_cast<const uint32_t*>(xs[r]) + slot, per_row, a);
+          else chunk_fma<F, MT>(c, xs[r] + slot, per_row, a);
 #pragma unroll
           for (int m = 0; m < MT; ++m) acc[m][r] = a[m];
         }
@@ -542,8 +611,8 @@ struct RowStreamer {
   }
 
   // The steps [lo, hi) of the single batch in `buf`, against an image whose first step is s_off.
-  __device__ __forceinline__ void consume_steps(const Chunk<F> (&buf)[U][R], const float* const (&xs)[R], int lo, int hi, int s_off,
-                                                float (&acc)[MT][R]) {
+  __device__ __forceinline__ void consume_steps(const Chunk<F> (&buf)[U][R], const uint8_t* const (&rows)[R], const float* const (&xs)[R],
+                                                int lo, int hi, int s_off, float (&acc)[MT][R]) {
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int s = s_begin + u;
@@ -554,8 +623,9 @@ struct RowStreamer {
           float a[MT];
 #pragma unroll
           for (int m = 0; m < MT; ++m) a[m] = acc[m][r];
-          if constexpr (XB) chunk_dot2<F, MT>(buf[u][r], reinterpret_cast<const uint32_t*>(xs[r]) + slot, per_row, a);
-          else chunk_fma<F, MT>(buf[u][r], xs[r] + slot, per_row, a);
+          const Chunk<F> c = ready(buf[u][r], rows[r], s);
+          if constexpr (XB) chunk_dot2<F, MT>(c, reinterpret_cast<const uint32_t*>(xs[r]) + slot, per_row, a);
+          else chunk_fma<F, MT>(c, xs[r] + slot, per_row, a);
 #pragma unroll
           for (int m = 0; m < MT; ++m) acc[m][r] = a[m];
         }
@@ -578,9 +648,9 @@ struct RowStreamer {
     const uint8_t* scales[R];
     const float* xs[R];
     rows_fn(group, rows, scales, xs);
-    consume_steps(buf_a, xs, 0, split, 0, acc);
+    consume_steps(buf_a, rows, xs, 0, split, 0, acc);
     restage();
-    consume_steps(buf_a, xs, split, s_end, split, acc);
+    consume_steps(buf_a, rows, xs, split, s_end, split, acc);
     done_fn(group, acc);
   }
 
@@ -608,7 +678,7 @@ struct RowStreamer {
       const uint8_t* scales[R];
       const float* xs[R];
       rows_fn(first_group, rows, scales, xs);
-      consume(buf_a, xs, 0, acc);
+      consume(buf_a, rows, xs, 0, acc);
       done_fn(first_group, acc);
     } else {
     int group = first_group, batch = 0, left = n_groups;
@@ -623,7 +693,7 @@ struct RowStreamer {
       const uint8_t* scales[R];
       const float* xs[R];
       rows_fn(group, rows, scales, xs);
-      consume(cur, xs, batch, acc);
+      consume(cur, rows, xs, batch, acc);
       if (last_batch) {
         done_fn(group, acc);
 #pragma unroll

@@ -28,7 +28,7 @@ extern "C" {
 
 /* engine/cuda/kernels.h:27 */
 typedef enum { LX_F32 = 0, LX_BF16 = 1 } lx_dtype;
-/* engine/cuda/kernels.h:243 (LX_W_BF16X is not on this path: calls with it answer 801) */
+/* engine/cuda/kernels.h:243 (LX_W_BF16X: the lossless form of bf16 below; lx_gemm_w and the grouped experts answer 801 for it) */
 typedef enum { LX_W_BF16 = 0, LX_W_INT8 = 1, LX_W_FP8 = 2, LX_W_NVFP4 = 3, LX_W_BF16X = 4 } lx_wtype;
 /* engine/cuda/kernels.h:431 */
 typedef enum { LX_MATH_BF16 = 0, LX_MATH_INT8 = 1, LX_MATH_FP8 = 2, LX_MATH_FP4 = 3 } lx_math;
@@ -47,6 +47,7 @@ typedef enum { LX_COPY_H2D = 0, LX_COPY_D2H = 1, LX_COPY_D2D = 2, LX_COPY_DEFAUL
  *   LX_W_FP8    data e4m3fn [N, K], scale f32 [N]          w = fp8 * scale[n]
  *   LX_W_NVFP4  data u8 [N, K/2] (low nibble = even k), scale e4m3 [N, K/16], global f32
  *                                                          w = e2m1 * scale[n, k/16] * global
+ *   LX_W_BF16X  data the encoding lx_bf16x_encode writes of bf16 [N, K] (8-byte aligned); no scale
  * A stack of experts is [E, N, K] laid out expert after expert (scales likewise); an NVFP4 stack may
  * carry one global per expert in expert_global (f32 [E] on the device, null = `global` for all).
  */
@@ -143,6 +144,33 @@ LX_API int lx_moe_experts_decode_bf16(const void* latent, const int32_t* ids, co
                                       const void* gate_up, const void* down, float* out, void* workspace, int T,
                                       int L, int I, int top_k, void* stream);
 LX_API int64_t lx_moe_bf16x_workspace_bytes(int T, int I, int top_k);
+
+/* ---- lossless bf16, LX_W_BF16X (replaces engine/cuda/kernels.h:567-611; CPU behaviour: engine/cpu/bf16x.cpp,
+ * engine/cpu/gemm.cpp:364-371, engine/cpu/moe.cpp:480-494) --------------------------------------------
+ * bf16 weights in about 12.2 bits a value, every bit kept: a value is one sign|mantissa byte and a 4-bit exponent
+ * code below the largest exponent of its span of 128 values; the rare value out of that range is listed in the
+ * row's header. The encoder writes the reference's bytes exactly, so encoded checkpoints are interchangeable.
+ *   lx_bf16x_row_bytes   bytes of one encoded row of K values (-1 unless 0 < K < 2^23)
+ *   lx_bf16x_bytes       bytes the encoding of w (bf16 [rows, K] on the device) needs: rows * row bytes plus the spill
+ *                        records of rows with more exceptions than header slots; -1 on bad arguments. Synchronizes.
+ *   lx_bf16x_encode      w -> out (8-byte aligned, out_bytes >= lx_bf16x_bytes); deterministic; synchronizes once,
+ *                        scratch from hipMallocAsync: load time, not graph capture
+ *   lx_bf16x_decode      the encoding back to bf16 [rows, K]
+ *   lx_gemv_bf16x        lx_gemv's contract on encoded rows; y is lx_gemv_decode_bf16's on the original weights to
+ *                        the bit (same lanes, steps, split and summation order), so a row's bits do not depend on M
+ *   lx_moe_experts_bf16x lx_moe_experts_decode_bf16's contract (any T, top_k <= 8, workspace of
+ *                        lx_moe_bf16x_workspace_bytes) on encoded stacks [E, 2I, L] and [E, L, I]; out equals
+ *                        lx_moe_experts_decode_bf16's on the original stacks to the bit. Nothing is allocated. */
+LX_API int64_t lx_bf16x_row_bytes(int K);
+LX_API int64_t lx_bf16x_bytes(const void* w, int64_t rows, int K, void* stream);
+LX_API int lx_bf16x_encode(const void* w, int64_t rows, int K, void* out, int64_t out_bytes, void* stream);
+LX_API int lx_bf16x_decode(const void* data, int64_t rows, int K, void* w, void* stream);
+LX_API int lx_gemv_bf16x(const void* x, lx_dtype x_dtype, int ld_x, const void* w, const void* bias,
+                         lx_dtype bias_dtype, void* y, lx_dtype y_dtype, int ld_y, int M, int N, int K, float alpha,
+                         float beta, void* stream);
+LX_API int lx_moe_experts_bf16x(const void* latent, const int32_t* ids, const float* weights, const void* gate_up,
+                                const void* down, float* out, void* workspace, int T, int L, int I, int top_k,
+                                void* stream);
 LX_API int lx_moe_experts_grouped(const void* latent, const int32_t* ids, const float* weights,
                                   const lx_weight* gate_up, const lx_weight* down, lx_math math, float* out,
                                   void* workspace, int T, int L, int I, int E, int top_k, void* stream);

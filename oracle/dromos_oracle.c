@@ -20,6 +20,8 @@
  *   lx_gemm_w INT8 / FP8 maths       pinned: exact integer / float64 products of the quantised values, bit for bit
  *   lx_moe_route                     pinned: stable sort of -(logit + bias) + float64 softmax, tie cases
  *   lx_moe_experts*                  pinned: float64 experts with the bf16-rounded intermediate
+ *   lx_bf16x_* / *_bf16x             pinned: decode(encode(w)) == w over every exponent pattern incl. spilled rows, sizes
+ *                                    by closed form, hand-built records; the products equal the bf16 products' bits
  */
 #include <math.h>
 #include <stdint.h>
@@ -29,7 +31,7 @@
 #define ORC_API __attribute__((visibility("default")))
 
 enum { LX_F32 = 0, LX_BF16 = 1 };
-enum { LX_W_BF16 = 0, LX_W_INT8 = 1, LX_W_FP8 = 2, LX_W_NVFP4 = 3 };
+enum { LX_W_BF16 = 0, LX_W_INT8 = 1, LX_W_FP8 = 2, LX_W_NVFP4 = 3, LX_W_BF16X = 4 };
 enum { LX_MATH_BF16 = 0, LX_MATH_INT8 = 1, LX_MATH_FP8 = 2, LX_MATH_FP4 = 3 };
 enum { ORC_OK = 0, ORC_INVALID = 1, ORC_NOMEM = 2, ORC_UNSUPPORTED = 801 };
 
@@ -290,12 +292,165 @@ ORC_API int lx_quantize_act(const void* x, int x_dtype, int ld_x, int math, void
   return ORC_OK;
 }
 
+/* ---- LX_W_BF16X: bf16 in 12 bits a value (layout: engine/cuda/bf16x.cuh:13-27; codec: engine/cpu/bf16x.cpp) ----
+ * A row record is S exception words, one top exponent per span of 128 values, zero bytes up to the header size,
+ * then 192 bytes a span: 128 sign|mantissa bytes and 16 words of 4-bit codes (top - exponent). */
+#define BX_SPAN 128
+#define BX_SPAN_BYTES 192
+#define BX_VACANT 0xffffffffu
+#define BX_MAX_K (1 << 23)
+
+static int bx_spans(int K) { return (K + BX_SPAN - 1) / BX_SPAN; }
+static int bx_header(int K) { return (4 * (2 + K / 2048) + bx_spans(K) + 7) / 8 * 8; } /* bf16x.cuh:46 */
+static int bx_slots(int K) { return (bx_header(K) - bx_spans(K)) / 4; }                 /* bf16x.cuh:47 */
+static int64_t bx_row_bytes(int K) { return bx_header(K) + (int64_t)BX_SPAN_BYTES * bx_spans(K); }
+static int64_t bx_spill_bytes(int64_t n) { return (4 * (n + 2) + 7) / 8 * 8; } /* bf16x.cpp:48 */
+static int bx_k_ok(int K) { return K > 0 && K < BX_MAX_K; }
+
+static uint32_t bx_get(const uint8_t* p) {
+  uint32_t v;
+  memcpy(&v, p, 4);
+  return v;
+}
+static void bx_put(uint8_t* p, uint32_t v) { memcpy(p, &v, 4); }
+static int bx_exponent(uint16_t v) { return (v >> 7) & 0xff; }
+
+/* The largest exponent among values [k0, k0 + 128) of a row of K (bf16x.cpp:25-32). */
+static int bx_top(const uint16_t* row, int K, int k0) {
+  int top = 0;
+  for (int k = k0; k < K && k < k0 + BX_SPAN; ++k)
+    if (bx_exponent(row[k]) > top) top = bx_exponent(row[k]);
+  return top;
+}
+
+/* Values whose exponent is more than 15 below their span's top (bf16x.cpp:35-46). */
+static int64_t bx_exceptions(const uint16_t* row, int K) {
+  int64_t n = 0;
+  for (int k0 = 0; k0 < K; k0 += BX_SPAN) {
+    int top = bx_top(row, K, k0);
+    for (int k = k0; k < K && k < k0 + BX_SPAN; ++k) n += top - bx_exponent(row[k]) > 15;
+  }
+  return n;
+}
+
+/* Where byte and nibble of value i of a span live: the nibble of value i is in code byte 4 * (i / 8) + i % 4, the
+ * low half for i % 8 < 4 (bf16x.cuh:22-25). */
+static uint8_t* bx_code_byte(uint8_t* span, int i) { return span + 128 + 4 * (i / 8) + (i % 4); }
+
+/* One row record at rec; its spill record (when n exceeds the slots) at rec + spill_off (bf16x.cpp:58-104). */
+static void bx_encode_row(const uint16_t* row, int K, uint8_t* rec, int64_t n, int64_t spill_off) {
+  const int S = bx_slots(K), H = bx_header(K), B = bx_spans(K);
+  memset(rec, 0, (size_t)bx_row_bytes(K));
+  for (int s = 0; s < S; ++s) bx_put(rec + 4 * s, BX_VACANT);
+  uint8_t* list = rec;
+  if (n > S) {
+    uint8_t* sp = rec + spill_off;
+    memset(sp, 0, (size_t)bx_spill_bytes(n));
+    bx_put(rec, 0x80000000u | (uint32_t)(spill_off / 8));
+    bx_put(sp, (uint32_t)n);
+    bx_put(sp + 4 * (n + 1), BX_VACANT);
+    list = sp + 4;
+  }
+  int64_t listed = 0;
+  for (int b = 0; b < B; ++b) {
+    uint8_t* span = rec + H + (int64_t)b * BX_SPAN_BYTES;
+    const int top = bx_top(row, K, b * BX_SPAN);
+    rec[4 * S + b] = (uint8_t)top;
+    for (int i = 0; i < BX_SPAN && b * BX_SPAN + i < K; ++i) {
+      const int k = b * BX_SPAN + i;
+      const uint16_t v = row[k];
+      span[i] = (uint8_t)(((v >> 8) & 0x80) | (v & 0x7f));
+      int code = top - bx_exponent(v);
+      if (code > 15) {
+        bx_put(list + 4 * listed++, ((uint32_t)k << 8) | (uint32_t)bx_exponent(v));
+        code = 0;
+      }
+      *bx_code_byte(span, i) |= (uint8_t)((i % 8) < 4 ? code : code << 4);
+    }
+  }
+}
+
+/* bf16 bits of value k of the row record at rec: the coded exponent unless an exception word names k (bf16x.cpp:162-193). */
+static uint16_t bx_value(const uint8_t* rec, int K, int k) {
+  const int S = bx_slots(K), b = k / BX_SPAN, i = k % BX_SPAN;
+  const uint8_t* span = rec + bx_header(K) + (int64_t)b * BX_SPAN_BYTES;
+  const uint8_t pair = *bx_code_byte((uint8_t*)span, i);
+  uint32_t e = (uint32_t)(rec[4 * S + b] - ((i % 8) < 4 ? pair & 15 : pair >> 4)) & 0xffu;
+  const uint8_t* list = rec;
+  int64_t n = S;
+  const uint32_t first = bx_get(rec);
+  if (first != BX_VACANT && (first & 0x80000000u)) {
+    const uint8_t* sp = rec + (int64_t)(first & 0x7fffffffu) * 8;
+    n = bx_get(sp);
+    list = sp + 4;
+  }
+  for (int64_t q = 0; q < n; ++q) {
+    const uint32_t word = bx_get(list + 4 * q);
+    if (word == BX_VACANT) break;
+    if ((word >> 8) == (uint32_t)k) e = word & 0xffu;
+  }
+  return (uint16_t)(((span[i] & 0x80u) << 8) | (e << 7) | (span[i] & 0x7fu));
+}
+
+/* engine/cpu/bf16x.cpp:129 */
+ORC_API int64_t lx_bf16x_row_bytes(int K) { return bx_k_ok(K) ? bx_row_bytes(K) : -1; }
+
+/* The spill area: records in row order (bf16x.cpp:107-123). at (optional): each row's offset in it, -1 for none. */
+static int64_t bx_layout(const uint16_t* w, int64_t rows, int K, int64_t* counts, int64_t* at) {
+  int64_t area = 0;
+  for (int64_t r = 0; r < rows; ++r) {
+    const int64_t n = bx_exceptions(w + r * K, K);
+    if (counts) counts[r] = n;
+    if (at) at[r] = -1;
+    if (n <= bx_slots(K)) continue;
+    if (at) at[r] = area;
+    area += bx_spill_bytes(n);
+  }
+  return area;
+}
+
+/* engine/cpu/bf16x.cpp:131-138 */
+ORC_API int64_t lx_bf16x_bytes(const void* w, int64_t rows, int K, void* stream) {
+  (void)stream;
+  if (rows <= 0 || !bx_k_ok(K) || !w) return -(int64_t)fail(ORC_INVALID);
+  return rows * bx_row_bytes(K) + bx_layout((const uint16_t*)w, rows, K, NULL, NULL);
+}
+
+/* engine/cpu/bf16x.cpp:140-160 */
+ORC_API int lx_bf16x_encode(const void* w, int64_t rows, int K, void* out, int64_t out_bytes, void* stream) {
+  (void)stream;
+  if (rows <= 0) return ORC_OK;
+  const int64_t rb = bx_k_ok(K) ? bx_row_bytes(K) : 0;
+  if (!rb || !w || !out || ((uintptr_t)out & 7) != 0 || out_bytes < rows * rb) return fail(ORC_INVALID);
+  int64_t* counts = (int64_t*)malloc(sizeof(int64_t) * (size_t)rows * 2);
+  if (!counts) return fail(ORC_NOMEM);
+  int64_t* at = counts + rows;
+  const int64_t area = bx_layout((const uint16_t*)w, rows, K, counts, at);
+  int st = ORC_OK;
+  if (rows * rb + area > out_bytes) st = fail(ORC_INVALID);
+  for (int64_t r = 0; r < rows && !st; ++r)
+    bx_encode_row((const uint16_t*)w + r * K, K, (uint8_t*)out + r * rb, counts[r], at[r] < 0 ? 0 : rows * rb + at[r] - r * rb);
+  free(counts);
+  return st;
+}
+
+/* engine/cpu/bf16x.cpp:162-197 */
+ORC_API int lx_bf16x_decode(const void* data, int64_t rows, int K, void* w, void* stream) {
+  (void)stream;
+  if (rows <= 0) return ORC_OK;
+  if (!bx_k_ok(K) || !data || !w) return fail(ORC_INVALID);
+  for (int64_t r = 0; r < rows; ++r)
+    for (int k = 0; k < K; ++k) ((uint16_t*)w)[r * K + k] = bx_value((const uint8_t*)data + r * bx_row_bytes(K), K, k);
+  return ORC_OK;
+}
+
 /* Element (n, k) of an [N, K] weight, exact, without its row factor (engine/cpu/quant.cpp:143-154). */
 static float weight_element(int type, const void* data, const void* scale, int64_t n, int64_t k, int64_t K) {
   switch (type) {
     case LX_W_BF16: return bf16_value(((const uint16_t*)data)[n * K + k]);
     case LX_W_INT8: return (float)((const int8_t*)data)[n * K + k];
     case LX_W_FP8: return orc_e4m3_to_f32(((const uint8_t*)data)[n * K + k]);
+    case LX_W_BF16X: return bf16_value(bx_value((const uint8_t*)data + n * bx_row_bytes((int)K), (int)K, (int)k));
     default: {
       uint8_t byte = ((const uint8_t*)data)[n * (K / 2) + k / 2];
       uint32_t code = (k & 1) ? (uint32_t)(byte >> 4) : (uint32_t)(byte & 15);
@@ -369,6 +524,7 @@ static int weight_ok(const lx_weight* w, int64_t K) {
     case LX_W_INT8:
     case LX_W_FP8: return w->scale != NULL;
     case LX_W_NVFP4: return w->scale != NULL && K % 16 == 0;
+    case LX_W_BF16X: return K < BX_MAX_K; /* only through the *_bf16x entries (engine/cpu/gemm.cpp:165) */
     default: return 0;
   }
 }
@@ -427,11 +583,22 @@ ORC_API int lx_gemv(const void* x, int x_dtype, int ld_x, const void* w, int w_t
   return gemv_any(x, x_dtype, ld_x, &wt, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
 }
 
+/* engine/cpu/gemm.cpp:364-371: the f32 product on the rows the encoding decodes to, so y is the bf16 weights' to the bit. */
+ORC_API int lx_gemv_bf16x(const void* x, int x_dtype, int ld_x, const void* w, const void* bias, int bias_dtype, void* y,
+                          int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
+  (void)stream;
+  if (M != 0 && N != 0 && ((uintptr_t)w & 7) != 0) return fail(ORC_INVALID);
+  lx_weight wt = {LX_W_BF16X, w, NULL, 1.0f, NULL};
+  return gemv_any(x, x_dtype, ld_x, &wt, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
+}
+
 /* engine/cpu/gemm.cpp:350-359 */
 ORC_API int lx_gemv_w(const void* x, int x_dtype, int ld_x, const lx_weight* w, const void* bias, int bias_dtype, void* y,
                       int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream) {
   (void)stream;
   if (!w) return fail(ORC_INVALID);
+  if (w->type == LX_W_BF16X)
+    return lx_gemv_bf16x(x, x_dtype, ld_x, w->data, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, stream);
   return gemv_any(x, x_dtype, ld_x, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta);
 }
 
@@ -664,6 +831,7 @@ static lx_weight expert_slice(const lx_weight* s, int64_t e, int64_t N, int64_t 
   int64_t rows = e * N;
   switch (s->type) {
     case LX_W_BF16: o.data = (const uint16_t*)s->data + rows * K; break;
+    case LX_W_BF16X: o.data = (const uint8_t*)s->data + rows * bx_row_bytes((int)K); break; /* moe.cpp:44-45 */
     case LX_W_INT8:
     case LX_W_FP8:
       o.data = (const uint8_t*)s->data + rows * K;
@@ -876,6 +1044,18 @@ ORC_API int lx_moe_experts_decode_bf16(const void* latent, const int32_t* ids, c
   return lx_moe_experts(latent, ids, weights, gate_up, down, out, T, L, I, top_k, stream);
 }
 
+/* engine/cpu/moe.cpp:480-494: lx_moe_experts with the rows read from the encoding. */
+ORC_API int lx_moe_experts_bf16x(const void* latent, const int32_t* ids, const float* weights, const void* gate_up,
+                                 const void* down, float* out, void* workspace, int T, int L, int I, int top_k, void* stream) {
+  (void)stream;
+  if (T <= 0) return ORC_OK;
+  int st = experts_args(latent, ids, weights, out, L, I, top_k);
+  if (st) return st;
+  if (top_k > 8 || !gate_up || !down || !workspace || L >= BX_MAX_K || I >= BX_MAX_K) return fail(ORC_INVALID);
+  lx_weight gu = {LX_W_BF16X, gate_up, NULL, 1.0f, NULL}, dn = {LX_W_BF16X, down, NULL, 1.0f, NULL};
+  return experts((const uint16_t*)latent, ids, weights, &gu, &dn, out, T, L, I, top_k, 0, ORC_WEIGHT_ONLY);
+}
+
 /* engine/cpu/moe.cpp:519-538 */
 ORC_API int lx_moe_experts_decode(const void* latent, const int32_t* ids, const float* weights, const lx_weight* gate_up,
                                   const lx_weight* down, float* out, void* workspace, int T, int L, int I, int top_k,
@@ -887,6 +1067,10 @@ ORC_API int lx_moe_experts_decode(const void* latent, const int32_t* ids, const 
   int st = experts_args(latent, ids, weights, out, L, I, top_k);
   if (st) return st;
   if (!gate_up || !down) return fail(ORC_INVALID);
+  if (gate_up->type == LX_W_BF16X || down->type == LX_W_BF16X) {
+    if (gate_up->type != LX_W_BF16X || down->type != LX_W_BF16X) return fail(ORC_UNSUPPORTED);
+    return lx_moe_experts_bf16x(latent, ids, weights, gate_up->data, down->data, out, workspace, T, L, I, top_k, stream);
+  }
   if (!stack_ok(gate_up, L) || !stack_ok(down, I)) return fail(ORC_INVALID);
   return experts((const uint16_t*)latent, ids, weights, gate_up, down, out, T, L, I, top_k, 0, ORC_WEIGHT_ONLY);
 }

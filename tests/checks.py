@@ -297,3 +297,56 @@ def quantize_reference_stack(w, fmt):
     parts = [quantize_reference(wb[e], fmt) for e in range(wb.shape[0])]
     eg = torch.tensor([p.glob for p in parts], dtype=torch.float32)
     return Weight(fmt, torch.stack([p.data for p in parts]), torch.stack([p.scale for p in parts]), parts[0].glob, eg)
+
+
+# ---- lossless bf16 (LX_W_BF16X) ----------------------------------------------------------------------------------
+
+
+def bf16x_weights(rows, K, seed, kind="trained"):
+    """bf16 [rows, K] whose exponents exercise the format.
+    trained: N(0, 0.02) with a sprinkle of values many binades down (a few exceptions a row, within the slots);
+    wild:    every bit pattern is possible (infinities, NaNs, denormals, both zeros), exponents spread over all 256;
+    spill:   rows where most values lie far below a few large ones (more exceptions than slots: spill records),
+             mixed with rows that have none."""
+    g = torch.Generator().manual_seed(seed)
+    if kind == "wild":
+        return torch.randint(-32768, 32768, (rows, K), generator=g, dtype=torch.int32).to(torch.int16).view(torch.bfloat16)
+    w = (torch.randn(rows, K, generator=g) * 0.02).to(torch.bfloat16)
+    if kind == "trained":
+        tiny = torch.rand(rows, K, generator=g) < 2.0 / K
+        w[tiny] = (w[tiny].float() * 2.0**-40).to(torch.bfloat16)
+        w[torch.rand(rows, K, generator=g) < 1.0 / K] = 0.0
+        return w
+    assert kind == "spill"
+    small = torch.rand(rows, K, generator=g) < 0.3
+    w[small] = (w[small].float() * 2.0**-30).to(torch.bfloat16)
+    w[1::3] = (torch.randn(K, generator=g) * 0.02).to(torch.bfloat16)  # rows without exceptions in between
+    return w
+
+
+def bf16x_geometry(K):
+    spans = (K + 127) // 128
+    header = (4 * (2 + K // 2048) + spans + 7) // 8 * 8
+    return spans, header, (header - spans) // 4, header + 192 * spans
+
+
+def bf16x_round_trip(lx, rows, K, seed, kind):
+    """encode -> the library's decode and the numpy reading of the layout both give back every bit; the size is the
+    closed form plus spill records; nothing is written past it."""
+    w = dev(lx, bf16x_weights(rows, K, seed, kind))
+    enc = ops.bf16x_encode(lx, w, slack=64)
+    _, _, slots, rb = bf16x_geometry(K)
+    assert ops.bf16x_row_bytes(lx, K) == rb
+    # Exceptions a row: values more than 15 binades under the largest exponent of their span of 128.
+    e = ((w.cpu().view(torch.int16).int() >> 7) & 0xFF)
+    pad = (-K) % 128
+    span_e = torch.nn.functional.pad(e, (0, pad), value=0).view(rows, -1, 128)
+    inside = torch.nn.functional.pad(torch.ones_like(e, dtype=torch.bool), (0, pad), value=False).view(rows, -1, 128)
+    counts = (((span_e.max(-1, keepdim=True).values - span_e) > 15) & inside).sum((-1, -2))
+    spill = sum((4 * (int(n) + 2) + 7) // 8 * 8 for n in counts if n > slots)
+    assert enc.numel() - 64 == rows * rb + spill
+    assert bool((enc[-64:] == 0xEE).all())
+    back = ops.bf16x_decode(lx, enc, rows, K)
+    assert torch.equal(back.view(torch.int16).cpu(), w.view(torch.int16).cpu())
+    assert torch.equal(ops.bf16x_decode_reference(enc[:-64], rows, K).view(torch.int16), w.view(torch.int16).cpu())
+    return w, enc[:-64], counts

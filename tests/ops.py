@@ -239,3 +239,103 @@ def gemm_bf16(lx, x, w, bias=None, y=None, alpha=1.0, beta=0.0, y_dtype=torch.fl
         y = torch.full((M, N), float("nan"), dtype=y_dtype, device=lx.device)
     lx("gemm_bf16", x, K, w, bias, y, DTYPE[y.dtype], N, M, N, K, float(alpha), float(beta))
     return y
+
+
+# ---- lossless bf16 (LX_W_BF16X) ----------------------------------------------------------------------------------
+
+
+def bf16x_row_bytes(lx, K):
+    fn = lx.lib.lx_bf16x_row_bytes
+    fn.restype = ctypes.c_int64
+    return int(fn(ctypes.c_int(K)))
+
+
+def bf16x_bytes(lx, w):
+    """lx_bf16x_bytes of bf16 rows w [rows, K] (a stack is flattened to rows)."""
+    K = w.shape[-1]
+    rows = w.numel() // K
+    fn = lx.lib.lx_bf16x_bytes
+    fn.restype = ctypes.c_int64
+    return int(fn(ctypes.c_void_p(w.data_ptr()), ctypes.c_int64(rows), ctypes.c_int(K), lx.stream))
+
+
+def bf16x_encode(lx, w, slack=0):
+    """The encoding of bf16 w [..., K] as a uint8 tensor of exactly lx_bf16x_bytes (+ slack bytes of 0xEE, to show
+    nothing is written past the end)."""
+    w = w.contiguous()
+    K = w.shape[-1]
+    rows = w.numel() // K
+    n = bf16x_bytes(lx, w)
+    assert n >= rows * bf16x_row_bytes(lx, K)
+    out = torch.full((n + slack,), 0xEE, dtype=torch.uint8, device=lx.device)
+    assert out.data_ptr() % 8 == 0
+    lx("bf16x_encode", w, ctypes.c_int64(rows), K, out, ctypes.c_int64(n))
+    return out
+
+
+def bf16x_decode(lx, data, rows, K):
+    w = torch.full((rows, K), -1, dtype=torch.int16, device=lx.device).view(torch.bfloat16)
+    lx("bf16x_decode", data, ctypes.c_int64(rows), K, w)
+    return w
+
+
+def gemv_bf16x(lx, x, data, N, bias=None, y=None, alpha=1.0, beta=0.0, y_dtype=torch.float32, entry="gemv_bf16x", status=False):
+    """lx_gemv_bf16x (or lx_gemv_decode_bf16 with `data` the plain bf16 weights)."""
+    M, K = x.shape
+    if y is None:
+        y = torch.full((M, N), float("nan"), dtype=y_dtype, device=lx.device)
+    args = (x, DTYPE[x.dtype], K, data, bias, DTYPE[bias.dtype] if bias is not None else F32, y, DTYPE[y.dtype], N, M, N, K,
+            float(alpha), float(beta))
+    if status:
+        return lx.status(entry, *args)
+    lx(entry, *args)
+    return y
+
+
+def experts_bf16x(lx, latent, ids, weights, gate_up, down, I, top_k, entry="moe_experts_bf16x", status=False):
+    """lx_moe_experts_bf16x on encoded stacks (or lx_moe_experts_decode_bf16 on plain bf16 stacks)."""
+    T, L = latent.shape
+    nbytes = int(lx.size("moe_bf16x_workspace_bytes", T, I, top_k))
+    ws = torch.full((max(nbytes, 1),), 0xFF, dtype=torch.uint8, device=lx.device)
+    out = torch.full((T, L), float("nan"), device=lx.device)
+    args = (latent, ids, weights, gate_up, down, out, ws, T, L, I, top_k)
+    if status:
+        return lx.status(entry, *args)
+    lx(entry, *args)
+    return out
+
+
+def bf16x_decode_reference(data, rows, K):
+    """The layout read back with numpy alone (no library): bf16 bits [rows, K] as uint16. Written from the format's
+    description: S exception words, a top exponent per span of 128, 192-byte spans of 128 sign|mantissa bytes and 64
+    bytes of 4-bit codes."""
+    import numpy as np
+
+    buf = data.cpu().numpy()
+    spans = (K + 127) // 128
+    header = (4 * (2 + K // 2048) + spans + 7) // 8 * 8
+    slots = (header - spans) // 4
+    rb = header + 192 * spans
+    out = np.zeros((rows, K), dtype=np.uint16)
+    for r in range(rows):
+        rec = buf[r * rb:(r + 1) * rb]
+        tops = rec[4 * slots:4 * slots + spans].astype(np.int32)
+        body = rec[header:].reshape(spans, 192)
+        sm = body[:, :128].astype(np.uint16)
+        pairs = body[:, 128:].reshape(spans, 16, 4)
+        codes = np.concatenate([pairs & 15, pairs >> 4], axis=2).reshape(spans, 128).astype(np.int32)
+        e = ((tops[:, None] - codes) & 0xFF).astype(np.uint16)
+        bits = ((sm & 0x80) << 8) | (e << 7) | (sm & 0x7F)
+        row = bits.reshape(-1)[:K].copy()
+        words = rec[:4 * slots].view(np.uint32)
+        if words[0] != 0xFFFFFFFF and words[0] & 0x80000000:
+            at = r * rb + int(words[0] & 0x7FFFFFFF) * 8
+            n = int(buf[at:at + 4].view(np.uint32)[0])
+            words = buf[at + 4:at + 4 + 4 * n].view(np.uint32)
+        for word in words:
+            if word == 0xFFFFFFFF:
+                break
+            k = int(word >> 8)
+            row[k] = (row[k] & 0x807F) | ((int(word) & 0xFF) << 7)
+        out[r] = row
+    return torch.from_numpy(out.view(np.int16)).view(torch.bfloat16)

@@ -24,7 +24,8 @@ def test_header_declares_the_hot_path():
                  "lx_quantize_w8", "lx_quantize_weight", "lx_dequantize_weight", "lx_moe_route", "lx_moe_experts",
                  "lx_moe_experts_decode", "lx_moe_decode_workspace_bytes", "lx_moe_experts_decode_bf16",
                  "lx_moe_bf16x_workspace_bytes", "lx_moe_experts_grouped", "lx_moe_grouped_workspace_bytes",
-                 "lx_rt_backend", "lx_rt_device_count", "lx_arch", "lx_tune_variants", "lx_bandwidth_probe"):
+                 "lx_bf16x_row_bytes", "lx_bf16x_bytes", "lx_bf16x_encode", "lx_bf16x_decode", "lx_gemv_bf16x",
+                 "lx_moe_experts_bf16x", "lx_rt_backend", "lx_rt_device_count", "lx_arch", "lx_tune_variants", "lx_bandwidth_probe"):
         assert must in names, must
 
 

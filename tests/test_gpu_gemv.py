@@ -107,8 +107,8 @@ def test_argument_errors(hip):
     assert ops.gemv_w(hip, torch.zeros(1, 40, device="cuda"), w4, K=40, N=8, status=True) == 1
     from dromos_amd.formats import Weight
 
-    wx = Weight(4, w.data)  # LX_W_BF16X: not on this path
-    assert ops.gemv_w(hip, x[:1], wx, status=True) == 801
+    wx = Weight(7, w.data)  # no such format
+    assert ops.gemv_w(hip, x[:1], wx, status=True) == 1
 
 
 @pytest.mark.parametrize("fmt", FMT)
