@@ -74,38 +74,16 @@ struct Exceptions {
   }
 };
 
-// Four exponents, one a byte, from a span's top and a word with the values' nibbles in the low half of each byte.
-// A nibble never exceeds the top (the encoder took it from top - exponent), so bytes do not borrow.
-__device__ __forceinline__ uint32_t quad_exponents(uint32_t top, uint32_t nibbles) {
-  return top * 0x01010101u - (nibbles & 0x0f0f0f0fu);
-}
-
-// bf16 bits of four values: `sm` their sign|mantissa bytes, `e` their exponents. A bf16's upper byte is the sign over
+// bf16 bits of four values: `sm` their sign|mantissa bytes, `e` their exponents, one a byte (a span's top in every
+// byte minus the values' nibbles: a nibble never exceeds the top it was taken from, so bytes do not borrow). A bf16's upper byte is the sign over
 // exponent bits 7..1, its lower byte exponent bit 0 over the mantissa; v_perm_b32 zips the two byte rows (selectors
 // 0..3 name bytes of the second operand, 4..7 of the first). Values 0, 1 land in .x, 2, 3 in .y, lower k in the low half.
 __device__ __forceinline__ u32x2 quad_bits(uint32_t sm, uint32_t e) {
-  const uint32_t upper = (sm & 0x80808080u) | ((e >> 1) & 0x7f7f7f7fu);
-  const uint32_t lower = (sm & 0x7f7f7f7fu) | ((e & 0x01010101u) << 7);
+  // Each a bit-field insert: the mask's bits from sm, the others from the shifted exponents.
+  const uint32_t upper = (sm & 0x80808080u) | ((e >> 1) & ~0x80808080u);
+  const uint32_t lower = (sm & 0x7f7f7f7fu) | ((e << 7) & ~0x7f7f7f7fu);
   return u32x2{__builtin_amdgcn_perm(upper, lower, 0x05010400u), __builtin_amdgcn_perm(upper, lower, 0x07030602u)};
 }
-
-// Eight consecutive values (k0 a multiple of 8) as the four dwords a bf16 row holds for them. sm_lo / sm_hi: their
-// sign|mantissa bytes; nibbles: their nibble word; top: their span's top. `rec` non-null: the row record's first byte,
-// and the row's exceptions are applied.
-__device__ __forceinline__ u32x4 octet_bits(uint32_t sm_lo, uint32_t sm_hi, uint32_t nibbles, uint32_t top, const uint8_t* rec,
-                                            int slots, uint32_t k0) {
-  uint32_t e_lo = quad_exponents(top, nibbles), e_hi = quad_exponents(top, nibbles >> 4);
-  if (rec) {
-    const Exceptions ex(rec, slots);
-    e_lo = ex.fix(e_lo, k0);
-    e_hi = ex.fix(e_hi, k0 + 4);
-  }
-  const u32x2 a = quad_bits(sm_lo, e_lo), b = quad_bits(sm_hi, e_hi);
-  return u32x4{a.x, a.y, b.x, b.y};
-}
-
-// True when the row record at `rec` lists any exception.
-__device__ __forceinline__ bool has_exceptions(const uint8_t* rec) { return *reinterpret_cast<const uint32_t*>(rec) != kVacant; }
 
 // One value (any k < K) of the row record at `rec`: its bf16 bits.
 __device__ __forceinline__ uint16_t value_bits(const uint8_t* rec, int K, int k) {

@@ -156,10 +156,6 @@ __device__ __forceinline__ void decode_dword<LX_W_BF16>(uint32_t d, float* out) 
   out[1] = __uint_as_float(d & 0xffff0000u);
 }
 template <>
-__device__ __forceinline__ void decode_dword<LX_W_BF16X>(uint32_t d, float* out) {
-  decode_dword<LX_W_BF16>(d, out);
-}
-template <>
 __device__ __forceinline__ void decode_dword<LX_W_INT8>(uint32_t d, float* out) {
   out[0] = static_cast<float>(static_cast<int>(static_cast<int8_t>(d)));
   out[1] = static_cast<float>(static_cast<int>(static_cast<int8_t>(d >> 8)));

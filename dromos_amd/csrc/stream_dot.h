@@ -23,6 +23,8 @@
 // output's bits depend only on its own x row (and its type), its weight row and the K split.
 #pragma once
 
+#include <type_traits>
+
 #include "bf16x.h"
 #include "common.h"
 
@@ -326,6 +328,16 @@ struct Chunk {
   u32x4 w;
   uint32_t scales;  // NVFP4: two e4m3 bytes (block of dwords 0-1, block of dwords 2-3)
 };
+// BF16X: the eight values' sign|mantissa bytes and nibble word, and the step's four tops, which every lane loads from
+// the same address; in a row's first chunk of a batch lanes 60 .. 63 load the first four words of the row's header
+// instead, so the row's exceptions (nearly always at most a few) ride on a load that is waited for anyway.
+template <>
+struct Chunk<LX_W_BF16X> {
+  uint32_t sm_lo, sm_hi, nib, tops;
+};
+// The format whose products a chunk enters once it is ready: BF16X rows are decoded to bf16.
+template <int F>
+constexpr int kProductFormat = F == LX_W_BF16X ? LX_W_BF16 : F;
 
 // Where the streams of an [N, K] matrix's rows start: row n's chunks at data + n * rb, its second stream (NVFP4 block
 // scales; BF16X span tops) at scale + n * scale_row. For BF16X `data` skips the first record's header, and both streams
@@ -356,23 +368,150 @@ struct RowBase {
 // the load can take the row from scalar registers and the offset from one vector register.
 template <int F>
 __device__ __forceinline__ void load_chunk(Chunk<F>& c, const uint8_t* row, const uint8_t* row_scales, int chunk) {
-  if constexpr (F == LX_W_BF16X) {
-    // `row` points at the record's first block, `row_scales` at its base exponents. The chunk's eight values: 8 bytes
-    // of sign|mantissa (w.x, w.y), their 4 bytes of codes (w.z), the block's base (w.w); finish_chunk makes them bf16.
-    const uint32_t span = static_cast<uint32_t>(chunk) >> 4, within = static_cast<uint32_t>(chunk) & 15u;
-    const uint8_t* p = row + span * static_cast<uint32_t>(bf16x::kSpanBytes);
-    const u32x2 sm = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(p + within * 8u));
-    c.w.x = sm.x;
-    c.w.y = sm.y;
-    c.w.z = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p + bf16x::kNibbles + within * 4u));
-    c.w.w = __builtin_nontemporal_load(row_scales + span);
-    return;
-  }
   const uint32_t off = static_cast<uint32_t>(chunk) * 16u;
   c.w = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(row + off));
   if constexpr (F == LX_W_NVFP4)
     c.scales = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(row_scales + (off >> 3)));
 }
+
+// A word every lane reads from the same address. A vector load on purpose: weights stream through once, and scalar
+// loads of streamed data (every one a miss of the small scalar cache) have measured far slower than a broadcast
+// vector load of the line the lanes' own loads fetch anyway.
+__device__ __forceinline__ uint32_t uniform_word(const uint8_t* p) {
+  return __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(p));
+}
+
+// What a lane needs to stream LX_W_BF16X rows, computed once. Step s covers spans 4s .. 4s + 3 (768 bytes of the record
+// after its header): lane l takes chunk l % 16 of span 4s + l / 16, i.e. 8 sign|mantissa bytes and one nibble word, and
+// the span's top is byte l / 16 of the s-th word of tops, which is the same word for the whole wavefront. A lane whose
+// chunk lies past the row's end takes the row's last chunk instead (its x is zero): offsets are clamped to the last
+// chunk's, and in the row's last step so is the byte picked from the tops.
+struct Bf16xLane {
+  uint32_t sm_off, nib_off;      // this lane's byte offsets in step 0, from the first span
+  uint32_t last_sm, last_nib;    // those of the row's last chunk
+  uint32_t top_sel, top_sel_last;  // v_perm selectors that replicate the lane's top byte (any step / the last step)
+  int hdr_bytes, slots, chunks, last_step;
+  __device__ __forceinline__ void set(int K, int lane) {
+    const bf16x::Geometry g(K);
+    hdr_bytes = g.header;
+    slots = g.slots;
+    chunks = K / 8;
+    last_step = (chunks - 1) / kWave;
+    const uint32_t quarter = static_cast<uint32_t>(lane) >> 4, within = static_cast<uint32_t>(lane) & 15u;
+    sm_off = quarter * bf16x::kSpanBytes + within * 8u;
+    nib_off = quarter * bf16x::kSpanBytes + bf16x::kNibbles + within * 4u;
+    const uint32_t last = static_cast<uint32_t>(chunks - 1), last_span = last >> 4;
+    last_sm = __umul24(last_span, bf16x::kSpanBytes) + (last & 15u) * 8u;
+    last_nib = __umul24(last_span, bf16x::kSpanBytes) + bf16x::kNibbles + (last & 15u) * 4u;
+    top_sel = quarter * 0x01010101u;
+    top_sel_last = min(quarter, last_span & 3u) * 0x01010101u;
+  }
+};
+
+__device__ __forceinline__ void load_chunk_bf16x(Chunk<LX_W_BF16X>& c, const uint8_t* row, const uint8_t* tops, int s, bool with_head,
+                                                 const Bf16xLane& g) {
+  const uint32_t step_off = static_cast<uint32_t>(s) * (4u * bf16x::kSpanBytes);
+  const u32x2 sm = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(row + min(g.sm_off + step_off, g.last_sm)));
+  c.sm_lo = sm.x;
+  c.sm_hi = sm.y;
+  c.nib = __builtin_nontemporal_load(reinterpret_cast<const uint32_t*>(row + min(g.nib_off + step_off, g.last_nib)));
+  const uint32_t lane = threadIdx.x & (kWave - 1);
+  c.tops = uniform_word(with_head && lane >= kWave - 4 ? row - g.hdr_bytes + 4u * (lane - (kWave - 4)) : tops + 4 * s);
+}
+
+// The chunk as the bf16 kernel would have loaded it: four words of two bf16 each.
+__device__ __forceinline__ u32x4 decode_chunk_bf16x(const Chunk<LX_W_BF16X>& c, int s, const Bf16xLane& g) {
+  const uint32_t tops = __builtin_amdgcn_readfirstlane(c.tops);
+  const uint32_t top4 = __builtin_amdgcn_perm(tops, tops, s == g.last_step ? g.top_sel_last : g.top_sel);
+  const u32x2 a = bf16x::quad_bits(c.sm_lo, top4 - (c.nib & 0x0f0f0f0fu));
+  const u32x2 b = bf16x::quad_bits(c.sm_hi, top4 - ((c.nib >> 4) & 0x0f0f0f0fu));
+  return u32x4{a.x, a.y, b.x, b.y};
+}
+
+// One exception word applied to the lane's decoded chunk (index `chunk`) if it names one of its values.
+__device__ __forceinline__ u32x4 patch_chunk_bf16x(u32x4 w, uint32_t word, uint32_t chunk) {
+  const uint32_t k = word >> 8;
+  if ((k >> 3) == chunk) {
+    const uint32_t sh = (k & 1u) * 16u + 7u;
+    const uint32_t keep = ~(0xffu << sh), bits = (word & 0xffu) << sh;
+    const uint32_t d = (k >> 1) & 3u;
+    w.x = d == 0 ? (w.x & keep) | bits : w.x;
+    w.y = d == 1 ? (w.y & keep) | bits : w.y;
+    w.z = d == 2 ? (w.z & keep) | bits : w.z;
+    w.w = d == 3 ? (w.w & keep) | bits : w.w;
+  }
+  return w;
+}
+
+// A row's exceptions as the products of one batch use them, the same in every lane. Up to four words sit in scalar
+// registers (kVacant: none); they came with the batch's loads and cover nearly every row that has any. A row with more
+// (its fourth word is taken and the header has further slots, or it has a spill record) costs one more load: lane l
+// takes word l of the list into `listed`, up to 64 of them; a list longer than that (`beyond` > 0) is walked in
+// memory for the rest. `steps` says which of the batch's steps hold an exception (bit u: step s0 + u), so that the
+// chunks of the other steps spend nothing.
+struct Bf16xExceptions {
+  uint32_t word[4];
+  uint32_t steps;
+  bool wide;           // the words are in `listed`, not in word[]
+  uint32_t listed;     // per lane
+  const uint32_t* list;
+  uint32_t count;      // words in the list (an upper bound: a kVacant ends it early)
+  // `first`: the row's first chunk of the batch, whose lanes 60 .. 63 hold the header's first four words; rec: the
+  // row record; U: the batch's steps.
+  template <int U>
+  __device__ __forceinline__ Bf16xExceptions(const Chunk<LX_W_BF16X>& first, const uint8_t* rec, int slots, int s0, std::integral_constant<int, U>) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t v = __builtin_amdgcn_readlane(first.tops, kWave - 4 + i);
+      word[i] = i < slots ? v : bf16x::kVacant;  // a header of fewer than four words: the rest are tops
+    }
+    const bool spilled = word[0] != bf16x::kVacant && (word[0] & bf16x::kSpilled);
+    wide = spilled || (slots > 4 && word[3] != bf16x::kVacant);
+    steps = 0u;
+    listed = bf16x::kVacant;
+    list = nullptr;
+    count = 0;
+    if (!wide) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t d = (word[i] >> 17) - static_cast<uint32_t>(s0);  // a word's step: k / 512
+        if (word[i] != bf16x::kVacant && d < 32u) steps |= 1u << d;
+      }
+    } else {
+      const bf16x::Exceptions ex(rec, slots);
+      list = ex.words;
+      count = ex.limit;
+      const uint32_t lane = threadIdx.x & (kWave - 1);
+      if (lane < count) listed = list[lane];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (__ballot(listed != bf16x::kVacant && (listed >> 17) == static_cast<uint32_t>(s0 + u)) != 0) steps |= 1u << u;
+      if (count > static_cast<uint32_t>(kWave)) steps = ~0u;
+    }
+  }
+
+  // The exceptions that fall into the lane's decoded chunk (index `chunk`), applied.
+  __device__ __forceinline__ u32x4 apply(u32x4 w, uint32_t chunk) const {
+    if (!wide) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+        if (word[i] != bf16x::kVacant) w = patch_chunk_bf16x(w, word[i], chunk);
+      return w;
+    }
+    const uint32_t n = count < static_cast<uint32_t>(kWave) ? count : static_cast<uint32_t>(kWave);
+    for (uint32_t i = 0; i < n; ++i) {
+      const uint32_t v = __builtin_amdgcn_readlane(listed, i);
+      if (v == bf16x::kVacant) return w;
+      w = patch_chunk_bf16x(w, v, chunk);
+    }
+    for (uint32_t i = kWave; i < count; ++i) {  // a list of more than 64 words: a row of noise, not of weights
+      const uint32_t v = list[i];
+      if (v == bf16x::kVacant) break;
+      w = patch_chunk_bf16x(w, v, chunk);
+    }
+    return w;
+  }
+};
 
 // acc[m] += sum over the chunk's k of x[m, k] * w[k], for MT activation rows; xs points at the LDS image of
 // row 0 for this lane's chunk (x_slot(s, lane, 0)), per_row floats separate the rows.
@@ -441,11 +580,6 @@ __device__ __forceinline__ void dword_pairs(uint32_t d, bf16x2* out);
 
 template <>
 __device__ __forceinline__ void dword_pairs<LX_W_BF16>(uint32_t d, bf16x2* out) {
-  out[0] = as_bf16x2(d);
-}
-
-template <>
-__device__ __forceinline__ void dword_pairs<LX_W_BF16X>(uint32_t d, bf16x2* out) {
   out[0] = as_bf16x2(d);
 }
 
@@ -537,15 +671,11 @@ template <int F, int MT, int R, int U, bool XB = false, bool ONE = false>
 struct RowStreamer {
   Chunk<F> buf_a[U][R], buf_b[ONE ? 1 : U][ONE ? 1 : R];
   int chunks, s_begin, s_end, per_row, batches, lane;
-  // BF16X: the row pointers of rows_fn point at a record's first block (its header lies hdr_bytes before), the scale
-  // pointers at its base exponents; a row with exceptions (its first word says so) takes them from the header.
-  int hdr_bytes = 0, slots = 0;
+  // BF16X: the row pointers of rows_fn point at a record's first span (its header lies before), the scale pointers at
+  // its tops; a row with exceptions (its first word says so) takes them from the header.
+  Bf16xLane x12;
 
-  __device__ __forceinline__ void set_bf16x(int K) {
-    const bf16x::Geometry g(K);
-    hdr_bytes = g.header;
-    slots = g.slots;
-  }
+  __device__ __forceinline__ void set_bf16x(int K) { x12.set(K, threadIdx.x & (kWave - 1)); }
 
   __device__ __forceinline__ RowStreamer(int chunks_, int s_begin_, int s_end_, int per_row_)
       : chunks(chunks_), s_begin(s_begin_), s_end(s_end_), per_row(per_row_) {
@@ -566,21 +696,28 @@ struct RowStreamer {
       // A step past the range, or a chunk past the row's end, re-reads a valid chunk; it is never multiplied
       // (the step is skipped) or multiplies zeros (the x image is zero there).
       const int s = min(s_begin + batch * U + u, last_step);
-      const int chunk = min(s * kWave + lane, chunks - 1);
+      if constexpr (F == LX_W_BF16X) {
 #pragma unroll
-      for (int r = 0; r < R; ++r) load_chunk<F>(buf[u][r], rows[r], scales[r], chunk);
+        for (int r = 0; r < R; ++r) load_chunk_bf16x(buf[u][r], rows[r], scales[r], s, u == 0, x12);
+      } else {
+        const int chunk = min(s * kWave + lane, chunks - 1);
+#pragma unroll
+        for (int r = 0; r < R; ++r) load_chunk<F>(buf[u][r], rows[r], scales[r], chunk);
+      }
     }
   }
 
-  // The chunk as the products take it: BF16X is decoded to bf16 bits here (s: the chunk's step).
-  __device__ __forceinline__ Chunk<F> ready(const Chunk<F>& c, const uint8_t* row, int s) const {
+  // The chunk as the products take it: BF16X is decoded to bf16 bits here (s: the chunk's step). FIX: the row's
+  // exceptions `ex` are applied; a word's step (k / 512) is the same for the whole wavefront, so only the chunks of
+  // that step spend vector instructions on it.
+  template <bool FIX, class Ex>
+  __device__ __forceinline__ Chunk<kProductFormat<F>> ready(const Chunk<F>& c, const Ex& ex, const uint8_t* row, int s, int u) const {
     if constexpr (F == LX_W_BF16X) {
-      const uint8_t* const rec = row - hdr_bytes;
-      // One word, the same for every lane, and vacant in nearly every row.
-      const bool has = bf16x::has_exceptions(rec);
-      const uint32_t k0 = static_cast<uint32_t>(min(s * kWave + lane, chunks - 1)) * 8u;
-      Chunk<F> o;
-      o.w = bf16x::octet_bits(c.w.x, c.w.y, c.w.z, c.w.w, has ? rec : nullptr, slots, k0);
+      Chunk<LX_W_BF16> o;
+      o.w = decode_chunk_bf16x(c, s, x12);
+      if constexpr (FIX) {
+        if ((ex.steps >> u) & 1u) o.w = ex.apply(o.w, static_cast<uint32_t>(min(s * kWave + lane, chunks - 1)));
+      }
       o.scales = 0;
       return o;
     } else {
@@ -588,49 +725,78 @@ struct RowStreamer {
     }
   }
 
-  __device__ __forceinline__ void consume(const Chunk<F> (&buf)[U][R], const uint8_t* const (&rows)[R], const float* const (&xs)[R],
-                                          int batch, float (&acc)[MT][R]) {
+  // Whether any row of the batch lists exceptions (BF16X; the same answer in every lane).
+  __device__ __forceinline__ bool any_exceptions(const Chunk<F> (&buf)[U][R]) const {
+    if constexpr (F == LX_W_BF16X) {
+      bool any = false;
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int s = s_begin + batch * U + u;
-      if (s < s_end) {
-        const int slot = x_chunk_word<F, XB>(s, lane);
+      for (int r = 0; r < R; ++r) any |= __builtin_amdgcn_readlane(buf[0][r].tops, kWave - 4) != bf16x::kVacant;
+      return any;
+    } else {
+      return false;
+    }
+  }
+
+  struct NoExceptions {};
+
+  // Row r's chunk of step s (buffer slot u) into the sums.
+  template <bool FIX, class Ex>
+  __device__ __forceinline__ void consume_one(const Chunk<F>& c, const Ex& ex, const uint8_t* row, const float* x_image, int s, int u, int s_off,
+                                              int r, float (&acc)[MT][R]) {
+    const int slot = x_chunk_word<F, XB>(s - s_off, lane);
+    float a[MT];
 #pragma unroll
-        for (int r = 0; r < R; ++r) {
-          float a[MT];
+    for (int m = 0; m < MT; ++m) a[m] = acc[m][r];
+    constexpr int PF = kProductFormat<F>;
+    const Chunk<PF> ready_chunk = ready<FIX>(c, ex, row, s, u);
+    if constexpr (XB) chunk_dot2<PF, MT>(ready_chunk, reinterpret_cast<const uint32_t*>(x_image) + slot, per_row, a);
+    else chunk_fma<PF, MT>(ready_chunk, x_image + slot, per_row, a);
 #pragma unroll
-          for (int m = 0; m < MT; ++m) a[m] = acc[m][r];
-          const Chunk<F> c = ready(buf[u][r], rows[r], s);
-          if constexpr (XB) chunk_dot2<F, MT>(c, reinterpret_cast<const uint32_t*>(xs[r]) + slot, per_row, a);
-          else chunk_fma<F, MT>(c, xs[r] + slot, per_row, a);
+    for (int m = 0; m < MT; ++m) acc[m][r] = a[m];
+  }
+
+  // The steps [lo, hi) of the batch in `buf` (whose first step is s0), against images whose first step is s_off, in
+  // the order the loads were asked for (step by step). With exceptions about (FIX) it goes row by row instead, so
+  // that one row's words are live at a time; a row's sums see its steps in ascending order either way.
+  template <bool FIX>
+  __device__ __forceinline__ void consume_range(const Chunk<F> (&buf)[U][R], const uint8_t* const (&rows)[R], const float* const (&xs)[R],
+                                                int s0, int lo, int hi, int s_off, float (&acc)[MT][R]) {
+    if constexpr (FIX && F == LX_W_BF16X) {
 #pragma unroll
-          for (int m = 0; m < MT; ++m) acc[m][r] = a[m];
+      for (int r = 0; r < R; ++r) {
+        const Bf16xExceptions ex(buf[0][r], rows[r] - x12.hdr_bytes, x12.slots, s0, std::integral_constant<int, U>{});
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+          if (s0 + u >= lo && s0 + u < hi) consume_one<true>(buf[u][r], ex, rows[r], xs[r], s0 + u, u, s_off, r, acc);
+      }
+    } else {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (s0 + u >= lo && s0 + u < hi) {
+#pragma unroll
+          for (int r = 0; r < R; ++r) consume_one<false>(buf[u][r], NoExceptions{}, rows[r], xs[r], s0 + u, u, s_off, r, acc);
         }
       }
     }
   }
 
+  // A batch none of whose rows lists exceptions (nearly every batch) runs as one straight block.
+  __device__ __forceinline__ void consume_checked(const Chunk<F> (&buf)[U][R], const uint8_t* const (&rows)[R], const float* const (&xs)[R],
+                                                  int s0, int lo, int hi, int s_off, float (&acc)[MT][R]) {
+    if (any_exceptions(buf)) consume_range<true>(buf, rows, xs, s0, lo, hi, s_off, acc);
+    else consume_range<false>(buf, rows, xs, s0, lo, hi, s_off, acc);
+  }
+
+  __device__ __forceinline__ void consume(const Chunk<F> (&buf)[U][R], const uint8_t* const (&rows)[R], const float* const (&xs)[R],
+                                          int batch, float (&acc)[MT][R]) {
+    const int s0 = s_begin + batch * U;
+    consume_checked(buf, rows, xs, s0, s0, s_end, 0, acc);
+  }
+
   // The steps [lo, hi) of the single batch in `buf`, against an image whose first step is s_off.
   __device__ __forceinline__ void consume_steps(const Chunk<F> (&buf)[U][R], const uint8_t* const (&rows)[R], const float* const (&xs)[R],
                                                 int lo, int hi, int s_off, float (&acc)[MT][R]) {
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int s = s_begin + u;
-      if (s >= lo && s < hi && s < s_end) {
-        const int slot = x_chunk_word<F, XB>(s - s_off, lane);
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          float a[MT];
-#pragma unroll
-          for (int m = 0; m < MT; ++m) a[m] = acc[m][r];
-          const Chunk<F> c = ready(buf[u][r], rows[r], s);
-          if constexpr (XB) chunk_dot2<F, MT>(c, reinterpret_cast<const uint32_t*>(xs[r]) + slot, per_row, a);
-          else chunk_fma<F, MT>(c, xs[r] + slot, per_row, a);
-#pragma unroll
-          for (int m = 0; m < MT; ++m) acc[m][r] = a[m];
-        }
-      }
-    }
+    consume_checked(buf, rows, xs, s_begin, lo, hi < s_end ? hi : s_end, s_off, acc);
   }
 
   // ONE only: the group's batch against two images in turn, the first holding steps [0, split), the second the
