@@ -406,6 +406,11 @@ int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int top_k, lx
 // The bf16-stack form without a workspace argument: the scratch is taken from and returned to the stream's
 // memory pool (engine/cuda/kernels.h:220-225; the reference's kernel allocates the same way). The expert count
 // is not an argument; kMaxExperts bounds the ids this call accepts.
+// A decode step's few tokens take the decode kernels (one pass over each picked expert, no grouping tables): the
+// result is then lx_moe_experts_decode_bf16's, and lx_moe_experts_bf16x's on the encoded stacks, to the bit, as the
+// reference states of the three (engine/cuda/kernels.h:598-610). More tokens take the grouped kernels.
+static bool few_tokens(int T, int top_k) { return T <= 8 && top_k <= 8; }
+
 int lx_moe_experts(const void* latent, const int32_t* ids, const float* weights, const void* gate_up, const void* down, float* out,
                    int T, int L, int I, int top_k, void* stream) {
   if (T <= 0) return kOk;
@@ -413,9 +418,11 @@ int lx_moe_experts(const void* latent, const int32_t* ids, const float* weights,
   const lx_weight gu{LX_W_BF16, gate_up, nullptr, 1.0f, nullptr}, dn{LX_W_BF16, down, nullptr, 1.0f, nullptr};
   hipStream_t s = as_stream(stream);
   void* ws = nullptr;
-  const int64_t bytes = grouped_workspace_bytes(T, L, I, kMaxExperts, top_k, LX_MATH_BF16);
+  const bool few = few_tokens(T, top_k);
+  const int64_t bytes = few ? lx_moe_decode_workspace_bytes(T, I, top_k) : grouped_workspace_bytes(T, L, I, kMaxExperts, top_k, LX_MATH_BF16);
   if (int st = status_of(hipMallocAsync(&ws, static_cast<size_t>(bytes), s))) return st;
-  const int st = experts_grouped(latent, ids, weights, gu, dn, out, ws, T, L, I, kMaxExperts, top_k, LX_MATH_BF16, s);
+  const int st = few ? experts_decode(latent, ids, weights, gu, dn, out, ws, T, L, I, top_k, s)
+                     : experts_grouped(latent, ids, weights, gu, dn, out, ws, T, L, I, kMaxExperts, top_k, LX_MATH_BF16, s);
   const int fr = status_of(hipFreeAsync(ws, s));
   return st ? st : fr;
 }
@@ -465,7 +472,8 @@ int lx_moe_experts_noalloc(const void* latent, const int32_t* ids, const float* 
                            float* out, int T, int L, int I, int top_k, void* stream) {
   if (T <= 0) return kOk;
   if (!latent || !ids || !weights || !out || L <= 0 || I <= 0 || top_k < 1 || !gate_up || !down) return fail(kInvalid);
-  const int64_t bytes = grouped_workspace_bytes(T, L, I, kMaxExperts, top_k, LX_MATH_BF16);
+  const bool few = T <= 8 && top_k <= 8;  // as lx_moe_experts chooses
+  const int64_t bytes = few ? lx_moe_decode_workspace_bytes(T, I, top_k) : grouped_workspace_bytes(T, L, I, kMaxExperts, top_k, LX_MATH_BF16);
   if (bytes > kScratchBytes) {
     fprintf(stderr, "lx_moe_experts_noalloc: T=%d L=%d I=%d top_k=%d needs %lld bytes of scratch, the fixed array holds %lld\n", T, L,
             I, top_k, static_cast<long long>(bytes), static_cast<long long>(kScratchBytes));
@@ -475,6 +483,7 @@ int lx_moe_experts_noalloc(const void* latent, const int32_t* ids, const float* 
   void* const ws = scratch_of_current_device(&st);
   if (!ws) return st;
   const lx_weight gu{LX_W_BF16, gate_up, nullptr, 1.0f, nullptr}, dn{LX_W_BF16, down, nullptr, 1.0f, nullptr};
+  if (few) return experts_decode(latent, ids, weights, gu, dn, out, ws, T, L, I, top_k, as_stream(stream));
   return experts_grouped(latent, ids, weights, gu, dn, out, ws, T, L, I, kMaxExperts, top_k, LX_MATH_BF16, as_stream(stream));
 }
 

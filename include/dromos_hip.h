@@ -131,7 +131,9 @@ LX_API int lx_quantize_act(const void* x, lx_dtype x_dtype, int ld_x, lx_math ma
  *                           stacks, LX_MATH_FP8 on fp8 or NVFP4 stacks, LX_MATH_FP4 on NVFP4 stacks (the latent rows are
  *                           quantised per token and the intermediate rows per pair by lx_quantize_act's rule; other
  *                           pairs answer 801, engine/cpu/moe.cpp:555-569)
- *   lx_moe_experts / lx_moe_experts_decode_bf16   the bf16-stack forms of the two */
+ *   lx_moe_experts / lx_moe_experts_decode_bf16   the bf16-stack forms of the two (lx_moe_experts takes the decode
+ *                           kernels for T <= 8, top_k <= 8 and is then lx_moe_experts_decode_bf16 to the bit, the
+ *                           grouped kernels otherwise; its workspace comes from hipMallocAsync on the stream) */
 LX_API int lx_moe_route(const float* logits, const float* selection_bias, int32_t* ids, float* weights,
                         float* entropy, float* confidence, int T, int E, int top_k, void* stream);
 LX_API int lx_moe_experts(const void* latent, const int32_t* ids, const float* weights, const void* gate_up,

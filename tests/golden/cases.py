@@ -173,6 +173,49 @@ def experts_bf16(lx):
     return [latent, ids, weights, gu.data, dn.data], {"out": out}
 
 
+def _bf16x_rows(rows, K, seed):
+    """Trained-looking bf16 rows with a few values far down (exceptions within the header slots), one row with many
+    (a spill record), and a partial last span."""
+    g = torch.Generator().manual_seed(seed)
+    w = (torch.randn(rows, K, generator=g) * 0.02).to(torch.bfloat16)
+    tiny = torch.rand(rows, K, generator=g) < 3.0 / K
+    w[tiny] = (w[tiny].float() * 2.0**-40).to(torch.bfloat16)
+    w[2, ::5] = (w[2, ::5].float() * 2.0**-25).to(torch.bfloat16)
+    w[4, 7] = 0.0
+    return w
+
+
+def bf16x_codec(lx):
+    w = _bf16x_rows(9, 1160, 5000)
+    enc = ops.bf16x_encode(lx, w.to(lx.device))
+    back = ops.bf16x_decode(lx, enc, 9, 1160)
+    return [w], {"data": enc, "dequantized": back}
+
+
+def bf16x_gemv(lx):
+    N, K, M = 40, 1160, 3
+    w = _bf16x_rows(N, K, 5100)
+    g = torch.Generator().manual_seed(5101)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    bias = torch.randn(N, generator=g)
+    d = lx.device
+    enc = ops.bf16x_encode(lx, w.to(d))
+    return [w, x, bias], {"y": ops.gemv_bf16x(lx, x.to(d), enc, N, bias=bias.to(d), alpha=0.5)}
+
+
+def bf16x_experts(lx):
+    E, L, I, top_k, T = 5, 136, 72, 2, 10
+    gu = _bf16x_rows(E * 2 * I, L, 5200).view(E, 2 * I, L)
+    dn = _bf16x_rows(E * L, I, 5201).view(E, L, I)
+    g = torch.Generator().manual_seed(5202)
+    latent = torch.randn(T, L, generator=g).to(torch.bfloat16)
+    ids = torch.stack([torch.randperm(E, generator=g)[:top_k] for _ in range(T)]).to(torch.int32)
+    weights = torch.softmax(torch.randn(T, top_k, generator=g), -1).float()
+    d = lx.device
+    out = ops.experts_bf16x(lx, latent.to(d), ids.to(d), weights.to(d), ops.bf16x_encode(lx, gu.to(d)), ops.bf16x_encode(lx, dn.to(d)), I, top_k)
+    return [latent, ids, weights, gu, dn], {"out": out}
+
+
 CASES = {}
 for _f in ("int8", "fp8", "nvfp4"):
     CASES[f"quantize_{_f}"] = (quantize, (_f,))
@@ -197,6 +240,9 @@ CASES["router"] = (router, ())
 CASES["gemm_bf16"] = (gemm_bf16, ())
 CASES["route"] = (route, ())
 CASES["experts_bf16"] = (experts_bf16, ())
+CASES["bf16x_codec"] = (bf16x_codec, ())
+CASES["bf16x_gemv"] = (bf16x_gemv, ())
+CASES["bf16x_experts"] = (bf16x_experts, ())
 
 # Outputs whose bits every backend must reproduce (codec and index work); the rest are f32 sums whose last
 # bits depend on the summation order (the reference's own differ between its ISA levels).

@@ -105,6 +105,9 @@ def test_experts_equal_the_bf16_experts_bit_for_bit(hip, oracle, T, E, L, I, top
     err = rel_l2(got, want)
     assert err <= 2e-3, err
     if T <= 8:
+        # engine/cuda/kernels.h:598-610: a decode step's lx_moe_experts on the bf16 stacks gives the same bits
+        legacy = ops.experts_bf16(hip, latent, ids, weights, gu, dn, I, top_k)
+        assert torch.equal(bits(legacy), bits(got))
         via = ops.experts_decode(hip, latent, ids, weights, Weight(W_BF16X, gu_x), Weight(W_BF16X, dn_x), I, top_k)
         assert torch.equal(bits(via), bits(got))
         assert ops.experts_decode(hip, latent, ids, weights, Weight(W_BF16X, gu_x), Weight(W_BF16, dn), I, top_k, status=True) == 801
