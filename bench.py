@@ -123,6 +123,33 @@ def make_gemv_case(lx, torch, fmt, M, N, K, seed, entry, invariant=False, math=0
     return step, nbytes, (ws, structs, ptrs, x, y, ws_buf)
 
 
+def make_bf16x_case(lx, torch, M, N, K, seed):
+    """lx_gemv_bf16x on rotated encodings of one bf16 master. Bytes: the encoded weight + x + y."""
+    from dromos_amd.abi import F32
+    from dromos_amd.formats import master_weight
+
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    master = master_weight(N, K, g).cuda()
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    size = lx.lib.lx_bf16x_bytes
+    size.restype = ctypes.c_int64
+    n = int(size(ctypes.c_void_p(master.data_ptr()), ctypes.c_int64(N), ctypes.c_int(K), lx.stream))
+    enc = torch.empty(n, dtype=torch.uint8, device="cuda")
+    assert lx.status("bf16x_encode", master, ctypes.c_int64(N), K, enc, ctypes.c_int64(n)) == 0
+    torch.cuda.synchronize()
+    del master
+    copies = max(3, -(-(640 << 20) // n))
+    encs = [enc] + [enc.clone() for _ in range(copies - 1)]
+    y = torch.empty(M, N, dtype=torch.float32, device="cuda")
+    nbytes = n + M * K * 2 + M * N * 4
+
+    def step(i):
+        st = lx.status("gemv_bf16x", x, 1, K, encs[i % copies], None, F32, y, F32, N, M, N, K, 1.0, 0.0)
+        assert st == 0, st
+
+    return step, nbytes, (encs, x, y)
+
+
 def make_moe_case(lx, torch, fmt, T, E, L, I, top_k, seed, steps_total):
     """A routed-experts step (route + experts) on bf16 / quantised stacks. Bytes: distinct experts x per-expert
     bytes, averaged over the steps' seeded routings, + latent + out + routing."""
@@ -362,6 +389,18 @@ def main():
             # inside the call, exact int32 sums); the bytes are the weight-only count.
             run_gemv(f"C2 int8 M={M} INT8 math", "int8", M, 14336, 4096, 1000 + M, entry="gemm_w", math=1)
             run_gemv(f"C2 fp8 M={M} FP8 math", "fp8", M, 14336, 4096, 1000 + M, entry="gemm_w", math=2)
+        for N, K in ((4096, 4096), (14336, 4096)):
+            # Not a headline configuration: the lossless 12-bit form of bf16 weights; the bytes are the encoding's, so
+            # GB/s is what the kernel streams and us_per_step compares with the bf16 product of the same shape.
+            step, nbytes, keep = make_bf16x_case(lx, torch, 1, N, K, 7000 + N)
+            us = timer.run(step, K_STEPS, W)
+            cases.append({"case": f"bf16x {N}x{K} M=1", "entry": "lx_gemv_bf16x", "format": "bf16x", "M": 1, "N": N, "K": K,
+                          "us_per_step": round(us, 3), "bytes_per_step": int(nbytes), "GBps": round(nbytes / us / 1e3, 1),
+                          "frac_of_hbm_peak": round(nbytes / us / 1e3 / HBM_PEAK_GBPS, 4), "bf16_bytes": 2 * N * K})
+            del keep
+            torch.cuda.empty_cache()
+            if (N, K) != (4096, 4096):
+                run_gemv(f"bf16 {N}x{K} M=1", "bf16", 1, N, K, 7000 + N)
         for T in (1, 8, 32, 64):
             run_moe(f"C4 moe bf16 T={T}", "bf16", T, 64, 2048, 1024, 8, 3000 + T)
         run_layer()

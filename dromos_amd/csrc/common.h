@@ -81,14 +81,34 @@ __device__ __forceinline__ float dpp_move(float v) {
   return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
 }
 
+// The two halves of an exchange across 16-lane rows (ROWS16: every lane gets its own value and that of the lane 16
+// away) or across the halves of the wavefront (32 away), by gfx950's lane-swap instructions: vector ALU work, where a
+// shuffle would go through the LDS pipeline and be waited for. In every lane {a, b} is {own, other} or {other, own}:
+// callers combine them with a commutative operation.
+template <bool ROWS16>
+__device__ __forceinline__ void swap_halves(float v, float& a, float& b) {
+  const uint32_t u = __float_as_uint(v);
+  if constexpr (ROWS16) {
+    const auto r = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    a = __uint_as_float(r[0]);
+    b = __uint_as_float(r[1]);
+  } else {
+    const auto r = __builtin_amdgcn_permlane32_swap(u, u, false, false);
+    a = __uint_as_float(r[0]);
+    b = __uint_as_float(r[1]);
+  }
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
   v += dpp_move<0xB1>(v);   // quad_perm [1, 0, 3, 2]
   v += dpp_move<0x4E>(v);   // quad_perm [2, 3, 0, 1]
   v += dpp_move<0x141>(v);  // row_half_mirror: the other quad of the half row
   v += dpp_move<0x140>(v);  // row_mirror: the other half of the 16-lane row
-  v += __shfl_xor(v, 16);
-  v += __shfl_xor(v, 32);
-  return v;
+  float a, b;
+  swap_halves<true>(v, a, b);  // the lane 16 away
+  v = a + b;
+  swap_halves<false>(v, a, b);  // the lane 32 away
+  return a + b;
 }
 
 __device__ __forceinline__ float wave_max(float v) {
@@ -96,9 +116,11 @@ __device__ __forceinline__ float wave_max(float v) {
   v = fmaxf(v, dpp_move<0x4E>(v));
   v = fmaxf(v, dpp_move<0x141>(v));
   v = fmaxf(v, dpp_move<0x140>(v));
-  v = fmaxf(v, __shfl_xor(v, 16));
-  v = fmaxf(v, __shfl_xor(v, 32));
-  return v;
+  float a, b;
+  swap_halves<true>(v, a, b);
+  v = fmaxf(a, b);
+  swap_halves<false>(v, a, b);
+  return fmaxf(a, b);
 }
 
 // ---- the weight formats as a wave streams them --------------------------------------------------------

@@ -137,6 +137,21 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs
       stage_all();
     }
   } else {
+    if constexpr (XB) {
+      if (a.phase_steps == 0) {
+        // Several bf16 rows: ask for them, then for the weights, and only then wait for the rows (loads return in
+        // order): the image is in place while the weights are still on their way, and each chunk is multiplied as it
+        // arrives instead of after everything has.
+        XRowRegsN<MT> xr;
+        stage_rows_load<F>(xr, static_cast<const uint16_t*>(a.x), a.ld_x, nullptr, a.M, a.K, steps);
+        st.prefetch(rows_fn, group, 0, 1);
+        if (xr.ready) stage_rows_store<F, MT>(xr, reinterpret_cast<uint32_t*>(xs), a.M, a.K, steps);
+        else stage_all();
+        __syncthreads();
+        st.run(rows_fn, done_fn, group, 0, 1);
+        return;
+      }
+    }
     st.prefetch(rows_fn, group, 0, 1);
     if constexpr (XB && ONE) {
       if (a.phase_steps > 0) {

@@ -276,23 +276,25 @@ __device__ __forceinline__ void stage_x_store_pairs(const XRegs<XV>& r, uint32_t
 // (row m, pass j) in row-major order, a thread's piece of a slot being vector j * blockDim + thread of row m. Usable
 // when the rows can be read 16 bytes at a time and there are at most kSlots slots; otherwise `ready` is false and
 // the caller falls back to stage_x_pairs.
-struct XRowRegs {
-  static constexpr int kSlots = 4;
+template <int SLOTS>
+struct XRowRegsN {
+  static constexpr int kSlots = SLOTS;
   u32x4 v[kSlots];
   int iters;  // passes per row
   bool ready;
 };
+using XRowRegs = XRowRegsN<4>;
 
-template <int F>
-__device__ __forceinline__ void stage_rows_load(XRowRegs& r, const uint16_t* x, int64_t ld_x, const int* row_of, int M, int64_t K,
+template <int F, int SLOTS>
+__device__ __forceinline__ void stage_rows_load(XRowRegsN<SLOTS>& r, const uint16_t* x, int64_t ld_x, const int* row_of, int M, int64_t K,
                                                 int steps) {
   const int n_vec = x_row_words<F, true>(steps) >> 2, k_vec = static_cast<int>(K) >> 3;
   r.iters = (n_vec + blockDim.x - 1) / blockDim.x;
-  r.ready = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && ((ld_x * 2) & 15) == 0 && (K & 7) == 0 && M * r.iters <= XRowRegs::kSlots;
+  r.ready = (reinterpret_cast<uintptr_t>(x) & 15) == 0 && ((ld_x * 2) & 15) == 0 && (K & 7) == 0 && M * r.iters <= SLOTS;
   if (!r.ready) return;
   int m = 0, j = 0;
 #pragma unroll
-  for (int u = 0; u < XRowRegs::kSlots; ++u) {
+  for (int u = 0; u < SLOTS; ++u) {
     // Clamped addresses (no predicated loads); what lies past K or M is replaced by zeros when it is stored.
     const int v = min(static_cast<int>(threadIdx.x) + j * static_cast<int>(blockDim.x), k_vec - 1);
     const int mc = min(m, M - 1);
@@ -301,14 +303,14 @@ __device__ __forceinline__ void stage_rows_load(XRowRegs& r, const uint16_t* x, 
   }
 }
 
-template <int F, int MT>
-__device__ __forceinline__ void stage_rows_store(const XRowRegs& r, uint32_t* xs, int M, int64_t K, int steps) {
+template <int F, int MT, int SLOTS>
+__device__ __forceinline__ void stage_rows_store(const XRowRegsN<SLOTS>& r, uint32_t* xs, int M, int64_t K, int steps) {
   constexpr int E = Fmt<F>::kElems;
   const int per_row = x_row_words<F, true>(steps);
   const int n_vec = per_row >> 2, k_vec = static_cast<int>(K) >> 3;
   int m = 0, j = 0;
 #pragma unroll
-  for (int u = 0; u < XRowRegs::kSlots; ++u) {
+  for (int u = 0; u < SLOTS; ++u) {
     const int v = threadIdx.x + j * blockDim.x;
     if (m < M && v < n_vec) {
       const int k = v << 3, st = k / (kWave * E), within = k % (kWave * E);
