@@ -9,7 +9,10 @@
 // reduction-order contract of the skinny GEMM, for every weight format.
 #include <stdlib.h>
 
+#include <map>
+#include <mutex>
 #include <type_traits>
+#include <utility>
 
 #include "common.h"
 #include "tile_mfma.h"
@@ -50,6 +53,7 @@ struct GemmArgs {
   const int8_t* xq;     // the INT8 math: quantised activations [M, K], rows K bytes apart
   const float* xscale;  // and their per-row scales
   const float* act_scale;  // BF16-math kernels on a quantised math's activation images: the rows' scales (else null)
+  void* partial;  // slab kernel with S > 1: the slices' partial tiles, [S][M][N] words (f32, or i32 for the INT8 math)
 };
 
 // The epilogue's operation order (engine/cpu/gemm.cpp:21-34); rf is the row factor, b the bias (0 without one).
@@ -738,6 +742,328 @@ bool launch_window(GemmArgs a, int* status, hipStream_t stream) {
   return true;
 }
 
+// ---- up to 64 activation rows, many tiles: the slab kernel ------------------------------------------------------
+//
+// The same arithmetic once more (a tile's K slices, each one ascending chain from zero, added in ascending order), laid
+// out so that the activations cost little: a workgroup takes ONE K slice (blockIdx.y) of many tiles, so its image is
+// the slice's columns of the M rows and nothing else, staged once; its wavefronts then walk their tiles' slices without
+// ever meeting again (no window to cross, no barrier after the first). With S > 1 the slices of a tile are in different
+// workgroups: each writes its partial tile to `partial`, and slab_reduce_kernel adds them in ascending slice order and
+// runs the epilogue, which is what the other kernels' first wavefront does through LDS. Neither the tiles a workgroup
+// takes nor which wavefront takes which enters a sum.
+template <int F, int MATH, bool XF32, int MT>
+__global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a) {
+  extern __shared__ __align__(16) f32x4 lds4[];
+  constexpr bool I8 = MATH != LX_MATH_BF16;
+  constexpr int E = Fmt<F>::kElems, J = I8 ? 1 : E / 8;
+  constexpr int CB = I8 ? 16 : E * 2;  // image bytes under one lane's 16-byte weight chunk
+  constexpr int SB = 4 * CB;           // image bytes of one load step
+  constexpr int SP = SB / 16;          // and its 16-byte pieces
+  using Acc = typename std::conditional<MATH == LX_MATH_INT8, i32x4, f32x4>::type;
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int waves = blockDim.x / kWave;
+  const int S = a.S, w = blockIdx.y, spw = a.steps_per_wave, t_begin = w * spw;
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const int tile_first = blockIdx.x * a.tiles_per_wg, tile_end = min(n_tiles, tile_first + a.tiles_per_wg);
+  const int g = lane >> 4, i = lane & 15;
+  uint8_t* const ximg = reinterpret_cast<uint8_t*>(lds4);
+
+  // A tile's loads, straight into the lanes that feed the matrix instruction: lane (g, i) takes chunk 4 s + g of row i
+  // for load step s (64 contiguous bytes of each of the tile's 16 rows per instruction). The LDS belongs to the image.
+  struct TilePtrs {
+    const uint8_t* row;        // this lane's row of the tile
+    const uint8_t* own_scale;  // NVFP4: its block scales
+  };
+  auto ptrs_of = [&](int t) {
+    TilePtrs p;
+    const int n0 = min(t, n_tiles - 1) * kTileRows, valid = min(kTileRows, a.N - n0);
+    const int64_t n = static_cast<int64_t>(n0) + min(i, valid - 1);
+    p.row = a.w + n * a.row_bytes;
+    p.own_scale = a.scale + n * a.scale_row_bytes;
+    return p;
+  };
+  u32x4 raw[2][4];
+  uint32_t sc[8];
+  auto issue_group = [&](const TilePtrs& p, int tb, int grp) {
+#pragma unroll
+    for (int st = 0; st < 4; ++st) {
+      const int c = min(4 * (tb + 4 * grp + st) + g, a.chunks - 1);
+      raw[grp][st] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p.row + static_cast<uint32_t>(c) * 16u));
+      if constexpr (F == LX_W_NVFP4) sc[4 * grp + st] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(p.own_scale) + c);
+    }
+  };
+  int tile = tile_first + wave;
+  TilePtrs cur = ptrs_of(tile);
+  if (tile < tile_end) {
+    issue_group(cur, t_begin, 0);
+    issue_group(cur, t_begin, 1);
+  }
+
+  // The image: row m holds the activations under steps [t_begin, t_begin + spw), zero from K on, in pieces of 16 image
+  // bytes; the weights above are already on their way.
+  {
+    const char* const xsrc = I8 ? reinterpret_cast<const char*>(a.xq) : static_cast<const char*>(a.xs.x);
+    const int64_t x_ld_bytes = I8 ? a.K : a.xs.ld * (XF32 ? 4 : 2);
+    const int row_pieces = spw * SP, pieces = a.M * row_pieces;
+    constexpr int kAhead = XF32 ? 2 : 4;
+    for (int v0 = threadIdx.x; v0 < pieces; v0 += kAhead * blockDim.x) {
+      u32x4 xr[kAhead][XF32 ? 2 : 1];
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+        const int v = min(v0 + u * static_cast<int>(blockDim.x), pieces - 1);
+        const int m = v / row_pieces, c = v - m * row_pieces;
+        const int piece = min(t_begin * SP + c, a.x_vecs - 1);  // clamped, zeroed when stored
+        const char* src = xsrc + m * x_ld_bytes + static_cast<int64_t>(piece) * (XF32 ? 32 : 16);
+        xr[u][0] = *reinterpret_cast<const u32x4*>(src);
+        if constexpr (XF32) xr[u][1] = *reinterpret_cast<const u32x4*>(src + 16);
+      }
+#pragma unroll
+      for (int u = 0; u < kAhead; ++u) {
+        const int v = v0 + u * blockDim.x;
+        const int m = v / row_pieces, c = v - m * row_pieces;
+        u32x4 val = xr[u][0];
+        if constexpr (XF32) {
+          bf16x2 q[4] = {pack_bf16(__uint_as_float(xr[u][0].x), __uint_as_float(xr[u][0].y)),
+                         pack_bf16(__uint_as_float(xr[u][0].z), __uint_as_float(xr[u][0].w)),
+                         pack_bf16(__uint_as_float(xr[u][1].x), __uint_as_float(xr[u][1].y)),
+                         pack_bf16(__uint_as_float(xr[u][1].z), __uint_as_float(xr[u][1].w))};
+          val = __builtin_bit_cast(u32x4, q);
+        }
+        if (t_begin * SP + c >= a.x_vecs) val = u32x4{0u, 0u, 0u, 0u};
+        // A piece past the image goes to a spare slot behind it (no branch around the store).
+        *reinterpret_cast<u32x4*>(ximg + (v < pieces ? m * a.x_pitch + c * 16 : a.M * a.x_pitch)) = val;
+      }
+    }
+  }
+  __syncthreads();
+
+  const uint8_t* xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) xrow[mt] = ximg + min(mt * 16 + i, a.M - 1) * a.x_pitch + g * CB;
+  const bool bias_f32 = a.bias && a.bias_dtype == LX_F32;
+  for (; tile < tile_end; tile += waves) {
+    const int next_tile = tile + waves;
+    const TilePtrs next = ptrs_of(next_tile < tile_end ? next_tile : tile);
+    Acc acc[MT];
+#pragma unroll
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = Acc{0, 0, 0, 0};
+    for (int off = 0; off < spw; off += 8) {
+#pragma unroll
+      for (int grp = 0; grp < 2; ++grp) {
+        uint32_t scales[4];
+        u32x4 grp_w[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          scales[u] = F == LX_W_NVFP4 ? sc[4 * grp + u] : 0u;
+          grp_w[u] = raw[grp][u];
+        }
+        // The same group of the next batch: of this tile, or of the wavefront's next one.
+        if (off + 8 < spw) issue_group(cur, t_begin + off + 8, grp);
+        else if (next_tile < tile_end) issue_group(next, t_begin, grp);
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+          const int so = off + 4 * grp + 2 * half;  // step within the slice
+          u32x4 wv[2];
+#pragma unroll
+          for (int st = 0; st < 2; ++st) wv[st] = grp_w[2 * half + st];
+#pragma unroll
+          for (int st = 0; st < 2; ++st) {
+            if (t_begin + so + st < a.steps) {
+#pragma unroll
+              for (int mt = 0; mt < MT; ++mt) {
+                const uint8_t* xs = xrow[mt] + (so + st) * SB;
+                if constexpr (I8) {
+                  acc[mt] = byte_mfma<MATH>(__builtin_bit_cast(i32x4, wv[st]), *reinterpret_cast<const i32x4*>(xs), acc[mt]);
+                } else {
+#pragma unroll
+                  for (int j = 0; j < J; ++j)
+                    acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(weight_fragment<F>(wv[st], scales[2 * half + st], j),
+                                                                      *reinterpret_cast<const bf16x8*>(xs + 16 * j), acc[mt], 0, 0, 0);
+                }
+              }
+            }
+          }
+        }
+      }
+    }
+    // The tile's slice is done: the partial tile, or with one slice the result itself.
+    const int nq = tile * kTileRows + 4 * g;
+    if (S > 1) {
+      Acc* const out = static_cast<Acc*>(a.partial) + 0;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + i;
+        if (m >= a.M) continue;
+        // Words (slice, m, n): this lane's four are consecutive.
+        uint32_t* at = reinterpret_cast<uint32_t*>(out) + (static_cast<int64_t>(w) * a.M + m) * a.N + nq;
+        if ((a.N & 3) == 0) {
+          *reinterpret_cast<Acc*>(at) = acc[mt];
+        } else {
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (nq + r < a.N) at[r] = __builtin_bit_cast(uint32_t, acc[mt][r]);
+        }
+      }
+    } else {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        const int m = mt * 16 + i;
+        if (m >= a.M) continue;
+        const float xscale = I8 ? a.xscale[m] : 1.0f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const int n = nq + r;
+          if (n < a.N) {
+            const float rf = I8 ? reinterpret_cast<const float*>(a.scale)[n] : row_factor(F, a.scale, a.global, n);
+            const float b = !a.bias ? 0.0f : bias_f32 ? static_cast<const float*>(a.bias)[n] : load_as_f32(a.bias, a.bias_dtype, n);
+            write_out(a, m, n, static_cast<float>(acc[mt][r]), I8 ? rf * xscale : rf, b);
+          }
+        }
+      }
+    }
+    cur = next;
+  }
+}
+
+// The slab kernel's second half for S > 1: out[m, n] from the S partial sums of (m, n), added in ascending slice order
+// from slice 0's, then the epilogue. One thread per (m, four consecutive n).
+template <int F, int MATH>
+__global__ void __launch_bounds__(256) slab_reduce_kernel(const GemmArgs a) {
+  constexpr bool I8 = MATH != LX_MATH_BF16;
+  using Acc = typename std::conditional<MATH == LX_MATH_INT8, i32x4, f32x4>::type;
+  using Word = typename std::conditional<MATH == LX_MATH_INT8, int, float>::type;
+  const int quads = (a.N + 3) / 4;
+  const int64_t item = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+  if (item >= static_cast<int64_t>(a.M) * quads) return;
+  const int m = static_cast<int>(item / quads), n0 = static_cast<int>(item - static_cast<int64_t>(m) * quads) * 4;
+  const Word* p = static_cast<const Word*>(a.partial) + static_cast<int64_t>(m) * a.N + n0;
+  const int64_t slice_words = static_cast<int64_t>(a.M) * a.N;
+  Acc sum;
+  if ((a.N & 3) == 0) {
+    sum = *reinterpret_cast<const Acc*>(p);
+    for (int sl = 1; sl < a.S; ++sl) sum += *reinterpret_cast<const Acc*>(p + sl * slice_words);
+  } else {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+      Word v = 0;
+      if (n0 + r < a.N) {
+        v = p[r];
+        for (int sl = 1; sl < a.S; ++sl) v += p[r + sl * slice_words];
+      }
+      sum[r] = v;
+    }
+  }
+  const bool bias_f32 = a.bias && a.bias_dtype == LX_F32;
+  const float xscale = I8 ? a.xscale[m] : 1.0f;
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const int n = n0 + r;
+    if (n < a.N) {
+      const float rf = I8 ? reinterpret_cast<const float*>(a.scale)[n] : row_factor(F, a.scale, a.global, n);
+      const float b = !a.bias ? 0.0f : bias_f32 ? static_cast<const float*>(a.bias)[n] : load_as_f32(a.bias, a.bias_dtype, n);
+      write_out(a, m, n, static_cast<float>(sum[r]), I8 ? rf * xscale : rf, b);
+    }
+  }
+}
+
+// The slab kernel's partial tiles live in a buffer the library keeps per (device, stream): calls on one stream run one
+// after the other, so they can share it, and a call that is being captured into a graph can use it where it could not
+// ask for memory. It is made by the first call on the stream that needs one (never during a capture: that call takes the
+// windowed kernel instead) and kept until the process ends.
+constexpr size_t kSlabScratchBytes = 64u << 20;
+
+void* slab_scratch(hipStream_t stream, size_t bytes, bool capturing) {
+  if (bytes > kSlabScratchBytes) return nullptr;
+  static std::mutex lock;
+  static std::map<std::pair<int, hipStream_t>, void*> buffers;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> g(lock);
+  void*& slot = buffers[{dev, stream}];
+  if (!slot && !capturing) {
+    if (hipMalloc(&slot, kSlabScratchBytes) != hipSuccess) {
+      (void)hipGetLastError();
+      slot = nullptr;
+    }
+  }
+  return slot;
+}
+
+// Where the slab kernel is tried before the windowed one. Measured on MI355X (fp8 and int8 weights, bf16 activations):
+// it wins where the windowed kernel's workgroups, which each stage all of K, are few or long: more than 48 rows
+// with at most 400 tiles (6144 x 4096 at 64 rows: 37 -> 25 us), and more than 16 rows with K >= 8192 and few tiles
+// (4096 x 8192 at 32 rows: 21 -> 18 us, at 64: 36 -> 26 us). With many tiles (14336 x 4096) its second pass over the
+// partial tiles costs more than the windows do. LX_SLAB_MIN_ROWS (a tuning knob) overrides: rows from which it is tried.
+inline bool slab_wanted(int M, int n_tiles, int64_t K) {
+  if (const char* e = getenv("LX_SLAB_MIN_ROWS")) return M >= atoi(e);
+  return n_tiles <= 400 && (M > 48 || (M > 16 && K >= 8192));
+}
+
+// Launches the slab kernel for a.M <= 64 rows; false when it does not apply: the slice's image does not fit LDS, the
+// matrix has too few tiles to give every compute unit a slab, or (S > 1) the stream is being captured, where the
+// partial tiles' memory cannot be asked for.
+template <int F, int MATH>
+bool launch_slab(GemmArgs a, int* status, hipStream_t stream) {
+  constexpr bool I8 = MATH != LX_MATH_BF16;
+  constexpr int SB = 4 * (I8 ? 16 : Fmt<F>::kElems * 2);
+  const int S = a.S, spw = a.steps_per_wave;
+  if (spw % 8 != 0 || S < 1) return false;
+  const bool xf32 = !I8 && a.xs.dtype == LX_F32;
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const size_t pitch = static_cast<size_t>(spw) * SB + 16;
+  const size_t image = static_cast<size_t>(a.M) * pitch + 16;
+  // One slab per compute unit and slice round: tiles_per_wg tiles of one slice, up to sixteen wavefronts on them.
+  const int slabs = compute_units() / S > 0 ? compute_units() / S : 1;
+  const int tpw = (n_tiles + slabs - 1) / slabs;
+  const int waves = tpw < 4 ? 4 : tpw > kMaxSplit ? kMaxSplit : tpw;
+  const size_t lds = image;
+  if (lds > kLdsMax - 1024) return false;
+  if (n_tiles * S < compute_units() * 4) return false;  // too little work to give every unit a slab of several tiles
+  void* partial = nullptr;
+  if (S > 1) {
+    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
+    // (The null stream is never captured, and asking about it is an error in some runtimes.)
+    if (stream && hipStreamIsCapturing(stream, &cap) != hipSuccess) {
+      (void)hipGetLastError();
+      return false;
+    }
+    partial = slab_scratch(stream, sizeof(float) * static_cast<size_t>(S) * a.M * a.N, cap != hipStreamCaptureStatusNone);
+    if (!partial) return false;
+  }
+  a.partial = partial;
+  a.tiles_per_wg = tpw;
+  a.x_vecs = a.K * (I8 ? 1 : 2) / 16;
+  a.x_pitch = static_cast<int>(pitch);
+  const dim3 grid((n_tiles + tpw - 1) / tpw, S);
+  auto launch = [&](auto kernel) {
+    if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), kLdsMax);
+    hipLaunchKernelGGL(kernel, grid, dim3(waves * kWave), lds, stream, a);
+    return status_of(hipGetLastError());
+  };
+  auto with_mt = [&](auto mt_tag) {
+    constexpr int MT = decltype(mt_tag)::value;
+    if constexpr (I8) return launch(slab_kernel<F, MATH, false, MT>);
+    else return xf32 ? launch(slab_kernel<F, MATH, true, MT>) : launch(slab_kernel<F, MATH, false, MT>);
+  };
+  int st;
+  switch ((a.M + 15) / 16) {
+    case 1: st = with_mt(std::integral_constant<int, 1>{}); break;
+    case 2: st = with_mt(std::integral_constant<int, 2>{}); break;
+    case 3: st = with_mt(std::integral_constant<int, 3>{}); break;
+    default: st = with_mt(std::integral_constant<int, 4>{}); break;
+  }
+  if (!st && S > 1) {
+    const int64_t items = static_cast<int64_t>(a.M) * ((a.N + 3) / 4);
+    hipLaunchKernelGGL((slab_reduce_kernel<F, MATH>), dim3(static_cast<unsigned>((items + 255) / 256)), dim3(256), 0, stream, a);
+    st = status_of(hipGetLastError());
+  }
+  *status = st;
+  return true;
+}
+
 // Launches the lean tile kernel for a.M <= 16 rows when its LDS image fits; false if it does not.
 template <int F, int MATH>
 bool launch_tile16(GemmArgs a, int* status, hipStream_t stream) {
@@ -1000,6 +1326,7 @@ int launch_skinny(GemmArgs a, hipStream_t stream) {
   // sixteen-wavefront workgroups; the lean kernel's image of all of K leaves too few of them resident there).
   if (MT > 1 || (a.M > 8 && n_tiles >= 320)) {
     int st = kOk;
+    if (slab_wanted(a.M, static_cast<int>(n_tiles), a.K) && launch_slab<F, LX_MATH_BF16>(a, &st, stream)) return st;
     if (launch_window<F, LX_MATH_BF16>(a, &st, stream)) return st;
   }
   if constexpr (MT == 1) {
@@ -1225,6 +1552,7 @@ int gemm_bytes_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w
         return status_of(hipGetLastError());
       };
       const int mt = (a.M + 15) / 16;
+      if ((mt > 1 || (a.M > 8 && n_tiles >= 320)) && slab_wanted(a.M, static_cast<int>(n_tiles), K) && launch_slab<F, MATH>(a, &st, s)) continue;
       if ((mt > 1 || (a.M > 8 && n_tiles >= 320)) && launch_window<F, MATH>(a, &st, s)) continue;
       if (mt == 1 && launch_tile16<F, MATH>(a, &st, s)) continue;
       if (mt == 1) {

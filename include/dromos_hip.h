@@ -88,6 +88,11 @@ LX_API int lx_gemv_decode_bf16(const void* x, lx_dtype x_dtype, int ld_x, const 
  * The quantised maths keep the activations' scales and bytes in the workspace (lx_gemm_workspace_bytes); with a
  * null workspace they take scratch from the stream's memory pool instead (hipMallocAsync / hipFreeAsync, as the
  * reference's kernels do: such a call allocates and cannot be captured in a graph).
+ * For some shapes (17 .. 64 rows, few weight tiles) the product is split over K between workgroups and a second
+ * kernel adds the partial sums in the fixed order: their memory is a buffer of 64 MiB that the library makes once
+ * per (device, stream), on the first such call outside a graph capture, and keeps until the process ends. Calls on
+ * one stream share it (they run one after the other); a graph captured with such a call must be launched on the
+ * stream it was captured on, or not at the same time as other lx_gemm_w calls there.
  * lx_gemm_skinny: bf16 x, up to 64 rows per pass, every format, with the reduction-order contract of
  * engine/cuda/kernels.h:457-474: the K split depends on (N, K) only, never on M, so a row's bits do not
  * depend on the batch. With the environment variable LX_BATCH_INVARIANT set (non-empty, not starting

@@ -268,3 +268,62 @@ def test_c3_shape_under_the_fp4_math(hip, oracle):
     want = ops.gemm_w(oracle, x, w.to("cpu"), MATH_FP4)
     err = rel_l2(got, want)
     assert err <= 1e-2 and err <= 1e-4, err
+
+
+# ---- the slab kernel (a workgroup per K slice of many tiles, partial tiles added by a second kernel) ----------------
+
+
+@pytest.mark.parametrize("fmt", FMT)
+@pytest.mark.parametrize("M,N,K", [(64, 6144, 4096), (32, 4096, 8192), (40, 2048, 8192), (57, 6000, 2048)])
+def test_slab_shapes_give_the_bits_of_every_other_kernel(hip, fmt, M, N, K):
+    # Shapes the slab kernel takes by itself: their rows equal the same rows computed sixteen at a time (the lean tile
+    # kernel) bit for bit, with bias, alpha and a bf16 output in the epilogue of the second pass.
+    g = torch.Generator().manual_seed(M + N)
+    w = random_weight(FORMATS[fmt], N, K, N + K).to("cuda")
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    bias = torch.randn(N, generator=g).cuda()
+    for y_dtype in (torch.float32, torch.bfloat16):
+        big = ops.gemm_w(hip, x, w, MATH_BF16, bias=bias, alpha=0.5, y_dtype=y_dtype)
+        for m0 in (0, 16, M - 16):
+            part = ops.gemm_w(hip, x[m0:m0 + 16].contiguous(), w, MATH_BF16, bias=bias, alpha=0.5, y_dtype=y_dtype)
+            assert torch.equal(big[m0:m0 + 16].view(torch.int16 if y_dtype == torch.bfloat16 else torch.int32),
+                               part.view(torch.int16 if y_dtype == torch.bfloat16 else torch.int32)), (y_dtype, m0)
+    want = ops.gemv_reference(x.cpu(), w.to("cpu").dense(), bias.cpu(), 0.5, 0.0, None)
+    checks.check_product(ops.gemm_w(hip, x, w, MATH_BF16, bias=bias, alpha=0.5).cpu(), want)
+
+
+@pytest.mark.parametrize("fmt", FMT)
+@pytest.mark.parametrize("M,N,K", [(17, 1027, 2048), (64, 300, 4096), (33, 4096, 1040), (48, 14336, 4096)])
+def test_slab_forced_equals_the_windowed_kernel(hip, fmt, M, N, K):
+    # The tuning knob sends any row count to the slab kernel where it fits (ragged N and K included): same bits as
+    # without it, for f32 and bf16 activations and beta != 0.
+    g = torch.Generator().manual_seed(N)
+    w = random_weight(FORMATS[fmt], N, K - K % 16, N).to("cuda")
+    K = K - K % 16
+    for x_dtype in (torch.bfloat16, torch.float32):
+        x = torch.randn(M, K, generator=g).to(x_dtype).cuda()
+        y0 = torch.randn(M, N, generator=g).cuda()
+        try:
+            os.environ["LX_SLAB_MIN_ROWS"] = "1000"
+            a = ops.gemm_w(hip, x, w, MATH_BF16, y=y0.clone(), alpha=1.25, beta=-0.5)
+            os.environ["LX_SLAB_MIN_ROWS"] = "1"
+            b = ops.gemm_w(hip, x, w, MATH_BF16, y=y0.clone(), alpha=1.25, beta=-0.5)
+        finally:
+            os.environ.pop("LX_SLAB_MIN_ROWS", None)
+        assert torch.equal(a.view(torch.int32), b.view(torch.int32)), x_dtype
+
+
+@pytest.mark.parametrize("math,fmt", [(MATH_INT8, "int8"), (MATH_FP8, "fp8")])
+def test_slab_under_the_byte_maths(hip, oracle, math, fmt):
+    M, N, K = 64, 6144, 4096
+    g = torch.Generator().manual_seed(9)
+    w = random_weight(FORMATS[fmt], N, K, 5)
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    got = ops.gemm_w(hip, x.cuda(), w.to("cuda"), math)
+    part = ops.gemm_w(hip, x[:16].contiguous().cuda(), w.to("cuda"), math)
+    assert torch.equal(got[:16].view(torch.int32), part.view(torch.int32))
+    want = ops.gemm_w(oracle, x, w, math)
+    if math == MATH_INT8:
+        assert torch.equal(got.cpu().view(torch.int32), want.view(torch.int32))  # exact integer sums
+    else:
+        assert rel_l2(got, want) <= 1e-4  # f32 sums of exact products against the double sums of the reference
