@@ -273,7 +273,8 @@ def main():
     ap.add_argument("--cases", default="all", choices=["headline", "gemv", "all", "layer"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="no timing: one 256 MiB device copy (the counters' yardstick) and 20 eager headline launches")
+                    help="no timing: one 256 MiB device copy (the counters' yardstick), then eager launches of the headline "
+                         "GEMV, the 16- and 64-row products, the one-token experts and the 32-token grouped experts")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported (one MI355X per box)")
@@ -290,12 +291,31 @@ def main():
         b = torch.ones(256 << 20, dtype=torch.uint8, device="cuda")
         for _ in range(3):
             a.copy_(b)  # reads 256 MiB and writes 256 MiB
+        del a, b
+        probe = {"copy_bytes_read": 256 << 20, "copy_bytes_written": 256 << 20, "launches": {}}
+
+        def launches(name, step, nbytes, n):
+            for i in range(n):
+                step(i)
+            torch.cuda.synchronize()
+            probe["launches"][name] = {"algorithmic_bytes_per_step": int(nbytes), "steps": n}
+
         step, nbytes, keep = make_gemv_case(lx, torch, "int8", 1, 14336, 4096, 1001, "gemv_w")
-        for i in range(20):
-            step(i)
-        torch.cuda.synchronize()
-        print(json.dumps({"pmc_probe": {"copy_bytes_read": 256 << 20, "copy_bytes_written": 256 << 20,
-                                        "gemv_algorithmic_bytes": nbytes, "gemv_launches": 20}}))
+        launches("C2 int8 M=1 (gemv_stream_kernel)", step, nbytes, 20)
+        del keep
+        for M in (16, 64):
+            step, nbytes, keep = make_gemv_case(lx, torch, "int8", M, 14336, 4096, 1000 + M, "gemm_w")
+            launches(f"C2 int8 M={M} (window_kernel)", step, nbytes, 10)
+            del keep
+        torch.cuda.empty_cache()
+        step, nbytes, keep, _ = make_moe_case(lx, torch, "bf16", 1, 64, 2048, 1024, 8, 3001, 16)
+        launches("C4 moe bf16 T=1 (route + decode_gate_up + decode_down)", step, nbytes, 16)
+        del keep
+        torch.cuda.empty_cache()
+        step, nbytes, keep, _ = make_moe_case(lx, torch, "fp8", 32, 128, 4096, 1536, 8, 5032, 8)
+        launches("C5 moe fp8 T=32 E=128 (route + group + grouped_gate_up + grouped_down + grouped_sum)", step, nbytes, 8)
+        del keep
+        print(json.dumps({"pmc_probe": probe}))
         return
     timer = Timer(lx, torch)
     K_STEPS, W = args.steps, args.warmup
