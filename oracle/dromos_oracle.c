@@ -17,9 +17,13 @@
  *   lx_dequantize_weight             pinned: closed-form dense values from the stored bytes
  *   lx_quantize_act                  pinned: the per-token rules in torch with IEEE f32 operations, FP4 tie / underflow cases
  *   lx_gemv* / lx_gemm_w / _skinny   pinned: float64 x @ W^T on the decoded values
- *   lx_gemm_w INT8 / FP8 maths       pinned: exact integer / float64 products of the quantised values, bit for bit
+ *   lx_gemm_w INT8 / FP8 / FP4 maths pinned: exact integer / float64 products of the quantised values, bit for bit
+ *   lx_gemm_bf16, lx_spec_gemv_f32   pinned: float64 x @ W^T + bias
+ *   lx_router_route                  pinned: equals lx_spec_gemv_f32 followed by lx_moe_route, word for word
+ *   lx_moe_summary(_history)         pinned: float64 weighted sums of the expert embeddings, the history's closed form
  *   lx_moe_route                     pinned: stable sort of -(logit + bias) + float64 softmax, tie cases
- *   lx_moe_experts*                  pinned: float64 experts with the bf16-rounded intermediate
+ *   lx_moe_experts* (every math)     pinned: float64 experts with the bf16-rounded intermediate (quantised maths: on the
+ *                                    quantised rows' exact values)
  *   lx_bf16x_* / *_bf16x             pinned: decode(encode(w)) == w over every exponent pattern incl. spilled rows, sizes
  *                                    by closed form, hand-built records; the products equal the bf16 products' bits
  */
