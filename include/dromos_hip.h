@@ -266,6 +266,44 @@ LX_API int lx_rt_device_props(int ordinal, lx_device_props* props);
 LX_API int lx_rt_mem_info(int64_t* free_bytes, int64_t* total_bytes);
 LX_API int lx_bandwidth_probe(int64_t bytes, int reps, double* read_gbps, double* spec_gbps, void* stream);
 
+/* ---- a model folder -> the weights on the device (the C form of the loader interface of engine/core/checkpoint.h:24-101;
+ * behaviour: engine/core/checkpoint.cpp). Host code, load time: these calls read files, allocate and synchronise. ---------
+ * A folder is safetensors (model.safetensors, or the shards model.safetensors.index.json names). A tensor's dtype names
+ * its format: BF16; F8_E4M3 with an F32 weight_scale per row (compressed-tensors FP8); U8 nibble pairs with an e4m3
+ * weight_scale per 16 values and an F32 weight_scale_2 per expert (GPTQ NVFP4). With the target equal to the folder's
+ * own format every projection is held exactly as the file stores it; otherwise the target's recipe decides per
+ * projection, and a projection whose file format differs is converted on the device (bf16 values, copied or
+ * dequantised, rounded by lx_quantize_weight; lx_bf16x_encode for LX_W_BF16X) one expert at a time. LX_W_NVFP4 loads
+ * only from an NVFP4 folder (round-to-nearest to NVFP4 is refused, as in the reference). The tied head "lm_head" comes
+ * from embedding.weight, whose bf16 gather table is a plain tensor. The model's config is not read here: shapes are
+ * taken from the file and checked against the formats' layouts, not against a config.
+ *   lx_ckpt_projection_format  the recipe: the format `projection` ("layers.4.mixer.qkv", "embedding") is held in under
+ *                              `target` (checkpoint.h: projection_format)
+ *   lx_ckpt_stored_format      LX_W_BF16 / LX_W_FP8 / LX_W_NVFP4: what the folder holds; -1 and lx_ckpt_error() on failure
+ *   lx_ckpt_load               0 and a handle, or 1 with the reason in lx_ckpt_error(); skip_experts leaves the routed
+ *                              expert stacks off the device (their shapes, formats and sizes stay readable)
+ *   lx_ckpt_projection         the lx_weight of a loaded projection ([N, K] or a stack [E, N, K]); null when absent or skipped
+ *   lx_ckpt_expert             expert e of a projection as its own lx_weight (its rows, scales and global)
+ *   lx_ckpt_expert_bytes       bytes of one expert's data and scales in the format it is (or would be) held in
+ *   lx_ckpt_tensor             a plain tensor (norms, embeddings, routers, biases): device pointer, dtype, shape */
+typedef struct lx_ckpt lx_ckpt;
+LX_API const char* lx_ckpt_error(void);
+LX_API int lx_ckpt_projection_format(lx_wtype target, const char* projection);
+LX_API int lx_ckpt_stored_format(const char* dir);
+LX_API int lx_ckpt_load(const char* dir, lx_wtype target, int skip_experts, lx_ckpt** out);
+LX_API void lx_ckpt_free(lx_ckpt* c);
+LX_API const lx_weight* lx_ckpt_projection(const lx_ckpt* c, const char* name);
+LX_API int lx_ckpt_count(const lx_ckpt* c);
+LX_API const char* lx_ckpt_name(const lx_ckpt* c, int i);
+LX_API int lx_ckpt_shape(const lx_ckpt* c, const char* name, int64_t* E, int64_t* N, int64_t* K, int* stack);
+LX_API int lx_ckpt_format_of(const lx_ckpt* c, const char* name);
+LX_API int lx_ckpt_expert(const lx_ckpt* c, const char* name, int64_t e, lx_weight* out);
+LX_API int lx_ckpt_expert_bytes(const lx_ckpt* c, const char* name, int64_t* data, int64_t* scale);
+LX_API const void* lx_ckpt_tensor(const lx_ckpt* c, const char* name, lx_dtype* dtype, int* rank, int64_t* shape, int capacity);
+LX_API int lx_ckpt_target(const lx_ckpt* c);
+LX_API int64_t lx_ckpt_device_bytes(const lx_ckpt* c);
+LX_API int64_t lx_ckpt_peak_device_bytes(const lx_ckpt* c);
+
 /* ---- measurement floors (no counterpart in the reference: for benches that state how far a product is from a
  * plain read of the same bytes). Both are asynchronous and capturable.
  *   lx_probe_read   reads `bytes` bytes at `data` (16-byte aligned) once, as the decode GEMV streams a weight: 16-byte

@@ -25,7 +25,8 @@ def test_header_declares_the_hot_path():
                  "lx_moe_experts_decode", "lx_moe_decode_workspace_bytes", "lx_moe_experts_decode_bf16",
                  "lx_moe_bf16x_workspace_bytes", "lx_moe_experts_grouped", "lx_moe_grouped_workspace_bytes",
                  "lx_bf16x_row_bytes", "lx_bf16x_bytes", "lx_bf16x_encode", "lx_bf16x_decode", "lx_gemv_bf16x",
-                 "lx_moe_experts_bf16x", "lx_rt_backend", "lx_rt_device_count", "lx_arch", "lx_tune_variants", "lx_bandwidth_probe"):
+                 "lx_moe_experts_bf16x", "lx_ckpt_load", "lx_ckpt_projection", "lx_ckpt_projection_format", "lx_ckpt_stored_format",
+                 "lx_ckpt_expert", "lx_ckpt_tensor", "lx_ckpt_free", "lx_rt_backend", "lx_rt_device_count", "lx_arch", "lx_tune_variants", "lx_bandwidth_probe"):
         assert must in names, must
 
 

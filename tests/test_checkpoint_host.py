@@ -1,0 +1,101 @@
+"""Host logic of the model-folder loader (lx_ckpt_*): the recipe, what a folder holds, and the safetensors reader's
+refusals. No device call is made here (the library is only loaded)."""
+
+import json
+import struct
+
+import pytest
+
+import folders
+from dromos_amd.abi import Kernels, W_BF16, W_BF16X, W_FP8, W_INT8, W_NVFP4, hip_library_path
+from dromos_amd.checkpoint import ModelWeights, projection_format
+
+
+@pytest.fixture(scope="module")
+def lib():
+    path = hip_library_path()
+    if not path.exists():
+        pytest.fail(f"{path} is not built: run `python -m dromos_amd.build`")
+    return Kernels(path, "cpu")
+
+
+def test_recipe_known_answers(lib):
+    # engine/core/checkpoint.cpp:15-27 in words, and recipe() at :124-166.
+    wide = ["layers.3.mixer.impl.mixer.out_proj", "layers.3.mixer.pass_lora_down", "layers.3.mixer.pass_lora_up", "layers.3.depth_memory.metadata_write"]
+    for target in (W_BF16, W_INT8, W_FP8, W_NVFP4, W_BF16X):
+        for key in wide:
+            assert projection_format(lib, target, key) == W_BF16, (target, key)
+        for key in ("layers.1.depth_memory.key", "layers.1.depth_memory.value"):
+            assert projection_format(lib, target, key) == (W_FP8 if target == W_NVFP4 else W_BF16)
+    assert [projection_format(lib, t, "embedding") for t in (W_BF16, W_INT8, W_FP8, W_NVFP4, W_BF16X)] == [W_BF16, W_INT8, W_BF16, W_FP8, W_BF16X]
+    experts = ["layers.0.moe.local_experts.gate_up", "layers.0.moe.local_experts.down"]
+    fp8_dense = ["layers.0.mixer.impl.mixer.in_proj", "layers.0.mixer.qkv", "layers.0.mixer.out"]
+    other = ["layers.0.moe.latent_down", "layers.0.moe.latent_up", "layers.0.moe.shared_expert.gate_up", "layers.0.depth_memory.query"]
+    for key in experts + fp8_dense + other:
+        assert projection_format(lib, W_BF16, key) == W_BF16
+        assert projection_format(lib, W_INT8, key) == W_INT8
+        assert projection_format(lib, W_BF16X, key) == W_BF16X
+    for key in experts + fp8_dense:
+        assert projection_format(lib, W_FP8, key) == W_FP8
+    for key in other:
+        assert projection_format(lib, W_FP8, key) == W_BF16
+    for key in experts:
+        assert projection_format(lib, W_NVFP4, key) == W_NVFP4
+    assert projection_format(lib, W_NVFP4, "layers.0.moe.latent_up") == W_BF16
+    for key in fp8_dense + ["layers.0.moe.latent_down", "layers.0.moe.shared_expert.gate_up"]:
+        assert projection_format(lib, W_NVFP4, key) == W_FP8
+    # the ".weight" suffix is optional; a component must match whole ("xmixer.qkv" is not "mixer.qkv")
+    assert projection_format(lib, W_FP8, "layers.0.mixer.qkv.weight") == W_FP8
+    assert projection_format(lib, W_FP8, "layers.0.xmixer.qkv") == W_BF16
+
+
+@pytest.mark.parametrize("layout,fmt", [("bf16", W_BF16), ("fp8", W_FP8), ("nvfp4", W_NVFP4)])
+@pytest.mark.parametrize("shards", [1, 3])
+def test_stored_format(lib, tmp_path, layout, fmt, shards):
+    folders.write(tmp_path, layout, shards=shards)
+    assert ModelWeights.stored_format(lib, tmp_path) == fmt
+
+
+def test_reader_refusals(lib, tmp_path):
+    with pytest.raises(RuntimeError, match="cannot open"):
+        ModelWeights.stored_format(lib, tmp_path / "nowhere")
+    d = tmp_path / "short"
+    d.mkdir()
+    (d / "model.safetensors").write_bytes(b"abc")
+    with pytest.raises(RuntimeError, match="too short"):
+        ModelWeights.stored_format(lib, d)
+
+    def folder(name, header, payload=b"\0" * 64, length=None):
+        f = tmp_path / name
+        f.mkdir()
+        body = json.dumps(header).encode() if not isinstance(header, bytes) else header
+        (f / "model.safetensors").write_bytes(struct.pack("<Q", len(body) if length is None else length) + body + payload)
+        return f
+
+    with pytest.raises(RuntimeError, match="longer than the file"):
+        ModelWeights.stored_format(lib, folder("long", {}, length=1 << 40))
+    with pytest.raises(RuntimeError, match="not valid JSON"):
+        ModelWeights.stored_format(lib, folder("json", b'{"a": [1, 2'))
+    with pytest.raises(RuntimeError, match="outside the file"):
+        ModelWeights.stored_format(lib, folder("outside", {"a": {"dtype": "F32", "shape": [64], "data_offsets": [0, 256]}}))
+    with pytest.raises(RuntimeError, match="shape says otherwise"):
+        ModelWeights.stored_format(lib, folder("bytes", {"a": {"dtype": "F32", "shape": [3], "data_offsets": [0, 8]}}))
+    with pytest.raises(RuntimeError, match="unknown dtype"):
+        ModelWeights.stored_format(lib, folder("dtype", {"a": {"dtype": "F4", "shape": [8], "data_offsets": [0, 8]}}))
+    with pytest.raises(RuntimeError, match="lacks dtype"):
+        ModelWeights.stored_format(lib, folder("lacks", {"a": {"dtype": "F32", "shape": [2]}}))
+    # metadata is skipped, escapes in names are read
+    ok = folder("ok", {"__metadata__": {"format": "pt"}, "a\\u0041.weight": {"dtype": "BF16", "shape": [2, 2], "data_offsets": [0, 8]}})
+    assert ModelWeights.stored_format(lib, ok) == W_BF16
+    # an index that sends a tensor to the wrong shard
+    folders.write(tmp_path / "sharded", "bf16", shards=2)
+    idx = tmp_path / "sharded" / "model.safetensors.index.json"
+    doc = json.loads(idx.read_text())
+    names = sorted(doc["weight_map"])
+    doc["weight_map"][names[0]] = doc["weight_map"][names[1]]
+    idx.write_text(json.dumps(doc))
+    with pytest.raises(RuntimeError, match="does not hold it"):
+        ModelWeights.stored_format(lib, tmp_path / "sharded")
+    idx.write_text(json.dumps({"metadata": {}}))
+    with pytest.raises(RuntimeError, match="weight_map"):
+        ModelWeights.stored_format(lib, tmp_path / "sharded")
