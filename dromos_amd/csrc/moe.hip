@@ -21,6 +21,14 @@ constexpr int kMaxPairs = 64;
 
 // ---- routing ---------------------------------------------------------------------------------------------
 
+// A biased logit as an unsigned number that orders as the float does: a greater float is a greater number, -0 and +0
+// are the same number, and a NaN is 0, below every other (-inf is 0x007fffff): it is picked before nothing.
+__device__ __forceinline__ uint32_t order_key(float b) {
+  const uint32_t u = __float_as_uint(b);
+  const uint32_t k = (u & 0x80000000u) ? ~u : u | 0x80000000u;
+  return b != b ? 0u : b == 0.0f ? 0x80000000u : k;
+}
+
 // One wavefront per token; a lane keeps its NPL logits (elements lane, lane + 64, ...) in registers, so the row
 // is read once. E <= 64 * NPL. The picks: with few experts (NPL <= 4) every element is ranked against all the
 // others (its rank among the biased logits, ties to the lower index, is its pick number); with many, top_k
@@ -32,7 +40,7 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
                                                          int E, int top_k) {
   __shared__ float picked_logit[kWaves][64];
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int64_t t = static_cast<int64_t>(blockIdx.x) * kWaves + wave;
+  const int64_t t = static_cast<int64_t>(blockIdx.x) * (blockDim.x / kWave) + wave;
   if (t >= T) return;
   const float* row = logits + t * E;
   float v[NPL], biased[NPL];
@@ -68,19 +76,25 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
     confidence[t] = 1.0f / z;  // the largest probability is exp(0) / z
   }
   if constexpr (NPL <= 4) {
+    // Element (u, ~index) as one 64-bit number: another element is picked before this one exactly when its number
+    // is the greater (a greater biased logit, or the same and a lower index).
+    uint32_t key[NPL];
+    uint64_t mine64[NPL];
     int rank[NPL];
 #pragma unroll
-    for (int j = 0; j < NPL; ++j) rank[j] = 0;
+    for (int j = 0; j < NPL; ++j) {
+      key[j] = order_key(biased[j]);
+      mine64[j] = static_cast<uint64_t>(key[j]) << 32 | static_cast<uint32_t>(~(lane + j * kWave));
+      rank[j] = 0;
+    }
 #pragma unroll
     for (int j2 = 0; j2 < NPL; ++j2) {
-      for (int l2 = 0; l2 < kWave; ++l2) {
-        const float other = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(biased[j2]), l2));
-        const int oi = l2 + j2 * kWave;
 #pragma unroll
-        for (int j = 0; j < NPL; ++j) {
-          const int i = lane + j * kWave;
-          rank[j] += (other > biased[j] || (other == biased[j] && oi < i)) && oi < E;
-        }
+      for (int l2 = 0; l2 < kWave; ++l2) {
+        const uint64_t other = static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(static_cast<int>(key[j2]), l2))) << 32 |
+                               static_cast<uint32_t>(~(l2 + j2 * kWave));
+#pragma unroll
+        for (int j = 0; j < NPL; ++j) rank[j] += other > mine64[j];
       }
     }
     int ranked = 0;
@@ -141,12 +155,17 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
   }
   __builtin_amdgcn_wave_barrier();
   __threadfence_block();
-  // Weights: softmax over the picks of their unbiased logits, summed in pick order.
+  // Weights: softmax over the picks of their unbiased logits, summed in pick order. Lane r takes pick r's logit.
+  const float mine = lane < top_k ? picked_logit[wave][lane] : NAN;
   float lmax = -INFINITY;
-  for (int r = 0; r < top_k; ++r) lmax = picked_logit[wave][r] > lmax ? picked_logit[wave][r] : lmax;
+  for (int r = 0; r < top_k; ++r) {
+    const float p = __int_as_float(__builtin_amdgcn_readlane(__float_as_int(mine), r));
+    lmax = p > lmax ? p : lmax;
+  }
+  const float ex = __expf(mine - lmax);
   float esum = 0.0f;
-  for (int r = 0; r < top_k; ++r) esum += __expf(picked_logit[wave][r] - lmax);
-  if (lane < top_k) weights[t * top_k + lane] = __expf(picked_logit[wave][lane] - lmax) / esum;
+  for (int r = 0; r < top_k; ++r) esum += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(ex), r));
+  if (lane < top_k) weights[t * top_k + lane] = ex / esum;
 }
 
 // The pairs of a step with more than one token, sorted by expert (stable), as the gate/up stage reads them:
@@ -532,7 +551,9 @@ int route(const float* logits, const float* selection_bias, int32_t* ids, float*
   if (T <= 0) return kOk;
   if (top_k < 1 || top_k > 64 || top_k > E || !logits || !ids || !weights || !entropy || !confidence) return fail(kInvalid);
   if (E > 4096) return fail(kNotSupported);
-  const dim3 grid((T + kWaves - 1) / kWaves), block(kThreads);
+  // One token: one wavefront, not a workgroup of sixteen of which fifteen leave at once.
+  const int waves = T < kWaves ? T : kWaves;
+  const dim3 grid((T + waves - 1) / waves), block(waves * kWave);
   if (E <= 64) hipLaunchKernelGGL(route_kernel<1>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
   else if (E <= 128) hipLaunchKernelGGL(route_kernel<2>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);
   else if (E <= 256) hipLaunchKernelGGL(route_kernel<4>, grid, block, 0, s, logits, selection_bias, ids, weights, entropy, confidence, T, E, top_k);

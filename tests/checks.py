@@ -241,6 +241,34 @@ def route_ties(lx):
     close(weights, torch.softmax(torch.tensor([[1.0, 0.0]]), -1), atol=1e-6)
 
 
+def awkward_logits(E, top_k, T=48):
+    """Logits and a bias where floats are awkward for a pick order: many equal values, signed zeros (equal: the lower
+    index goes first), denormals (distinct from zero), infinities and NaNs (never picked while anything else can be),
+    rows of one value, a row with fewer rankable values than picks."""
+    g = torch.Generator().manual_seed(E * 31 + top_k)
+    pool = torch.tensor([0.0, -0.0, 1e-40, -1e-40, 1.0, 1.0, -1.0, 2.5, float("inf"), float("-inf"), float("nan"), -float("nan"), 3e-39])
+    logits = pool[torch.randint(0, len(pool), (T, E), generator=g)].contiguous()
+    logits[0] = 0.0
+    logits[1] = float("-inf")
+    logits[2] = float("nan")
+    logits[3, : E // 2] = -0.0
+    logits[4] = torch.where(torch.arange(E) % 2 == 0, torch.tensor(-0.0), torch.tensor(0.0))
+    logits[5, top_k - 1:] = float("nan")
+    bias = pool[torch.randint(0, 8, (E,), generator=g)].contiguous()
+    return logits, bias
+
+
+def same_routes(a, w, E):
+    """Two lx_moe_route results: the same ids; the same weights on every row whose picks all exist. A row with fewer
+    rankable logits than picks gets the id E for the rest, and its weights are not compared: the reference's softmax
+    then reads the element behind the row (engine/cpu/moe.cpp:383-395), which is nobody's contract."""
+    assert torch.equal(a[0].cpu(), w[0].cpu())
+    whole = (a[0].cpu() < E).all(-1)
+    x, y = a[1].cpu()[whole], w[1].cpu()[whole]
+    both = torch.isnan(x) & torch.isnan(y)
+    close(torch.where(both, 0.0, x), torch.where(both, 0.0, y), atol=1e-5)
+
+
 # ---- experts ------------------------------------------------------------------------------------------------
 
 

@@ -34,6 +34,14 @@ def test_route_matches_the_oracle(hip, oracle):
         close(u, v, atol=1e-5)
 
 
+
+@pytest.mark.parametrize("E,top_k", [(64, 8), (40, 8), (128, 8), (200, 6), (256, 64), (512, 8)])
+def test_route_picks_on_awkward_values_match_the_oracle(hip, oracle, E, top_k):
+    logits, bias = checks.awkward_logits(E, top_k)
+    for b in (None, bias):
+        checks.same_routes(ops.route(hip, logits.cuda(), None if b is None else b.cuda(), top_k), ops.route(oracle, logits, b, top_k), E)
+
+
 def test_route_empty_and_invalid(hip):
     logits = torch.zeros(2, 8, device="cuda")
     ids = torch.zeros(2, 2, dtype=torch.int32, device="cuda")

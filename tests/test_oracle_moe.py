@@ -24,6 +24,13 @@ def test_route_without_bias_and_ties(oracle):
     checks.route_ties(oracle)
 
 
+@pytest.mark.parametrize("E,top_k", [(64, 8), (40, 8), (128, 8), (200, 6), (256, 64), (512, 8)])
+def test_route_on_awkward_values_equals_the_reference_backend(oracle, ref, E, top_k):
+    logits, bias = checks.awkward_logits(E, top_k)
+    for b in (None, bias):
+        checks.same_routes(ops.route(oracle, logits, b, top_k), ops.route(ref, logits, b, top_k), E)
+
+
 def test_route_equals_the_reference_backend(oracle, ref):
     g = torch.Generator().manual_seed(5)
     logits = torch.randn(64, 128, generator=g) * 2
