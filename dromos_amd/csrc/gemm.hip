@@ -702,8 +702,9 @@ bool launch_window(GemmArgs a, int* status, hipStream_t stream) {
   const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
   auto image = [&](int win) { return static_cast<size_t>(a.M) * (static_cast<size_t>(S) * win * SB + 16) + 16; };
   auto lds_for = [&](int tpw, int win) { return static_cast<size_t>(tpw) * S * kStageBytes + image(win); };
-  // Tiles to a workgroup: sixteen wavefronts' worth (the more tiles share an image, the less the activations cost).
-  const int tpw = kMaxSplit / S;
+  // Tiles to a workgroup: four at most (the more tiles share an image, the less the activations cost, but workgroups
+  // of sixteen wavefronts are too few to cover the device: 16384 x 4096 at 32 rows 24.7 -> 20.9 us with four tiles).
+  const int tpw = kMaxSplit / S < 4 ? kMaxSplit / S : 4;
   // The window: the largest of 8, 4, 2 steps whose image fits LDS and whose pieces its threads can hold.
   const size_t held = (xf32 ? 2u : 4u) * tpw * S * kWave;
   int win = 8;
@@ -805,13 +806,17 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
     const char* const xsrc = I8 ? reinterpret_cast<const char*>(a.xq) : static_cast<const char*>(a.xs.x);
     const int64_t x_ld_bytes = I8 ? a.K : a.xs.ld * (XF32 ? 4 : 2);
     const int row_pieces = spw * SP, pieces = a.M * row_pieces;
-    constexpr int kAhead = XF32 ? 2 : 4;
+    // A piece's row and place in it: a shift and a mask where a row's pieces are a power of two (row_shift >= 0), as
+    // they are for most K; a division costs a wavefront dozens of instructions per piece.
+    const int row_shift = a.row_shift;
+    auto row_of = [&](int v) { return row_shift >= 0 ? v >> row_shift : v / row_pieces; };
+    constexpr int kAhead = XF32 ? 4 : 8;
     for (int v0 = threadIdx.x; v0 < pieces; v0 += kAhead * blockDim.x) {
       u32x4 xr[kAhead][XF32 ? 2 : 1];
 #pragma unroll
       for (int u = 0; u < kAhead; ++u) {
         const int v = min(v0 + u * static_cast<int>(blockDim.x), pieces - 1);
-        const int m = v / row_pieces, c = v - m * row_pieces;
+        const int m = row_of(v), c = v - m * row_pieces;
         const int piece = min(t_begin * SP + c, a.x_vecs - 1);  // clamped, zeroed when stored
         const char* src = xsrc + m * x_ld_bytes + static_cast<int64_t>(piece) * (XF32 ? 32 : 16);
         xr[u][0] = *reinterpret_cast<const u32x4*>(src);
@@ -820,7 +825,7 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
 #pragma unroll
       for (int u = 0; u < kAhead; ++u) {
         const int v = v0 + u * blockDim.x;
-        const int m = v / row_pieces, c = v - m * row_pieces;
+        const int m = row_of(min(v, pieces - 1)), c = v - m * row_pieces;
         u32x4 val = xr[u][0];
         if constexpr (XF32) {
           bf16x2 q[4] = {pack_bf16(__uint_as_float(xr[u][0].x), __uint_as_float(xr[u][0].y)),
@@ -940,8 +945,16 @@ __global__ void __launch_bounds__(256) slab_reduce_kernel(const GemmArgs a) {
   const int64_t slice_words = static_cast<int64_t>(a.M) * a.N;
   Acc sum;
   if ((a.N & 3) == 0) {
+    // Up to eight slices' words are asked for at once (a slice past the last repeats it and is not added).
     sum = *reinterpret_cast<const Acc*>(p);
-    for (int sl = 1; sl < a.S; ++sl) sum += *reinterpret_cast<const Acc*>(p + sl * slice_words);
+    for (int base = 1; base < a.S; base += 8) {
+      Acc part[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) part[u] = *reinterpret_cast<const Acc*>(p + min(base + u, a.S - 1) * slice_words);
+#pragma unroll
+      for (int u = 0; u < 8; ++u)
+        if (base + u < a.S) sum += part[u];
+    }
   } else {
 #pragma unroll
     for (int r = 0; r < 4; ++r) {
@@ -992,14 +1005,15 @@ void* slab_scratch(hipStream_t stream, size_t bytes, bool capturing) {
   return slot;
 }
 
-// Where the slab kernel is tried before the windowed one. Measured on MI355X (fp8 and int8 weights, bf16 activations):
-// it wins where the windowed kernel's workgroups, which each stage all of K, are few or long: more than 48 rows
-// with at most 400 tiles (6144 x 4096 at 64 rows: 37 -> 25 us), and more than 16 rows with K >= 8192 and few tiles
-// (4096 x 8192 at 32 rows: 21 -> 18 us, at 64: 36 -> 26 us). With many tiles (14336 x 4096) its second pass over the
-// partial tiles costs more than the windows do. LX_SLAB_MIN_ROWS (a tuning knob) overrides: rows from which it is tried.
+// Where the slab kernel is tried before the windowed one. Measured on MI355X (fp8, int8 and bf16 weights, bf16
+// activations): it wins where the windowed kernel's workgroups, which each stage all of K, are few or long: more than 32
+// rows with at most 400 tiles (6144 x 4096 at 48 rows: 29 -> 21 us, at 64: 37 -> 24 us), and more than 16 rows with
+// K >= 8192 and few tiles (4096 x 8192 at 32 rows: 21 -> 17 us, at 64: 35 -> 24 us). With many tiles (14336 x 4096) its
+// second pass over the partial tiles costs more than the windows do. LX_SLAB_MIN_ROWS (a tuning knob) overrides: rows
+// from which it is tried.
 inline bool slab_wanted(int M, int n_tiles, int64_t K) {
   if (const char* e = getenv("LX_SLAB_MIN_ROWS")) return M >= atoi(e);
-  return n_tiles <= 400 && (M > 48 || (M > 16 && K >= 8192));
+  return n_tiles <= 400 && (M > 32 || (M > 16 && K >= 8192));
 }
 
 // Launches the slab kernel for a.M <= 64 rows; false when it does not apply: the slice's image does not fit LDS, the
@@ -1037,6 +1051,10 @@ bool launch_slab(GemmArgs a, int* status, hipStream_t stream) {
   a.tiles_per_wg = tpw;
   a.x_vecs = a.K * (I8 ? 1 : 2) / 16;
   a.x_pitch = static_cast<int>(pitch);
+  const int row_pieces = spw * (SB / 16);
+  a.row_shift = -1;
+  for (int sh = 0; sh < 20; ++sh)
+    if ((1 << sh) == row_pieces) a.row_shift = sh;
   const dim3 grid((n_tiles + tpw - 1) / tpw, S);
   auto launch = [&](auto kernel) {
     if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), kLdsMax);
