@@ -795,13 +795,12 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
   };
   int tile = tile_first + wave;
   TilePtrs cur = ptrs_of(tile);
-  if (tile < tile_end) {
-    issue_group(cur, t_begin, 0);
-    issue_group(cur, t_begin, 1);
-  }
 
   // The image: row m holds the activations under steps [t_begin, t_begin + spw), zero from K on, in pieces of 16 image
-  // bytes; the weights above are already on their way.
+  // bytes. Loads return in the order they were asked for: the first round of activations is asked for BEFORE the
+  // weights, so the image is complete (and the matrix instructions can start on the first weights) while most of the
+  // weights are still on their way; asked for behind them, the activations would arrive last and the whole slab would
+  // be loaded before any of it is multiplied.
   {
     const char* const xsrc = I8 ? reinterpret_cast<const char*>(a.xq) : static_cast<const char*>(a.xs.x);
     const int64_t x_ld_bytes = I8 ? a.K : a.xs.ld * (XF32 ? 4 : 2);
@@ -811,8 +810,8 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
     const int row_shift = a.row_shift;
     auto row_of = [&](int v) { return row_shift >= 0 ? v >> row_shift : v / row_pieces; };
     constexpr int kAhead = XF32 ? 4 : 8;
-    for (int v0 = threadIdx.x; v0 < pieces; v0 += kAhead * blockDim.x) {
-      u32x4 xr[kAhead][XF32 ? 2 : 1];
+    u32x4 xr[kAhead][XF32 ? 2 : 1];
+    auto ask = [&](int v0) {
 #pragma unroll
       for (int u = 0; u < kAhead; ++u) {
         const int v = min(v0 + u * static_cast<int>(blockDim.x), pieces - 1);
@@ -822,6 +821,8 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
         xr[u][0] = *reinterpret_cast<const u32x4*>(src);
         if constexpr (XF32) xr[u][1] = *reinterpret_cast<const u32x4*>(src + 16);
       }
+    };
+    auto put = [&](int v0) {
 #pragma unroll
       for (int u = 0; u < kAhead; ++u) {
         const int v = v0 + u * blockDim.x;
@@ -838,6 +839,16 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
         // A piece past the image goes to a spare slot behind it (no branch around the store).
         *reinterpret_cast<u32x4*>(ximg + (v < pieces ? m * a.x_pitch + c * 16 : a.M * a.x_pitch)) = val;
       }
+    };
+    ask(threadIdx.x);
+    // (A wavefront without a tile asks for a valid one's all the same: behind a branch the compiler could not count the
+    // loads in flight and would make the stores below wait for all of them.)
+    issue_group(cur, t_begin, 0);
+    issue_group(cur, t_begin, 1);
+    put(threadIdx.x);
+    for (int v0 = threadIdx.x + kAhead * blockDim.x; v0 < pieces; v0 += kAhead * blockDim.x) {
+      ask(v0);
+      put(v0);
     }
   }
   __syncthreads();
