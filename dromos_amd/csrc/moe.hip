@@ -184,10 +184,13 @@ __global__ void __launch_bounds__(kWave) decode_sort_kernel(const int32_t* __res
   const int p = threadIdx.x;
   // A lane past P holds an id above every other: it ranks behind all pairs and is never written.
   const int mine = p < P ? ids[p] : 0x7fffffff;
+  // (id, index) as one 64-bit number: one compare a pair, all 64 lanes' numbers unrolled.
+  const uint64_t mine64 = static_cast<uint64_t>(static_cast<uint32_t>(mine)) << 32 | static_cast<uint32_t>(p);
   int rank = 0;
-  for (int q = 0; q < P; ++q) {
-    const int other = __builtin_amdgcn_readlane(mine, q);
-    rank += other < mine || (other == mine && q < p);
+#pragma unroll
+  for (int q = 0; q < kWave; ++q) {
+    const uint64_t other = static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(mine, q))) << 32 | static_cast<uint32_t>(q);
+    rank += other < mine64;
   }
   if (p < P) {
     s_ids[p] = mine;
