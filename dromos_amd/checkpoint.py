@@ -42,7 +42,7 @@ def _lib(lx):
 
 
 def _error(lib):
-    return RuntimeError(lib.lx_ckpt_error().decode())
+    return RuntimeError(lib.lx_ckpt_error().decode("utf-8", "replace"))  # a damaged file's names may not be text
 
 
 def projection_format(lx, target, projection):

@@ -99,3 +99,43 @@ def test_reader_refusals(lib, tmp_path):
     idx.write_text(json.dumps({"metadata": {}}))
     with pytest.raises(RuntimeError, match="weight_map"):
         ModelWeights.stored_format(lib, tmp_path / "sharded")
+
+
+def test_damaged_files_are_refused_or_read_never_worse(lib, tmp_path):
+    """Random damage to the headers, the index and the file sizes of a one-file and a three-shard folder: every answer is
+    a format or a refusal with a reason (a reader that trusted a length or an offset would fault instead)."""
+    import random
+
+    rnd = random.Random(20)
+    folders.write(tmp_path / "one", "fp8", shards=1)
+    folders.write(tmp_path / "three", "nvfp4", shards=3)
+    good = {(d, f.name): f.read_bytes() for d in ("one", "three") for f in (tmp_path / d).iterdir()}
+    refused = 0
+    for _ in range(400):
+        key = rnd.choice(sorted(good))
+        data = bytearray(good[key])
+        span = 8 + struct.unpack("<Q", data[:8])[0] if key[1].endswith(".safetensors") else len(data)
+        kind = rnd.randrange(5)
+        if kind == 0:
+            for _ in range(rnd.randrange(1, 6)):
+                data[rnd.randrange(span)] = rnd.randrange(256)
+        elif kind == 1:
+            del data[rnd.randrange(len(data)):]
+        elif kind == 2 and key[1].endswith(".safetensors"):
+            data[:8] = struct.pack("<Q", rnd.choice([0, 1, 7, 1 << 63, (1 << 64) - 1, len(data), len(data) - 8, rnd.randrange(1 << 40)]))
+        elif kind == 3:
+            at = rnd.randrange(span)
+            del data[at:at + rnd.randrange(1, 40)]
+        else:
+            digits = [i for i in range(8, span) if 48 <= data[i] <= 57]
+            at = rnd.choice(digits)
+            data[at:at + 1] = rnd.choice([b"99999999999999999999", b"-1", b"1e99", b"0.5", b""])
+        path = tmp_path / key[0] / key[1]
+        path.write_bytes(bytes(data))
+        try:
+            assert ModelWeights.stored_format(lib, tmp_path / key[0]) in (W_BF16, W_FP8, W_NVFP4)
+        except RuntimeError as e:
+            assert str(e)
+            refused += 1
+        path.write_bytes(good[key])
+    assert refused > 300
