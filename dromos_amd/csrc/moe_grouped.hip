@@ -81,18 +81,22 @@ Tables tables_at(void* ws, int P, int E) {
   return t;
 }
 
-// Inclusive scan of v over the workgroup's kMaxExperts threads (Hillis-Steele in LDS).
+// Inclusive scan of v over the workgroup's kMaxExperts threads: every wavefront scans its 64 values in registers, the
+// wavefronts' totals meet in LDS (two barriers a scan, where a scan through LDS alone took twenty).
 __device__ __forceinline__ int block_scan(int v, int* buf) {
-  const int e = threadIdx.x;
-  buf[e] = v;
-  __syncthreads();
-  for (int d = 1; d < kMaxExperts; d <<= 1) {
-    const int add = e >= d ? buf[e - d] : 0;
-    __syncthreads();
-    buf[e] += add;
-    __syncthreads();
+  const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+  int x = v;
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int y = __shfl_up(x, d);
+    if (lane >= d) x += y;
   }
-  return buf[e];
+  if (lane == kWave - 1) buf[wave] = x;
+  __syncthreads();
+  int base = 0;
+  for (int w = 0; w < wave; ++w) base += buf[w];
+  __syncthreads();
+  return x + base;
 }
 
 __global__ void __launch_bounds__(kMaxExperts) group_kernel(const int32_t* __restrict__ ids, int P, int E, Tables t) {
@@ -235,12 +239,27 @@ __global__ void __launch_bounds__(256) grouped_sum_kernel(const GroupedArgs a) {
   const int t = static_cast<int>(item / a.L), l = static_cast<int>(item % a.L);
   float o = 0.0f;
   bool first = true;
-  for (int k = 0; k < a.top_k; ++k) {
-    const int g = a.t.pos[t * a.top_k + k];
-    if (g < 0) continue;
-    const float wc = a.weights[t * a.top_k + k] * a.contrib[static_cast<int64_t>(g) * a.L + l];
-    o = first ? wc : o + wc;
-    first = false;
+  // Eight slots at a time: their positions and weights are asked for together, then their rows' elements, so a thread
+  // waits for memory twice per eight slots and not twice per slot. (A slot past top_k repeats the last and is not added.)
+  for (int k0 = 0; k0 < a.top_k; k0 += 8) {
+    int g[8];
+    float w[8], c[8];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      const int k = min(k0 + u, a.top_k - 1);
+      g[u] = a.t.pos[t * a.top_k + k];
+      w[u] = a.weights[t * a.top_k + k];
+    }
+#pragma unroll
+    for (int u = 0; u < 8; ++u) c[u] = a.contrib[static_cast<int64_t>(g[u] < 0 ? 0 : g[u]) * a.L + l];
+#pragma unroll
+    for (int u = 0; u < 8; ++u) {
+      if (k0 + u < a.top_k && g[u] >= 0) {
+        const float wc = w[u] * c[u];
+        o = first ? wc : o + wc;
+        first = false;
+      }
+    }
   }
   a.out[item] = o;
 }
