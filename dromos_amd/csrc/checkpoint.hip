@@ -561,7 +561,10 @@ class Loader {
     size_t bf16 = 0, data = 0, scale = 0;
     for (const Projection& p : list) {
       if (skip_experts_ && is_expert(p.key)) continue;
-      if (p.key != "embedding") bf16 = std::max(bf16, static_cast<size_t>(target_ == LX_W_BF16X ? p.shape.E : 1) * p.shape.N * p.shape.K * 2);
+      // Held as the file has it: uploaded to its place, nothing converted (but a quantised embedding is always
+      // dequantised once, into the gather table).
+      if (p.dst == p.src && !(p.key == "embedding" && p.src != LX_W_BF16)) continue;
+      if (p.key != "embedding") bf16 = std::max(bf16, static_cast<size_t>(p.dst == LX_W_BF16X ? p.shape.E : 1) * p.shape.N * p.shape.K * 2);
       if (p.src == LX_W_BF16) continue;
       data = std::max(data, static_cast<size_t>(p.shape.N) * data_row_bytes(p.src, p.shape.K));
       scale = std::max(scale, static_cast<size_t>(p.shape.N) * scale_row_bytes(p.src, p.shape.K));
