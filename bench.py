@@ -12,7 +12,7 @@ steps) and the graph is launched between two HIP events on its stream; W untimed
 
 Prints one JSON line. `value` is the headline case (INT8 weight-only GEMV, W 14336 x 4096, M = 1, bf16 x);
 `cases` lists every measured case (by default one per benchmark configuration: C1, C2 int8 / fp8 at M = 1, 4, 16, 64 in
-both modes, C3 M = 1, 8, C4 T = 1, 8, 32, 64, C5) with its own time, GB/s and fraction of peak. Bytes per step are the
+both modes, C3 M = 1, 8, C4 T = 1, 8, 32, 64, C5 and its four dense products) with its own time, GB/s and fraction of peak. Bytes per step are the
 algorithmic bytes: weights + scales + x + y (bench/bench_gemv.py:51-56 of the reference uses the same count).
 `floor` states what the memory system allows at these sizes, measured the same way in the same run: an empty launch,
 and a plain read of the same weight copies (lx_probe_read: the GEMV's access pattern without the product); a GEMV case
@@ -423,6 +423,9 @@ def main():
                 run_gemv(f"bf16 {N}x{K} M=1", "bf16", 1, N, K, 7000 + N)
         for T in (1, 8, 32, 64):
             run_moe(f"C4 moe bf16 T={T}", "bf16", T, 64, 2048, 1024, 8, 3000 + T)
+        for name, N, K in (("QKV", 6144, 4096), ("O", 4096, 4096), ("in_proj", 16384, 4096), ("out_proj", 4096, 8192)):
+            # The dense products of the C5 layer one by one (the layer case below runs them back to back with the experts).
+            run_gemv(f"C5 fp8 M=32 {name} {N}x{K}", "fp8", 32, N, K, 5000 + N + K, entry="gemm_w")
         run_layer()
     elif args.cases == "headline":
         run_moe("C4 moe bf16 T=1", "bf16", 1, 64, 2048, 1024, 8, 3001)
