@@ -60,6 +60,10 @@ inline int split_for_shape(int64_t K, int64_t N) {
   // batch-invariant mode, 11.4 -> 9.9 at 16, 15.1 -> 13.9 at 32; measured also at 5632 and 7168 rows, bf16 and int8).
   // NVFP4's steps are twice as long and keep the eight.
   if (S == 8 && static_cast<double>(S) > want && load_steps_for<F>(K) / S < 16 && F != LX_W_NVFP4) S = 4;
+  // Two slices where the rounding went down from 2.4 or more (906 .. 1066 tiles) leave the device short of wavefronts: four
+  // do better while a slice still holds two batches (16384 x 4096 fp8 at one / four rows in the batch-invariant mode
+  // 15.5 / 16.0 -> 13.2 / 13.8 us, bf16 28.8 / 29.3 -> 22.9 / 23.2; 20480 rows and more are better off with two).
+  if (S == 2 && want >= 2.4 && load_steps_for<F>(K) / 4 >= 16) S = 4;
   return S < by_k ? S : by_k;
 }
 
