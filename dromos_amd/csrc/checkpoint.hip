@@ -270,12 +270,17 @@ class Folder {
       if (!esize) refuse(path + ": tensor \"" + m.first + "\" has the unknown dtype " + t.dtype);
       t.stored = t.dtype == "BF16" ? Stored::kBf16 : t.dtype == "F32" ? Stored::kF32 : t.dtype == "F8_E4M3" ? Stored::kFp8
                  : t.dtype == "U8" ? Stored::kU8 : t.dtype == "I8" ? Stored::kI8 : Stored::kOther;
+      double count = 1;
       for (const Json& d : sh->items) {
-        if (d.kind != Json::kNumber || d.number < 0) refuse(path + ": tensor \"" + m.first + "\" has a bad shape");
+        // A dimension is a whole number, and the element count stays far inside what an int64 (and a double) holds exactly.
+        if (d.kind != Json::kNumber || !(d.number >= 0) || d.number > 1e15 || d.number != static_cast<double>(static_cast<int64_t>(d.number)))
+          refuse(path + ": tensor \"" + m.first + "\" has a bad shape");
+        count *= d.number;
+        if (count > 1e15) refuse(path + ": tensor \"" + m.first + "\" has a bad shape");
         t.shape.push_back(static_cast<int64_t>(d.number));
       }
       const double b = off->items[0].number, e = off->items[1].number;
-      if (b < 0 || e < b || e > static_cast<double>(room)) refuse(path + ": tensor \"" + m.first + "\" lies outside the file");
+      if (off->items[0].kind != Json::kNumber || off->items[1].kind != Json::kNumber || !(b >= 0) || !(e >= b) || e > static_cast<double>(room)) refuse(path + ": tensor \"" + m.first + "\" lies outside the file");
       t.data = base + static_cast<size_t>(b);
       t.bytes = static_cast<size_t>(e - b);
       if (t.bytes != static_cast<size_t>(t.numel()) * esize) refuse(path + ": tensor \"" + m.first + "\" has " + std::to_string(t.bytes) + " bytes, its shape says otherwise");
