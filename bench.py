@@ -307,6 +307,14 @@ def main():
             step, nbytes, keep = make_gemv_case(lx, torch, "int8", M, 14336, 4096, 1000 + M, "gemm_w")
             launches(f"C2 int8 M={M} (window_kernel)", step, nbytes, 10)
             del keep
+        os.environ["LX_BATCH_INVARIANT"] = "1"
+        step, nbytes, keep = make_gemv_case(lx, torch, "int8", 4, 14336, 4096, 1004, "gemv_w")
+        launches("C2 int8 M=4 batch-invariant (tile16_kernel)", step, nbytes, 10)
+        del keep
+        os.environ.pop("LX_BATCH_INVARIANT", None)
+        step, nbytes, keep = make_gemv_case(lx, torch, "fp8", 64, 6144, 4096, 5064, "gemm_w")
+        launches("fp8 6144x4096 M=64 (slab_kernel + slab_reduce_kernel)", step, nbytes, 10)
+        del keep
         torch.cuda.empty_cache()
         step, nbytes, keep, _ = make_moe_case(lx, torch, "bf16", 1, 64, 2048, 1024, 8, 3001, 16)
         launches("C4 moe bf16 T=1 (route + decode_gate_up + decode_down)", step, nbytes, 16)
