@@ -53,7 +53,7 @@ struct GemmArgs {
   const int8_t* xq;     // the INT8 math: quantised activations [M, K], rows K bytes apart
   const float* xscale;  // and their per-row scales
   const float* act_scale;  // BF16-math kernels on a quantised math's activation images: the rows' scales (else null)
-  void* partial;  // slab kernel with S > 1: the slices' partial tiles, [S][M][N] words (f32, or i32 for the INT8 math)
+  void* partial;  // slab kernel with S > 1: the slices' partial tiles, [S][tile][16 rows][lane] x 4 words (f32, or i32 for the INT8 math)
 };
 
 // The epilogue's operation order (engine/cpu/gemm.cpp:21-34); rf is the row factor, b the bias (0 without one).
@@ -915,21 +915,12 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
     // The tile's slice is done: the partial tile, or with one slice the result itself.
     const int nq = tile * kTileRows + 4 * g;
     if (S > 1) {
-      Acc* const out = static_cast<Acc*>(a.partial) + 0;
+      // Partial tiles lie as the wavefront holds them: [slice][tile][16 activation rows][lane] vectors of four words, so a
+      // store instruction writes 1 KB of whole cache lines (rows of the output would be 64-byte halves of lines, which
+      // the cache has to fetch first).
+      Acc* const out = static_cast<Acc*>(a.partial) + ((static_cast<int64_t>(w) * n_tiles + tile) * MT) * kWave + lane;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        const int m = mt * 16 + i;
-        if (m >= a.M) continue;
-        // Words (slice, m, n): this lane's four are consecutive.
-        uint32_t* at = reinterpret_cast<uint32_t*>(out) + (static_cast<int64_t>(w) * a.M + m) * a.N + nq;
-        if ((a.N & 3) == 0) {
-          *reinterpret_cast<Acc*>(at) = acc[mt];
-        } else {
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (nq + r < a.N) at[r] = __builtin_bit_cast(uint32_t, acc[mt][r]);
-        }
-      }
+      for (int mt = 0; mt < MT; ++mt) out[mt * kWave] = acc[mt];
     } else {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
@@ -954,39 +945,27 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
 // The slab kernel's second half for S > 1: out[m, n] from the S partial sums of (m, n), added in ascending slice order
 // from slice 0's, then the epilogue. One thread per (m, four consecutive n).
 template <int F, int MATH>
-__global__ void __launch_bounds__(256) slab_reduce_kernel(const GemmArgs a) {
+__global__ void __launch_bounds__(256) slab_reduce_kernel(const GemmArgs a, int mts) {
   constexpr bool I8 = MATH != LX_MATH_BF16;
   using Acc = typename std::conditional<MATH == LX_MATH_INT8, i32x4, f32x4>::type;
-  using Word = typename std::conditional<MATH == LX_MATH_INT8, int, float>::type;
-  const int quads = (a.N + 3) / 4;
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const int64_t vectors = static_cast<int64_t>(n_tiles) * mts * kWave;  // of one slice
   const int64_t item = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
-  if (item >= static_cast<int64_t>(a.M) * quads) return;
-  const int m = static_cast<int>(item / quads), n0 = static_cast<int>(item - static_cast<int64_t>(m) * quads) * 4;
-  const Word* p = static_cast<const Word*>(a.partial) + static_cast<int64_t>(m) * a.N + n0;
-  const int64_t slice_words = static_cast<int64_t>(a.M) * a.N;
-  Acc sum;
-  if ((a.N & 3) == 0) {
-    // Up to eight slices' words are asked for at once (a slice past the last repeats it and is not added).
-    sum = *reinterpret_cast<const Acc*>(p);
-    for (int base = 1; base < a.S; base += 8) {
-      Acc part[8];
+  if (item >= vectors) return;
+  const int lane = static_cast<int>(item & (kWave - 1)), mt = static_cast<int>((item >> 6) % mts), tile = static_cast<int>((item >> 6) / mts);
+  const int m = mt * 16 + (lane & 15), n0 = tile * kTileRows + 4 * (lane >> 4);
+  const Acc* p = static_cast<const Acc*>(a.partial) + item;
+  // Up to eight slices' vectors are asked for at once (a slice past the last repeats it and is not added).
+  Acc sum = *p;
+  for (int base = 1; base < a.S; base += 8) {
+    Acc part[8];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) part[u] = *reinterpret_cast<const Acc*>(p + min(base + u, a.S - 1) * slice_words);
+    for (int u = 0; u < 8; ++u) part[u] = p[min(base + u, a.S - 1) * vectors];
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
-        if (base + u < a.S) sum += part[u];
-    }
-  } else {
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      Word v = 0;
-      if (n0 + r < a.N) {
-        v = p[r];
-        for (int sl = 1; sl < a.S; ++sl) v += p[r + sl * slice_words];
-      }
-      sum[r] = v;
-    }
+    for (int u = 0; u < 8; ++u)
+      if (base + u < a.S) sum += part[u];
   }
+  if (m >= a.M) return;
   const bool bias_f32 = a.bias && a.bias_dtype == LX_F32;
   const float xscale = I8 ? a.xscale[m] : 1.0f;
 #pragma unroll
@@ -1065,7 +1044,8 @@ bool launch_slab(GemmArgs a, int* status, hipStream_t stream) {
       (void)hipGetLastError();
       return false;
     }
-    partial = slab_scratch(stream, sizeof(float) * static_cast<size_t>(S) * a.M * a.N, cap != hipStreamCaptureStatusNone);
+    const size_t mts = static_cast<size_t>((a.M + 15) / 16);
+    partial = slab_scratch(stream, sizeof(float) * 4 * kWave * mts * n_tiles * S, cap != hipStreamCaptureStatusNone);
     if (!partial) return false;
   }
   a.partial = partial;
@@ -1095,8 +1075,9 @@ bool launch_slab(GemmArgs a, int* status, hipStream_t stream) {
     default: st = with_mt(std::integral_constant<int, 4>{}); break;
   }
   if (!st && S > 1) {
-    const int64_t items = static_cast<int64_t>(a.M) * ((a.N + 3) / 4);
-    hipLaunchKernelGGL((slab_reduce_kernel<F, MATH>), dim3(static_cast<unsigned>((items + 255) / 256)), dim3(256), 0, stream, a);
+    const int mts = (a.M + 15) / 16;
+    const int64_t items = static_cast<int64_t>(n_tiles) * mts * kWave;
+    hipLaunchKernelGGL((slab_reduce_kernel<F, MATH>), dim3(static_cast<unsigned>((items + 255) / 256)), dim3(256), 0, stream, a, mts);
     st = status_of(hipGetLastError());
   }
   *status = st;
