@@ -1007,10 +1007,10 @@ void* slab_scratch(hipStream_t stream, size_t bytes, bool capturing) {
 
 // Where the slab kernel is tried before the windowed one. Measured on MI355X (fp8, int8 and bf16 weights, bf16
 // activations): it wins where the windowed kernel's workgroups, which each stage all of K, are few or long: more than 32
-// rows with at most 400 tiles (6144 x 4096 at 48 rows: 29 -> 21 us, at 64: 37 -> 24 us), and more than 16 rows with
-// K >= 8192 and few tiles (4096 x 8192 at 32 rows: 21 -> 17 us, at 64: 35 -> 24 us). With many tiles (14336 x 4096) its
-// second pass over the partial tiles costs more than the windows do. LX_SLAB_MIN_ROWS (a tuning knob) overrides: rows
-// from which it is tried.
+// rows with at most 400 tiles (6144 x 4096 at 48 rows: 22.7 -> 18.7 us, at 64: 26.2 -> 22.4 us; 4096 x 4096 at 64:
+// 21.5 -> 17.6 us), and more than 16 rows with K >= 8192 and few tiles (4096 x 8192 at 32 rows: 21.3 -> 15.3 us, at 64:
+// 35.7 -> 22.7 us). With many tiles (14336 x 4096) its second pass over the partial tiles costs more than the windows do.
+// LX_SLAB_MIN_ROWS (a tuning knob) overrides: rows from which it is tried.
 inline bool slab_wanted(int M, int n_tiles, int64_t K) {
   if (const char* e = getenv("LX_SLAB_MIN_ROWS")) return M >= atoi(e);
   return n_tiles <= 400 && (M > 32 || (M > 16 && K >= 8192));
