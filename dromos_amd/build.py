@@ -14,7 +14,7 @@ ROOT = Path(__file__).resolve().parent.parent
 CSRC = ROOT / "dromos_amd" / "csrc"
 LIB_DIR = ROOT / "dromos_amd" / "lib"
 HIP_LIB = LIB_DIR / "libdromos_hip.so"
-SOURCES = ["runtime.hip", "quant.hip", "gemv.hip", "gemv_bf16.hip", "gemv_int8.hip", "gemv_fp8.hip", "gemv_nvfp4.hip", "gemv_bf16x.hip", "bf16x.hip", "gemm.hip",
+SOURCES = ["runtime.hip", "quant.hip", "gemv.hip", "gemv_bf16.hip", "gemv_int8.hip", "gemv_fp8.hip", "gemv_nvfp4.hip", "gemv_bf16x.hip", "bf16x.hip", "gemm.hip", "gemm_walk_bf16.hip", "gemm_walk_int8.hip", "gemm_walk_fp8.hip", "gemm_walk_nvfp4.hip",
            "moe.hip", "moe_grouped.hip", "router.hip", "checkpoint.hip"]
 
 # -ffp-contract=off: the epilogues and the ordered sums are written as separate multiplies and adds, as the

@@ -15,6 +15,7 @@
 #include <utility>
 
 #include "common.h"
+#include "gemm_args.h"
 #include "tile_mfma.h"
 
 namespace dro {
@@ -23,52 +24,6 @@ int gemv_any(const void* x, int x_dtype, int ld_x, const lx_weight& w, const voi
              int y_dtype, int ld_y, int M, int N, int K, float alpha, float beta, void* stream);
 
 namespace {
-
-constexpr size_t kLdsMax = 160 * 1024;  // LDS a workgroup may take
-
-struct XRows {
-  const void* x;
-  int dtype;
-  int64_t ld;  // elements between rows
-};
-
-struct GemmArgs {
-  XRows xs;
-  const uint8_t* w;
-  const uint8_t* scale;
-  float global;
-  const void* bias;
-  int bias_dtype;
-  void* y;
-  int y_dtype;
-  int64_t ld_y;
-  int M, N, K;
-  float alpha, beta;
-  int chunks, steps, steps_per_wave, S;
-  int64_t row_bytes, scale_row_bytes;
-  int tiles_per_wg, x_vecs, x_row_vecs, x_pitch, x_iters;  // the LDS activation image (XL and panel kernels)
-  int x_phased;  // lean kernel with two slices a wavefront: the image holds half of K at a time
-  int win;       // windowed kernel: load steps of every slice the image holds at a time (2, 4 or 8)
-  int win_steps_shift, win_shift, row_shift;  // log2 of win, of the 16-byte pieces in a window, and in an image row
-  const int8_t* xq;     // the INT8 math: quantised activations [M, K], rows K bytes apart
-  const float* xscale;  // and their per-row scales
-  const float* act_scale;  // BF16-math kernels on a quantised math's activation images: the rows' scales (else null)
-  void* partial;  // slab kernel with S > 1: the slices' partial tiles, [S][tile][16 rows][lane] x 4 words (f32, or i32 for the INT8 math)
-};
-
-// The epilogue's operation order (engine/cpu/gemm.cpp:21-34); rf is the row factor, b the bias (0 without one).
-__device__ __forceinline__ void write_out(const GemmArgs& a, int m, int n, float sum, float rf, float b) {
-  float t = (a.act_scale ? rf * a.act_scale[m] : rf) * sum;
-  if (a.bias) t += b;
-  float v = a.alpha * t;
-  const int64_t at = m * a.ld_y + n;
-  if (a.beta != 0.0f) v = a.beta * load_as_f32(a.y, a.y_dtype, at) + v;
-  store_from_f32(a.y, a.y_dtype, at, v);
-}
-
-__device__ __forceinline__ void write_out(const GemmArgs& a, int wtype, int m, int n, float sum) {
-  write_out(a, m, n, sum, row_factor(wtype, a.scale, a.global, n), a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f);
-}
 
 // XL: the activation rows (at most 16, MT == 1) are staged once per workgroup into LDS as bf16, behind the
 // wavefronts' regions: rows of x_row_vecs * 8 values (K rounded up to whole weight batches, zero from K on),
@@ -1338,10 +1293,41 @@ int launch_skinny_x(const GemmArgs& a, size_t lds, unsigned grid, unsigned threa
   return status_of(hipGetLastError());
 }
 
+// The walk kernel (gemm_walk.h) where it is the faster family. Measured on MI355X (bf16 activations, 9 .. 64 rows): it
+// wins where a wavefront's walk is at most 16 groups of four load steps (K = 4096 of one-byte weights) and the matrix
+// has the tiles to give most compute units a workgroup: 14336 x 4096 int8 at 16 / 32 / 64 rows 16.0 / 20.7 / 29.9 ->
+// 15.2 / 18.1 / 25.4 us, 16384 x 4096 fp8 at 32 rows 21.5 -> 17.5 us, 6144 x 4096 14.2 -> 12.7 us, 4096 x 4096
+// 13.6 -> 12.7 us; on 4096 x 8192 (32 groups) and at 8 rows and fewer the tile kernels are faster. The variant table
+// ("gemm_w_<format>": 0 = the tile kernels, 1 .. 3 = walk with 1, 2, 4 tiles a workgroup) overrides; no variant changes
+// a sum.
+template <int F>
+bool try_walk(const GemmArgs& a, int* status, hipStream_t stream) {
+  if (a.xs.dtype != LX_BF16) return false;
+  static const char* const kKey = F == LX_W_BF16 ? "gemm_w_bf16" : F == LX_W_INT8 ? "gemm_w_int8" : F == LX_W_FP8 ? "gemm_w_fp8" : "gemm_w_nvfp4";
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const int tuned = tuned_variant(kKey, a.M, a.N, a.K);
+  int W;
+  if (tuned == 0) return false;
+  if (tuned >= 1 && tuned <= 3) {
+    W = 1 << (tuned - 1);
+  } else {
+    if (a.M <= 8 || a.steps > 64 || n_tiles < 192) return false;
+    W = n_tiles >= 512 ? 4 : 2;
+  }
+  if constexpr (F == LX_W_BF16) return launch_walk_bf16(a, W, status, stream);
+  else if constexpr (F == LX_W_INT8) return launch_walk_int8(a, W, status, stream);
+  else if constexpr (F == LX_W_FP8) return launch_walk_fp8(a, W, status, stream);
+  else return launch_walk_nvfp4(a, W, status, stream);
+}
+
 template <int F, int MT>
 int launch_skinny(GemmArgs a, hipStream_t stream) {
   const int S = a.S;
   const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
+  {
+    int st = kOk;
+    if (try_walk<F>(a, &st, stream)) return st;
+  }
   // More than eight rows: the windowed kernel (for 9 .. 16 rows where the matrix has the tiles to fill its
   // sixteen-wavefront workgroups; the lean kernel's image of all of K leaves too few of them resident there).
   if (MT > 1 || (a.M > 8 && n_tiles >= 320)) {

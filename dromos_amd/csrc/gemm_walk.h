@@ -1,0 +1,312 @@
+// The walk kernel (a template on the weight format; one source per format instantiates it): the matrix-core product for up to 64 bf16 activation rows (BF16 math) in which a wavefront walks
+// along a tile's rows instead of taking one short piece of them.
+//
+// The arithmetic is the tile kernels' (tile_mfma.h): a tile is 16 weight rows; K is cut into S contiguous slices of
+// steps_per_wave load steps; a slice's products are one ascending chain of v_mfma_f32_16x16x32_bf16 from zero, the S
+// partial tiles are added in ascending slice order, then the epilogue. S depends on (format, K, N) only, so a row's
+// bits are those of every other kernel of the library, whatever M is (engine/cuda/kernels.h:453-477).
+//
+// A wavefront takes all S slices of its tile one after the other and keeps their sums apart (in an LDS area of its own)
+// until the end, where it adds them in ascending order: no two wavefronts ever exchange partial tiles. The W
+// wavefronts of a workgroup (W tiles) are at the same k at the same time, so the activation image is one window of
+// four load steps, twice, whatever K, M and S are. Workgroup b starts with slice b % S and goes round: weight rows are
+// a power of two apart, and a device whose wavefronts all read the same offset of their rows at the same moment keeps
+// hitting the same few memory channels (measured: a plain read in that pattern takes 11.4 us where 9.8 us is possible).
+// What keeps the memory busy is depth: a wavefront always has four groups of four load steps (16 KB) on their way,
+// asked for one group at a time as the oldest is used, so the device's requests are paced instead of arriving all at
+// once, and the activations are asked for two windows ahead, just before the weights of the same distance (loads come
+// back in the order they were asked for). One barrier per window.
+//
+// Inside an image a 16-byte piece of k of the 16 rows of an activation tile is one 256-byte block, the rows rotated by
+// four slots per piece, so that the fragment reads (16 rows of one piece) and the staging writes (4 rows x 4 pieces per
+// 16 lanes) touch every bank once. The weights arrive in memory order (256 contiguous bytes of each of four rows per
+// instruction) and pass through a 4 KB image of the wavefront's own (chunk c of row r at slot c ^ r) into fragment order.
+#pragma once
+
+#include <type_traits>
+
+#include "common.h"
+#include "gemm_args.h"
+#include "tile_mfma.h"
+
+namespace dro {
+namespace walk {
+
+template <int N>
+using Tag = std::integral_constant<int, N>;
+
+template <int F, int MT, int W>
+__global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
+  extern __shared__ __align__(16) f32x4 lds4[];
+  constexpr int E = Fmt<F>::kElems, J = E / 8;
+  constexpr int PB = 4 * J;          // 16-byte pieces of an image row under one load step
+  constexpr int Q = MT * 4 * J / W;  // staging pieces a lane holds per window
+  static_assert(Q * W == MT * 4 * J && Q >= 1, "the wavefronts share a window's pieces evenly");
+  constexpr int kImage = MT * 4 * PB * 256;  // one window
+  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
+  const int tw = wave;  // tile of the workgroup
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const int tile = blockIdx.x * W + tw;
+  const int n0 = min(tile, n_tiles - 1) * kTileRows, valid = min(kTileRows, a.N - n0);  // a tile past the last repeats it
+  const int g = lane >> 4, i = lane & 15;
+  uint8_t* const lds = reinterpret_cast<uint8_t*>(lds4);
+  uint8_t* const stage = lds + wave * 4096;
+  uint8_t* const img = lds + W * 4096;  // + buffer * kImage
+  const int groups = a.steps >> 2, last = groups - 1;  // groups of four load steps in a row
+  const int gps = a.steps_per_wave >> 2;               // groups of a slice
+  const int first_slice = blockIdx.x % a.S, rot = first_slice * gps;
+  // The l-th group this workgroup takes (l past the end repeats the last one).
+  auto group_of = [&](int l) {
+    const int gq = min(l, last) + rot;
+    return gq >= groups ? gq - groups : gq;
+  };
+
+  // Staging: item idx = (tile of rows * 4 + step of the window) * J + quad of pieces; wavefront tw takes
+  // items tw, tw + W, ... A lane's piece of an item: row 4 (lane / 16) + (lane % 16) / 4, piece lane % 4 of the quad.
+  const int r = 4 * g + (i >> 2), e3 = i & 3;
+  const uint32_t lds_lane = e3 * 256 + ((r + 4 * e3) & 15) * 16;
+  const char* const xbase = static_cast<const char*>(a.xs.x);
+  const uint32_t ld_bytes = static_cast<uint32_t>(a.xs.ld) * 2u;
+  uint32_t x_off[Q];  // byte offset of this lane's piece of item `it` within window 0
+#pragma unroll
+  for (int it = 0; it < Q; ++it) {
+    const int idx = tw + it * W;
+    const int pq = idx & (J - 1), u = (idx / J) & 3, mt = idx / (4 * J);
+    x_off[it] = static_cast<uint32_t>(min(16 * mt + r, a.M - 1)) * ld_bytes + static_cast<uint32_t>(u * 4 * E + pq * 32 + e3 * 8) * 2u;
+  }
+  u32x4 xr[2][Q];  // two windows on their way
+  auto stage_load = [&](auto set, int gamma) {
+    const char* const src = xbase + static_cast<uint32_t>(group_of(gamma)) * (16u * E * 2u);  // a window is 16 E values of k
+#pragma unroll
+    for (int it = 0; it < Q; ++it) xr[decltype(set)::value][it] = *reinterpret_cast<const u32x4*>(src + x_off[it]);
+  };
+  auto stage_store = [&](auto set, int gamma) {
+    uint8_t* const dst = img + (gamma & 1) * kImage + tw * 1024 + lds_lane;
+#pragma unroll
+    for (int it = 0; it < Q; ++it) *reinterpret_cast<u32x4*>(dst + it * (W * 1024)) = xr[decltype(set)::value][it];
+  };
+
+  // This lane's weight loads: rows 4 q + g of the tile, chunk i of a group (256 contiguous bytes per 16 lanes).
+  const uint8_t* const tile_w = a.w + static_cast<int64_t>(n0) * a.row_bytes;
+  const uint8_t* const own_scale = a.scale + (static_cast<int64_t>(n0) + min(i, valid - 1)) * a.scale_row_bytes;  // NVFP4 only
+  uint32_t row_off[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) row_off[q] = static_cast<uint32_t>(min(4 * q + g, valid - 1)) * static_cast<uint32_t>(a.row_bytes) + i * 16u;
+  u32x4 raw[4][4];
+  uint32_t sc[4][4];
+  auto issue_group = [&](auto slot, int gamma) {
+    constexpr int SL = decltype(slot)::value;
+    const int gq = group_of(gamma);
+    const uint32_t c = static_cast<uint32_t>(gq) * 256u;  // a group is 256 bytes of a row
+#pragma unroll
+    for (int q = 0; q < 4; ++q) raw[SL][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tile_w + (row_off[q] + c)));
+    if constexpr (F == LX_W_NVFP4) {
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        sc[SL][u] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale) + (16 * gq + 4 * u + g));
+    }
+  };
+  // Row 4 q + g, chunk i goes into the wavefront's image; row i, chunk 4 s + g comes out.
+  uint32_t put_at[4], get_at[4];
+#pragma unroll
+  for (int q = 0; q < 4; ++q) {
+    put_at[q] = (4 * q + g) * 256 + ((i ^ (4 * q + g)) & 15) * 16;
+    get_at[q] = i * 256 + (((4 * q + g) ^ i) & 15) * 16;
+  }
+  u32x4 wv[4];
+  uint32_t wsc[4];
+  auto to_image = [&](auto slot) {
+    constexpr int SL = decltype(slot)::value;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) *reinterpret_cast<u32x4*>(stage + put_at[q]) = raw[SL][q];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) wsc[u] = F == LX_W_NVFP4 ? sc[SL][u] : 0u;
+  };
+
+  // The activations first, then the weights: what is asked for first comes back first.
+  stage_load(Tag<0>{}, 0);
+  stage_load(Tag<1>{}, 1);
+  issue_group(Tag<0>{}, 0);
+  issue_group(Tag<1>{}, 1);
+  issue_group(Tag<2>{}, 2);
+  issue_group(Tag<3>{}, 3);
+  stage_store(Tag<0>{}, 0);
+  stage_load(Tag<0>{}, 2);
+  to_image(Tag<0>{});
+  uint32_t scales[4];
+#pragma unroll
+  for (int u = 0; u < 4; ++u) scales[u] = wsc[u];
+  // (A wavefront's LDS instructions run in the order they were issued: the reads see the writes before them.)
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int s = 0; s < 4; ++s) wv[s] = *reinterpret_cast<const u32x4*>(stage + get_at[s]);
+  asm volatile("" ::: "memory");
+  issue_group(Tag<0>{}, 4);
+
+  // A fragment read: piece g * J + j of the step, this lane's row i of the activation tile.
+  uint32_t rd_lane[J];
+#pragma unroll
+  for (int j = 0; j < J; ++j) rd_lane[j] = (g * J + j) * 256 + ((i + 4 * ((g * J + j) & 3)) & 15) * 16;
+
+  // The slice at hand; a finished slice's sum waits in the wavefront's own area behind the images.
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+  f32x4* const sums = reinterpret_cast<f32x4*>(img + 2 * kImage) + wave * (a.S * MT * kWave) + lane;  // [slice][mt][lane]
+  int slice_end = gps, slice = first_slice;
+
+  // The gamma-th group the workgroup takes (its fragments are in wv).
+  auto one_group = [&](auto phase, int gamma) {
+    constexpr int P = decltype(phase)::value;  // gamma % 4
+    __syncthreads();  // every wavefront has left window gamma - 1, and window gamma is complete
+    const uint8_t* const xb = img + (P & 1) * kImage;
+    // The products of the group, pair by pair (a pair = load step s, matrix instruction j of the step). A pair's
+    // activation fragments are asked for two pairs ahead, the next pair's weights are expanded under this pair's matrix
+    // instructions, and the group's chores (the next window into the other image, the next group through the
+    // wavefront's image, their loads) are spread over the pairs. The scheduler is held to this order: left alone it
+    // asks for data right before its use.
+    constexpr int kPairs = 4 * J, kAhead = 2;
+    bf16x8 b[kAhead + 1][MT];
+    auto read_pair = [&](int p, bf16x8 (&dst)[MT]) {
+      const int s = p / J, j = p % J;
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) dst[mt] = *reinterpret_cast<const bf16x8*>(xb + (mt * 4 + s) * (PB * 256) + rd_lane[j]);
+    };
+#pragma unroll
+    for (int p = 0; p < kAhead; ++p) read_pair(p, b[p]);
+    bf16x8 wf = weight_fragment<F>(wv[0], scales[0], 0);
+    u32x4 wv_next[4];
+#pragma unroll
+    for (int p = 0; p < kPairs; ++p) {
+      if (p + kAhead < kPairs) read_pair(p + kAhead, b[(p + kAhead) % (kAhead + 1)]);
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, b[p % (kAhead + 1)][mt], acc[mt], 0, 0, 0);
+      if (p + 1 < kPairs) wf = weight_fragment<F>(wv[(p + 1) / J], scales[(p + 1) / J], (p + 1) % J);
+      if (p == 0) {
+        // The next window goes into the other image, the window after the next is asked for.
+        stage_store(Tag<(P + 1) & 1>{}, gamma + 1);
+        stage_load(Tag<(P + 1) & 1>{}, gamma + 3);
+      }
+      if (p == 1) {
+        // The next group goes into the wavefront's image; its registers take the group four ahead of it.
+        to_image(Tag<(P + 1) & 3>{});
+        issue_group(Tag<(P + 1) & 3>{}, gamma + 5);
+      }
+      if (p == kPairs - 1) {
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int s = 0; s < 4; ++s) wv_next[s] = *reinterpret_cast<const u32x4*>(stage + get_at[s]);
+        asm volatile("" ::: "memory");
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      scales[u] = wsc[u];
+      wv[u] = wv_next[u];
+    }
+    // A slice ends.
+    if (gamma + 1 == slice_end) {
+#pragma unroll
+      for (int mt = 0; mt < MT; ++mt) {
+        sums[(slice * MT + mt) * kWave] = acc[mt];
+        acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
+      }
+      slice_end += gps;
+      slice = slice + 1 == a.S ? 0 : slice + 1;
+    }
+  };
+  for (int gamma = 0; gamma < groups; gamma += 4) {
+    one_group(Tag<0>{}, gamma);
+    one_group(Tag<1>{}, gamma + 1);
+    one_group(Tag<2>{}, gamma + 2);
+    one_group(Tag<3>{}, gamma + 3);
+  }
+
+  // The slices' sums in ascending order (the wavefront reads what it wrote itself: LDS keeps its order).
+  asm volatile("" ::: "memory");
+  f32x4 total[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    total[mt] = sums[mt * kWave];
+    for (int sl = 1; sl < a.S; ++sl) total[mt] += sums[(sl * MT + mt) * kWave];
+  }
+
+  if (tile >= n_tiles) return;
+  // A lane holds four consecutive outputs of one activation row: one 16-byte store where y allows it.
+  const int nq = n0 + 4 * g;
+  const bool wide = a.y_dtype == LX_F32 && a.beta == 0.0f && nq + 3 < a.N && (a.ld_y & 3) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15) == 0;
+  float rf[4], bs[4];
+#pragma unroll
+  for (int rr = 0; rr < 4; ++rr) {
+    const int n = min(nq + rr, a.N - 1);
+    rf[rr] = row_factor(F, a.scale, a.global, n);
+    bs[rr] = a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f;
+  }
+#pragma unroll
+  for (int mt = 0; mt < MT; ++mt) {
+    const int m = mt * 16 + i;
+    if (m >= a.M) continue;
+    if (wide) {
+      const float xs = a.act_scale ? a.act_scale[m] : 1.0f;
+      f32x4 out;
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr) {
+        float t = (a.act_scale ? rf[rr] * xs : rf[rr]) * total[mt][rr];
+        if (a.bias) t += bs[rr];
+        out[rr] = a.alpha * t;
+      }
+      *reinterpret_cast<f32x4*>(static_cast<float*>(a.y) + static_cast<int64_t>(m) * a.ld_y + nq) = out;
+    } else {
+#pragma unroll
+      for (int rr = 0; rr < 4; ++rr)
+        if (nq + rr < a.N) write_out(a, m, nq + rr, total[mt][rr], rf[rr], bs[rr]);
+    }
+  }
+}
+
+template <int F, int W>
+int launch_w(const GemmArgs& a, unsigned grid, hipStream_t stream) {
+  constexpr int J = Fmt<F>::kElems / 8, PB = 4 * J;
+  const int MT = (a.M + 15) / 16;
+  const size_t lds = static_cast<size_t>(W) * 4096 + 2 * static_cast<size_t>(MT) * 4 * PB * 256 + static_cast<size_t>(W) * a.S * MT * kWave * 16;
+  if (lds > kLdsMax) return kNotSupported;
+  auto launch = [&](auto kernel) {
+    if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), kLdsMax);
+    hipLaunchKernelGGL(kernel, dim3(grid), dim3(W * kWave), lds, stream, a);
+    return status_of(hipGetLastError());
+  };
+  switch (MT) {
+    case 1: return launch(walk_kernel<F, 1, W>);
+    case 2: return launch(walk_kernel<F, 2, W>);
+    case 3: return launch(walk_kernel<F, 3, W>);
+    default: return launch(walk_kernel<F, 4, W>);
+  }
+}
+
+template <int F>
+bool launch_format(const GemmArgs& a, int W, int* status, hipStream_t stream) {
+  constexpr int E = Fmt<F>::kElems;
+  const int S = a.S, spw = a.steps_per_wave;
+  if (a.M < 1 || a.M > 64 || S < 1 || spw % 8 != 0) return false;
+  // Whole slices, and groups in fours.
+  if (S * spw != a.steps || static_cast<int64_t>(a.steps) * 4 * E != a.K || a.steps % 16 != 0) return false;
+  if (static_cast<int64_t>(a.M) * a.xs.ld * 2 + static_cast<int64_t>(a.K) * 2 >= (int64_t{1} << 31)) return false;
+  if (static_cast<int64_t>(kTileRows) * a.row_bytes >= (int64_t{1} << 31)) return false;
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
+  const unsigned grid = static_cast<unsigned>((n_tiles + W - 1) / W);
+  int st;
+  switch (W) {
+    case 4: st = launch_w<F, 4>(a, grid, stream); break;
+    case 2: st = launch_w<F, 2>(a, grid, stream); break;
+    case 1: st = launch_w<F, 1>(a, grid, stream); break;
+    default: return false;
+  }
+  if (st == kNotSupported) return false;
+  *status = st;
+  return true;
+}
+
+}  // namespace walk
+}  // namespace dro

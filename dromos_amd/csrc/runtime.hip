@@ -73,13 +73,19 @@ struct Registered {
   int gemv_format;  // the lx_wtype whose order class admits a variant, or -1 for no rule
 };
 
-// The kernels with variants. The GEMV of each format has three: its K split of 1, 2 or 4 wavefronts.
+// The kernels with variants. The GEMV of each format has three: its K split of 1, 2 or 4 wavefronts (admitted where the
+// split is the shape's order class). The matrix-core product of each format (9 .. 64 activation rows) has four: the tile
+// kernels, or the walk kernel with 1, 2 or 4 tiles a workgroup; none changes a sum, so all are admitted.
 const std::map<std::string, Registered>& registry() {
   static const auto* r = new std::map<std::string, Registered>{
       {"gemv_w_bf16", {{"s1", "s2", "s4"}, LX_W_BF16}},
       {"gemv_w_int8", {{"s1", "s2", "s4"}, LX_W_INT8}},
       {"gemv_w_fp8", {{"s1", "s2", "s4"}, LX_W_FP8}},
       {"gemv_w_nvfp4", {{"s1", "s2", "s4"}, LX_W_NVFP4}},
+      {"gemm_w_bf16", {{"tiles", "walk1", "walk2", "walk4"}, -1}},
+      {"gemm_w_int8", {{"tiles", "walk1", "walk2", "walk4"}, -1}},
+      {"gemm_w_fp8", {{"tiles", "walk1", "walk2", "walk4"}, -1}},
+      {"gemm_w_nvfp4", {{"tiles", "walk1", "walk2", "walk4"}, -1}},
   };
   return *r;
 }

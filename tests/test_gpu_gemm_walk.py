@@ -1,0 +1,117 @@
+"""GPU parity: the walk kernel of lx_gemm_w / lx_gemm_skinny (9 .. 64 bf16 activation rows, a wavefront walking a whole
+tile) against float64 on the decoded values, and bit for bit against the tile kernels it replaces on the shapes it
+takes: the variant table forces each family ("gemm_w_<format>": 0 = tiles, 1 .. 3 = walk with 1, 2, 4 tiles a
+workgroup), and no variant may change an output bit, a row's bits may not depend on the batch."""
+
+import pytest
+import torch
+
+import checks
+import ops
+from dromos_amd.abi import FORMATS, MATH_BF16, MATH_FP8
+from dromos_amd.formats import random_weight
+
+pytestmark = pytest.mark.gpu
+FMT = checks.FMT_NAMES
+# K whose rows are whole slices of whole four-group walks in the format (the shapes the kernel takes), N with a ragged last tile
+SHAPES = {"bf16": [(150, 512), (4096, 1024)], "int8": [(150, 1024), (4096, 2048)], "fp8": [(150, 1024), (4096, 4096)], "nvfp4": [(150, 2048), (4096, 4096)]}
+
+
+def force(hip, fmt, M, N, K, variant):
+    hip.lib.lx_tune_clear()
+    if variant is not None:
+        assert hip.lib.lx_tune_force(f"gemm_w_{fmt}".encode(), M, N, K, variant) == 0
+
+
+@pytest.fixture(autouse=True)
+def clear_table(hip):
+    yield
+    hip.lib.lx_tune_clear()
+
+
+def test_variants_are_registered(hip):
+    import ctypes
+
+    hip.lib.lx_tune_variant_name.restype = ctypes.c_char_p
+    for fmt in FMT:
+        key = f"gemm_w_{fmt}".encode()
+        assert hip.lib.lx_tune_variants(key) == 4
+        assert [hip.lib.lx_tune_variant_name(key, v).decode() for v in range(4)] == ["tiles", "walk1", "walk2", "walk4"]
+        assert all(hip.lib.lx_tune_set(key, 32, 4096, 4096, v) == 0 for v in range(4))  # none changes a sum: all admitted
+        assert hip.lib.lx_tune_set(key, 32, 4096, 4096, 4) == 803
+
+
+@pytest.mark.parametrize("M", [9, 16, 17, 33, 48, 64])
+@pytest.mark.parametrize("fmt", FMT)
+def test_every_variant_gives_the_same_bits(hip, fmt, M):
+    for N, K in SHAPES[fmt]:
+        g = torch.Generator().manual_seed(M + N)
+        w = random_weight(FORMATS[fmt], N, K, N + K)
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        bias = torch.randn(N, generator=g)
+        want = ops.gemv_reference(x, w.dense(), bias, 1.0, 0.0, None)
+        wd, xd, bd = w.to("cuda"), x.cuda(), bias.cuda()
+        outs = {}
+        for variant in (0, 1, 2, 3, None):
+            force(hip, fmt, M, N, K, variant)
+            y = torch.full((M, N), float("nan"), device="cuda")
+            outs[variant] = ops.gemm_w(hip, xd, wd, MATH_BF16, bias=bd, y=y).clone()
+        checks.check_product(outs[0].cpu(), want)
+        for variant, out in outs.items():
+            assert torch.equal(out.view(torch.int32), outs[0].view(torch.int32)), f"variant {variant} changes bits at {fmt} {N}x{K} M={M}"
+
+
+@pytest.mark.parametrize("fmt", FMT)
+def test_walk_rows_do_not_depend_on_the_batch(hip, fmt):
+    N, K = SHAPES[fmt][1]
+    w = random_weight(FORMATS[fmt], N, K, 3).to("cuda")
+    g = torch.Generator().manual_seed(8)
+    x = torch.randn(64, K, generator=g).to(torch.bfloat16).cuda()
+    force(hip, fmt, 64, N, K, 3)
+    full = ops.gemm_skinny(hip, x, w)
+    for M in (1, 8, 9, 16, 31, 40):
+        for variant in (2, 3):
+            force(hip, fmt, M, N, K, variant)
+            part = ops.gemm_skinny(hip, x[:M].contiguous(), w)
+            assert torch.equal(part, full[:M]), f"rows of an M={M} call (variant {variant}) differ from the rows of the M=64 call"
+
+
+@pytest.mark.parametrize("alpha,beta", [(1.0, 0.0), (-1.5, 1.0)])
+@pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("bias_dtype", [None, torch.bfloat16])
+@pytest.mark.parametrize("fmt", FMT)
+def test_walk_epilogue_matrix(hip, fmt, bias_dtype, y_dtype, alpha, beta):
+    # Both epilogue forms (the 16-byte store, the element-wise one), strided x and y, nothing written past N.
+    N, K = SHAPES[fmt][0]
+    M, pad = 20, 8
+    g = torch.Generator().manual_seed(5)
+    w = random_weight(FORMATS[fmt], N, K, 6)
+    xb = torch.randn(M, K + pad, generator=g).to(torch.bfloat16)
+    bias = None if bias_dtype is None else torch.randn(N, generator=g).to(bias_dtype)
+    y0 = torch.randn(M, N + pad, generator=g).to(y_dtype)
+    want = ops.gemv_reference(xb[:, :K], w.dense(), bias, alpha, beta, y0[:, :N])
+    for variant in (0, 3):
+        force(hip, fmt, M, N, K, variant)
+        y = y0.clone().cuda()
+        ops.gemm_w(hip, xb.cuda(), w.to("cuda"), MATH_BF16, bias=None if bias is None else bias.cuda(), y=y, alpha=alpha, beta=beta,
+                   ld_x=K + pad, ld_y=N + pad, N=N)
+        checks.check_product(y.cpu()[:, :N], want)
+        assert torch.equal(y.cpu()[:, N:], y0[:, N:]), "wrote past the N columns of y"
+        if variant == 0:
+            first = y.clone()
+        else:
+            assert torch.equal(y.view(torch.int16 if y_dtype == torch.bfloat16 else torch.int32),
+                               first.view(torch.int16 if y_dtype == torch.bfloat16 else torch.int32))
+
+
+def test_walk_under_a_quantised_math(hip):
+    # The FP8 math on NVFP4 weights runs the BF16-math kernels on the activations' images with the rows' scales in the
+    # epilogue: the walk kernel and the tile kernels agree there too.
+    N, K, M = 4096, 4096, 32
+    w = random_weight(FORMATS["nvfp4"], N, K, 4).to("cuda")
+    x = torch.randn(M, K, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).cuda()
+    outs = []
+    for variant in (0, 3):
+        force(hip, "nvfp4", M, N, K, variant)
+        outs.append(ops.gemm_w(hip, x, w, MATH_FP8).clone())
+    assert torch.equal(outs[0].view(torch.int32), outs[1].view(torch.int32))
