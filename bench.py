@@ -45,6 +45,7 @@ class Timer:
     def __init__(self, lx, torch):
         self.lx, self.torch = lx, torch
         self.stream = torch.cuda.Stream()
+        lx.reserve_stream(self.stream.cuda_stream)  # what lx_rt_stream_create gives the engine's own streams
         lib = lx.lib
         self.ev = []
         for _ in range(2):
@@ -131,9 +132,7 @@ def make_bf16x_case(lx, torch, M, N, K, seed):
     g = torch.Generator(device="cpu").manual_seed(seed)
     master = master_weight(N, K, g).cuda()
     x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
-    size = lx.lib.lx_bf16x_bytes
-    size.restype = ctypes.c_int64
-    n = int(size(ctypes.c_void_p(master.data_ptr()), ctypes.c_int64(N), ctypes.c_int(K), lx.stream))
+    n = int(lx.status("bf16x_bytes", master, N, K))
     enc = torch.empty(n, dtype=torch.uint8, device="cuda")
     assert lx.status("bf16x_encode", master, ctypes.c_int64(N), K, enc, ctypes.c_int64(n)) == 0
     torch.cuda.synchronize()

@@ -935,29 +935,41 @@ __global__ void __launch_bounds__(256) slab_reduce_kernel(const GemmArgs a, int 
 }
 
 // The slab kernel's partial tiles live in a buffer the library keeps per (device, stream): calls on one stream run one
-// after the other, so they can share it, and a call that is being captured into a graph can use it where it could not
-// ask for memory. It is made by the first call on the stream that needs one (never during a capture: that call takes the
-// windowed kernel instead) and kept until the process ends.
+// after the other, so they can share it. A product never makes one (it neither allocates nor synchronises, and does the
+// same under graph capture as outside): the buffer is made when the stream is (lx_rt_stream_create), or when a host
+// that brings its own streams reserves one (lx_rt_stream_reserve), and a call on a stream without one takes the windowed
+// kernel.
 constexpr size_t kSlabScratchBytes = 64u << 20;
 
-void* slab_scratch(hipStream_t stream, size_t bytes, bool capturing) {
+struct SlabBuffers {
+  std::mutex lock;
+  std::map<std::pair<int, hipStream_t>, void*> of;
+};
+SlabBuffers& slab_buffers() {
+  static auto* b = new SlabBuffers;
+  return *b;
+}
+
+void* slab_scratch(hipStream_t stream, size_t bytes) {
   if (bytes > kSlabScratchBytes) return nullptr;
-  static std::mutex lock;
-  static std::map<std::pair<int, hipStream_t>, void*> buffers;
   int dev = 0;
   if (hipGetDevice(&dev) != hipSuccess) {
     (void)hipGetLastError();
     return nullptr;
   }
-  std::lock_guard<std::mutex> g(lock);
-  void*& slot = buffers[{dev, stream}];
-  if (!slot && !capturing) {
-    if (hipMalloc(&slot, kSlabScratchBytes) != hipSuccess) {
-      (void)hipGetLastError();
-      slot = nullptr;
-    }
-  }
-  return slot;
+  SlabBuffers& b = slab_buffers();
+  std::lock_guard<std::mutex> g(b.lock);
+  auto it = b.of.find({dev, stream});
+  return it == b.of.end() ? nullptr : it->second;
+}
+
+// Which of the tile kernels' own choices the variant table fixes ("gemm_w_<format>": 4 = never the slab kernel,
+// 5 = the slab kernel wherever it fits); anything else leaves the measured rule.
+constexpr int kVariantWindow = 4, kVariantSlab = 5;
+
+template <int F>
+const char* gemm_key() {
+  return F == LX_W_BF16 ? "gemm_w_bf16" : F == LX_W_INT8 ? "gemm_w_int8" : F == LX_W_FP8 ? "gemm_w_fp8" : "gemm_w_nvfp4";
 }
 
 // Where the slab kernel is tried before the windowed one. Measured on MI355X (fp8, int8 and bf16 weights, bf16
@@ -965,15 +977,14 @@ void* slab_scratch(hipStream_t stream, size_t bytes, bool capturing) {
 // rows with at most 400 tiles (6144 x 4096 at 48 rows: 22.7 -> 18.7 us, at 64: 26.2 -> 22.4 us; 4096 x 4096 at 64:
 // 21.5 -> 17.6 us), and more than 16 rows with K >= 8192 and few tiles (4096 x 8192 at 32 rows: 21.3 -> 15.3 us, at 64:
 // 35.7 -> 22.7 us). With many tiles (14336 x 4096) its second pass over the partial tiles costs more than the windows do.
-// LX_SLAB_MIN_ROWS (a tuning knob) overrides: rows from which it is tried.
-inline bool slab_wanted(int M, int n_tiles, int64_t K) {
-  if (const char* e = getenv("LX_SLAB_MIN_ROWS")) return M >= atoi(e);
+inline bool slab_wanted(int M, int n_tiles, int64_t K, int tuned) {
+  if (tuned == kVariantWindow) return false;
+  if (tuned == kVariantSlab) return true;
   return n_tiles <= 400 && (M > 32 || (M > 16 && K >= 8192));
 }
 
 // Launches the slab kernel for a.M <= 64 rows; false when it does not apply: the slice's image does not fit LDS, the
-// matrix has too few tiles to give every compute unit a slab, or (S > 1) the stream is being captured, where the
-// partial tiles' memory cannot be asked for.
+// matrix has too few tiles to give every compute unit a slab, or (S > 1) the stream has no buffer for the partial tiles.
 template <int F, int MATH>
 bool launch_slab(GemmArgs a, int* status, hipStream_t stream) {
   constexpr bool I8 = MATH != LX_MATH_BF16;
@@ -993,14 +1004,8 @@ bool launch_slab(GemmArgs a, int* status, hipStream_t stream) {
   if (n_tiles * S < compute_units() * 4) return false;  // too little work to give every unit a slab of several tiles
   void* partial = nullptr;
   if (S > 1) {
-    hipStreamCaptureStatus cap = hipStreamCaptureStatusNone;
-    // (The null stream is never captured, and asking about it is an error in some runtimes.)
-    if (stream && hipStreamIsCapturing(stream, &cap) != hipSuccess) {
-      (void)hipGetLastError();
-      return false;
-    }
     const size_t mts = static_cast<size_t>((a.M + 15) / 16);
-    partial = slab_scratch(stream, sizeof(float) * 4 * kWave * mts * n_tiles * S, cap != hipStreamCaptureStatusNone);
+    partial = slab_scratch(stream, sizeof(float) * 4 * kWave * mts * n_tiles * S);
     if (!partial) return false;
   }
   a.partial = partial;
@@ -1298,16 +1303,15 @@ int launch_skinny_x(const GemmArgs& a, size_t lds, unsigned grid, unsigned threa
 // has the tiles to give most compute units a workgroup: 14336 x 4096 int8 at 16 / 32 / 64 rows 16.0 / 20.7 / 29.9 ->
 // 15.2 / 18.1 / 25.4 us, 16384 x 4096 fp8 at 32 rows 21.5 -> 17.5 us, 6144 x 4096 14.2 -> 12.7 us, 4096 x 4096
 // 13.6 -> 12.7 us; on 4096 x 8192 (32 groups) and at 8 rows and fewer the tile kernels are faster. The variant table
-// ("gemm_w_<format>": 0 = the tile kernels, 1 .. 3 = walk with 1, 2, 4 tiles a workgroup) overrides; no variant changes
-// a sum.
+// ("gemm_w_<format>": 0 = the tile kernels by their own rule, 1 .. 3 = walk with 1, 2, 4 tiles a workgroup, 4 / 5 = the
+// tile kernels without / with the slab kernel) overrides; no variant changes a sum.
 template <int F>
 bool try_walk(const GemmArgs& a, int* status, hipStream_t stream) {
   if (a.xs.dtype != LX_BF16) return false;
-  static const char* const kKey = F == LX_W_BF16 ? "gemm_w_bf16" : F == LX_W_INT8 ? "gemm_w_int8" : F == LX_W_FP8 ? "gemm_w_fp8" : "gemm_w_nvfp4";
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
-  const int tuned = tuned_variant(kKey, a.M, a.N, a.K);
+  const int tuned = tuned_variant(gemm_key<F>(), a.M, a.N, a.K);
   int W;
-  if (tuned == 0) return false;
+  if (tuned == 0 || tuned == kVariantWindow || tuned == kVariantSlab) return false;
   if (tuned >= 1 && tuned <= 3) {
     W = 1 << (tuned - 1);
   } else {
@@ -1332,7 +1336,7 @@ int launch_skinny(GemmArgs a, hipStream_t stream) {
   // sixteen-wavefront workgroups; the lean kernel's image of all of K leaves too few of them resident there).
   if (MT > 1 || (a.M > 8 && n_tiles >= 320)) {
     int st = kOk;
-    if (slab_wanted(a.M, static_cast<int>(n_tiles), a.K) && launch_slab<F, LX_MATH_BF16>(a, &st, stream)) return st;
+    if (slab_wanted(a.M, static_cast<int>(n_tiles), a.K, tuned_variant(gemm_key<F>(), a.M, a.N, a.K)) && launch_slab<F, LX_MATH_BF16>(a, &st, stream)) return st;
     if (launch_window<F, LX_MATH_BF16>(a, &st, stream)) return st;
   }
   if constexpr (MT == 1) {
@@ -1558,7 +1562,7 @@ int gemm_bytes_math(const void* x, int x_dtype, int64_t ld_x, const lx_weight& w
         return status_of(hipGetLastError());
       };
       const int mt = (a.M + 15) / 16;
-      if ((mt > 1 || (a.M > 8 && n_tiles >= 320)) && slab_wanted(a.M, static_cast<int>(n_tiles), K) && launch_slab<F, MATH>(a, &st, s)) continue;
+      if ((mt > 1 || (a.M > 8 && n_tiles >= 320)) && slab_wanted(a.M, static_cast<int>(n_tiles), K, tuned_variant(gemm_key<F>(), a.M, N, K)) && launch_slab<F, MATH>(a, &st, s)) continue;
       if ((mt > 1 || (a.M > 8 && n_tiles >= 320)) && launch_window<F, MATH>(a, &st, s)) continue;
       if (mt == 1 && launch_tile16<F, MATH>(a, &st, s)) continue;
       if (mt == 1) {
@@ -1622,6 +1626,37 @@ int gemm_image_math(int math, const void* x, int x_dtype, int64_t ld_x, const lx
   if (!st) st = gemm_bf16_scaled(xhat, LX_BF16, K, w, bias, bias_dtype, y, y_dtype, ld_y, M, N, K, alpha, beta, scales, stream);
   if (own) (void)hipFreeAsync(own, s);
   return st;
+}
+
+// The stream's buffer for the slab kernel's partial tiles (runtime.hip makes one with every stream it creates).
+int slab_reserve(hipStream_t stream) {
+  int dev = 0;
+  if (int e = status_of(hipGetDevice(&dev))) return e;
+  SlabBuffers& b = slab_buffers();
+  std::lock_guard<std::mutex> g(b.lock);
+  void*& slot = b.of[{dev, stream}];
+  if (slot) return kOk;
+  if (hipMalloc(&slot, kSlabScratchBytes) != hipSuccess) {
+    (void)hipGetLastError();
+    b.of.erase({dev, stream});
+    return fail(kNoMemory);
+  }
+  return kOk;
+}
+
+int slab_release(hipStream_t stream) {
+  int dev = 0;
+  if (int e = status_of(hipGetDevice(&dev))) return e;
+  void* buffer = nullptr;
+  {
+    SlabBuffers& b = slab_buffers();
+    std::lock_guard<std::mutex> g(b.lock);
+    auto it = b.of.find({dev, stream});
+    if (it == b.of.end()) return kOk;
+    buffer = it->second;
+    b.of.erase(it);
+  }
+  return status_of(hipFree(buffer));
 }
 
 }  // namespace dro

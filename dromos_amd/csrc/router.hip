@@ -1,6 +1,6 @@
 // The calls either side of the routed experts in a decode layer, and the legacy forms of the products:
-// lx_spec_gemv_f32, lx_router_route, lx_moe_summary, lx_moe_summary_history, lx_moe_experts_w8, lx_gemm_bf16
-// (contracts: engine/cuda/kernels.h:66-70,211-233,253-261,814-819; CPU behaviour: engine/cpu/gemm.cpp:304-337,
+// lx_spec_gemv_f32, lx_gemm_f32, lx_router_route, lx_moe_summary, lx_moe_summary_history, lx_moe_experts_w8, lx_gemm_bf16
+// (contracts: engine/cuda/kernels.h:66-76,211-233,253-261,814-819; CPU behaviour: engine/cpu/gemm.cpp:304-337,
 // engine/cpu/spec.cpp:21-28, engine/cpu/moe.cpp:399-442,460-476,512-517).
 #include "common.h"
 #include "moe_common.h"
@@ -15,16 +15,20 @@ namespace {
 constexpr int kThreads = 256;
 constexpr int kSpecRows = 8;  // engine/cpu/spec.cpp:12
 
-// y[m, n] = sum_k x[m, k] * w[n, k] + bias[n] on f32 weights: one wavefront per output column n for all M <= 8 rows,
-// a lane taking four consecutive k of every 256 (a 16-byte load where the rows allow it), f32 FMAs in ascending k, the
-// lane sums combined by one fixed tree. Nothing in a row's sums depends on the other rows.
+// y[m, n] = sum_k x[m, k] * w[n, k] + bias[n] on f32 weights: one wavefront per output column n and block of eight rows
+// (blockIdx.y; the last block may hold fewer), a lane taking four consecutive k of every 256 (a 16-byte load where the
+// rows allow it), f32 FMAs in ascending k, the lane sums combined by one fixed tree. Nothing in a row's sums depends on
+// the other rows.
 template <bool VEC>
 __global__ void __launch_bounds__(kThreads) spec_gemv_f32_kernel(const float* __restrict__ x, int64_t ld_x, const float* __restrict__ w,
                                                                  const float* __restrict__ bias, float* __restrict__ y, int64_t ld_y,
-                                                                 int M, int N, int K) {
+                                                                 int rows, int N, int K) {
   const int lane = threadIdx.x & (kWave - 1);
   const int64_t n = static_cast<int64_t>(blockIdx.x) * (kThreads / kWave) + threadIdx.x / kWave;
   if (n >= N) return;
+  const int m0 = blockIdx.y * kSpecRows, M = min(kSpecRows, rows - m0);
+  x += m0 * ld_x;
+  y += m0 * ld_y;
   const float* wrow = w + n * K;
   float acc[kSpecRows];
 #pragma unroll
@@ -63,7 +67,7 @@ __global__ void __launch_bounds__(kThreads) spec_gemv_f32_kernel(const float* __
 
 int spec_gemv(const float* x, int ld_x, const float* w, const float* bias, float* y, int ld_y, int M, int N, int K, hipStream_t s) {
   const bool vec = K % 4 == 0 && ld_x % 4 == 0 && reinterpret_cast<uintptr_t>(x) % 16 == 0 && reinterpret_cast<uintptr_t>(w) % 16 == 0;
-  const dim3 grid((N + kThreads / kWave - 1) / (kThreads / kWave));
+  const dim3 grid((N + kThreads / kWave - 1) / (kThreads / kWave), (M + kSpecRows - 1) / kSpecRows);
   if (vec) hipLaunchKernelGGL(spec_gemv_f32_kernel<true>, grid, dim3(kThreads), 0, s, x, ld_x, w, bias, y, ld_y, M, N, K);
   else hipLaunchKernelGGL(spec_gemv_f32_kernel<false>, grid, dim3(kThreads), 0, s, x, ld_x, w, bias, y, ld_y, M, N, K);
   return status_of(hipGetLastError());
@@ -101,6 +105,16 @@ using namespace dro;
 extern "C" {
 
 int64_t lx_moe_decode_workspace_bytes(int T, int I, int top_k);
+
+// engine/cuda/kernels.h:72-76, engine/cpu/gemm.cpp:316-337: the same product for any number of rows (the routers and
+// the depth head at more than eight rows); a row's bits are those of lx_spec_gemv_f32.
+int lx_gemm_f32(const float* x, int ld_x, const float* w, const float* bias, float* y, int ld_y, int M, int N, int K, void* stream) {
+  if (M < 0 || N < 0 || K <= 0 || ld_x < K || ld_y < N) return fail(kInvalid);
+  if (M == 0 || N == 0) return kOk;
+  if (!x || !w || !y) return fail(kInvalid);
+  if (M > 65535 * kSpecRows) return fail(kInvalid);
+  return spec_gemv(x, ld_x, w, bias, y, ld_y, M, N, K, as_stream(stream));
+}
 
 int lx_spec_gemv_f32(const float* x, int ld_x, const float* w, const float* bias, float* y, int ld_y, int M, int N, int K,
                      void* stream) {

@@ -57,6 +57,10 @@ void allow_lds(const void* kernel, int limit) {
   raised.emplace_back(dev, kernel, limit);
 }
 
+// gemm.hip: the per-stream buffer of the slab kernel's partial tiles.
+int slab_reserve(hipStream_t stream);
+int slab_release(hipStream_t stream);
+
 // Admission rule of the GEMV's variants (gemv.hip).
 bool gemv_admits(int wtype, int variant, int N, int K);
 
@@ -75,17 +79,18 @@ struct Registered {
 
 // The kernels with variants. The GEMV of each format has three: its K split of 1, 2 or 4 wavefronts (admitted where the
 // split is the shape's order class). The matrix-core product of each format (9 .. 64 activation rows) has four: the tile
-// kernels, or the walk kernel with 1, 2 or 4 tiles a workgroup; none changes a sum, so all are admitted.
+// kernels by their own rule, the walk kernel with 1, 2 or 4 tiles a workgroup, the tile kernels without or with the slab
+// kernel; none changes a sum, so all are admitted.
 const std::map<std::string, Registered>& registry() {
   static const auto* r = new std::map<std::string, Registered>{
       {"gemv_w_bf16", {{"s1", "s2", "s4"}, LX_W_BF16}},
       {"gemv_w_int8", {{"s1", "s2", "s4"}, LX_W_INT8}},
       {"gemv_w_fp8", {{"s1", "s2", "s4"}, LX_W_FP8}},
       {"gemv_w_nvfp4", {{"s1", "s2", "s4"}, LX_W_NVFP4}},
-      {"gemm_w_bf16", {{"tiles", "walk1", "walk2", "walk4"}, -1}},
-      {"gemm_w_int8", {{"tiles", "walk1", "walk2", "walk4"}, -1}},
-      {"gemm_w_fp8", {{"tiles", "walk1", "walk2", "walk4"}, -1}},
-      {"gemm_w_nvfp4", {{"tiles", "walk1", "walk2", "walk4"}, -1}},
+      {"gemm_w_bf16", {{"tiles", "walk1", "walk2", "walk4", "window", "slab"}, -1}},
+      {"gemm_w_int8", {{"tiles", "walk1", "walk2", "walk4", "window", "slab"}, -1}},
+      {"gemm_w_fp8", {{"tiles", "walk1", "walk2", "walk4", "window", "slab"}, -1}},
+      {"gemm_w_nvfp4", {{"tiles", "walk1", "walk2", "walk4", "window", "slab"}, -1}},
   };
   return *r;
 }
@@ -166,7 +171,26 @@ __global__ void fill_random_kernel(unsigned* p, int64_t n) {
 
 }  // namespace
 
+namespace {
+// lx_tune_run's choice for the launches it makes on this thread: it goes before the table.
+thread_local const char* g_run_kernel = nullptr;
+thread_local int g_run_variant = -1;
+// bf16 values spread evenly over (-scale, scale), a fixed function of the index and the seed.
+__global__ void fill_bf16_kernel(uint16_t* p, int64_t n, unsigned seed, float scale) {
+  const int64_t i = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  unsigned x = (static_cast<unsigned>(i) + seed) * 2654435761u + 0x9e3779b9u;
+  x ^= x >> 16;
+  x *= 0x85ebca6bu;
+  x ^= x >> 13;
+  const float v = (static_cast<float>(x >> 8) * (1.0f / 8388608.0f) - 1.0f) * scale;
+  p[i] = f32_to_bf16_bits(v);
+}
+
+}  // namespace
+
 int tuned_variant(const char* kernel, int M, int N, int K) {
+  if (g_run_kernel && strcmp(g_run_kernel, kernel) == 0) return g_run_variant;
   std::lock_guard<std::mutex> g(table_lock());
   if (table().empty()) return -1;
   auto it = table().find(Key{kernel, bucket(M), N, K});
@@ -228,9 +252,17 @@ int lx_rt_stream_create(void** stream) {
   hipStream_t s = nullptr;
   const int e = status_of(hipStreamCreateWithFlags(&s, hipStreamNonBlocking));  // default priority
   *stream = s;
+  // What the products keep per stream is made here, so that no product ever allocates; a stream that cannot have it
+  // still works (those products take another kernel).
+  if (!e) (void)slab_reserve(s);
   return e;
 }
-int lx_rt_stream_destroy(void* stream) { return status_of(hipStreamDestroy(as_stream(stream))); }
+int lx_rt_stream_destroy(void* stream) {
+  (void)slab_release(as_stream(stream));
+  return status_of(hipStreamDestroy(as_stream(stream)));
+}
+int lx_rt_stream_reserve(void* stream) { return slab_reserve(as_stream(stream)); }
+int lx_rt_stream_release(void* stream) { return slab_release(as_stream(stream)); }
 int lx_rt_stream_sync(void* stream) { return status_of(hipStreamSynchronize(as_stream(stream))); }
 
 int lx_rt_event_create(void** event) {
@@ -465,6 +497,115 @@ const char* lx_tune_variant_name(const char* kernel, int variant) {
   auto reg = registry().find(kernel);
   if (reg == registry().end() || variant < 0 || variant >= static_cast<int>(reg->second.variants.size())) return "";
   return reg->second.variants[variant].c_str();
+}
+
+
+// ---- the autotuner's entry points (engine/cuda/tunable.h:57-75, engine/cuda/tunable.cu:158-185) --------------------
+
+namespace {
+
+// What a runnable kernel is timed on: weights of its format made from seeded bf16 values by the library's own quantiser,
+// bf16 activations; kept per problem for the life of the process (the tuner asks for each many times).
+struct TuneInputs {
+  void* w = nullptr;
+  void* scale = nullptr;
+  void* x = nullptr;
+  float global = 1.0f;
+};
+
+int format_of_kernel(const std::string& kernel, bool* gemv) {
+  static const char* const kNames[4] = {"bf16", "int8", "fp8", "nvfp4"};
+  for (int f = 0; f < 4; ++f) {
+    if (kernel == std::string("gemv_w_") + kNames[f]) return *gemv = true, f;
+    if (kernel == std::string("gemm_w_") + kNames[f]) return *gemv = false, f;
+  }
+  return -1;
+}
+
+int tune_inputs(int format, int M, int N, int K, hipStream_t s, TuneInputs* out) {
+  static std::mutex lock;
+  static std::map<std::tuple<int, int, int, int, int>, TuneInputs> cache;
+  int dev = 0;
+  if (int e = status_of(hipGetDevice(&dev))) return e;
+  std::lock_guard<std::mutex> g(lock);
+  auto it = cache.find({dev, format, M, N, K});
+  if (it != cache.end()) return *out = it->second, kOk;
+  TuneInputs in;
+  void* master = nullptr;
+  const int64_t wn = static_cast<int64_t>(N) * K, xn = static_cast<int64_t>(M) * K;
+  auto release = [&] {
+    (void)hipFree(master);
+    (void)hipFree(in.w);
+    (void)hipFree(in.scale);
+    (void)hipFree(in.x);
+  };
+  if (hipMalloc(&master, wn * 2) != hipSuccess || hipMalloc(&in.x, xn * 2) != hipSuccess) return release(), fail(kNoMemory);
+  hipLaunchKernelGGL(fill_bf16_kernel, dim3(static_cast<unsigned>((wn + 255) / 256)), dim3(256), 0, s, static_cast<uint16_t*>(master), wn, 17u, 0.04f);
+  hipLaunchKernelGGL(fill_bf16_kernel, dim3(static_cast<unsigned>((xn + 255) / 256)), dim3(256), 0, s, static_cast<uint16_t*>(in.x), xn, 91u, 1.0f);
+  int st = status_of(hipGetLastError());
+  if (!st && format == LX_W_BF16) {
+    in.w = master;
+    master = nullptr;
+  } else if (!st) {
+    const int64_t data_bytes = format == LX_W_NVFP4 ? wn / 2 : wn;
+    const int64_t scale_bytes = format == LX_W_NVFP4 ? wn / 16 : static_cast<int64_t>(N) * 4;
+    if (hipMalloc(&in.w, data_bytes) != hipSuccess || hipMalloc(&in.scale, scale_bytes) != hipSuccess) return release(), fail(kNoMemory);
+    lx_weight q{static_cast<lx_wtype>(format), in.w, in.scale, 1.0f, nullptr};
+    st = lx_quantize_weight(master, &q, N, K, s);
+    in.global = q.global;
+  }
+  if (!st) st = status_of(hipStreamSynchronize(s));
+  (void)hipFree(master);
+  master = nullptr;
+  if (st) return release(), st;
+  cache[{dev, format, M, N, K}] = in;
+  *out = in;
+  return kOk;
+}
+
+}  // namespace
+
+int lx_tune_runnable(const char* kernel) {
+  bool gemv;
+  return kernel && format_of_kernel(kernel, &gemv) >= 0 ? 1 : 0;
+}
+
+int lx_tune_key(const char* kernel, const lx_tune_problem* problem, char* out, int capacity) {
+  if (!kernel || !problem) return 0;
+  std::string key = kernel;
+  if (problem->weight != 0 || problem->math != 0) key += "@w" + std::to_string(problem->weight) + "m" + std::to_string(problem->math);
+  if (problem->experts != 1) key += "@e" + std::to_string(problem->experts);
+  if (out && capacity > 0) {
+    const size_t n = key.size() < static_cast<size_t>(capacity - 1) ? key.size() : static_cast<size_t>(capacity - 1);
+    memcpy(out, key.data(), n);
+    out[n] = '\0';
+  }
+  return static_cast<int>(key.size());
+}
+
+// Runs one variant of a registered product on inputs of its own and writes y as f32 [M, N] to `out` (device memory).
+// The kernels' names carry their weight format, so a problem names it again or leaves it 0; the BF16 math and single
+// weights only.
+int lx_tune_run(const char* kernel, int variant, const lx_tune_problem* problem, float* out, void* stream) {
+  if (!kernel || !problem || !out) return fail(kInvalid);
+  bool gemv = false;
+  const int format = format_of_kernel(kernel, &gemv);
+  if (format < 0) return kNotSupported;
+  if (variant < 0 || variant >= lx_tune_variants(kernel)) return kNotSupported;
+  const int M = problem->M, N = problem->N, K = problem->K;
+  if (M <= 0 || N <= 0 || K <= 0) return fail(kInvalid);
+  if (problem->experts != 1 || problem->math != LX_MATH_BF16 || (problem->weight != 0 && problem->weight != format)) return kNotSupported;
+  if ((gemv && M > 8) || (format == LX_W_NVFP4 && K % 16 != 0)) return kNotSupported;
+  TuneInputs in;
+  if (int e = tune_inputs(format, M, N, K, as_stream(stream), &in)) return e;
+  const lx_weight w{static_cast<lx_wtype>(format), in.w, in.scale, in.global, nullptr};
+  g_run_kernel = kernel;
+  g_run_variant = variant;
+  const int st = gemv ? lx_gemv_w(in.x, LX_BF16, K, &w, nullptr, LX_F32, out, LX_F32, N, M, N, K, 1.0f, 0.0f, stream)
+                      : lx_gemm_w(in.x, LX_BF16, K, &w, LX_MATH_BF16, nullptr, LX_F32, out, LX_F32, N, M, N, K, 1.0f, 0.0f, nullptr, stream);
+  g_run_kernel = nullptr;
+  g_run_variant = -1;
+  return st;
 }
 
 }  // extern "C"

@@ -185,6 +185,8 @@ LX_API int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int to
 /* ---- the calls either side of the experts in a decode layer (replaces engine/cuda/kernels.h:211-233, 253-261,
  * 814-819; the model calls them at engine/model/metis.cpp:2086-2096) and the legacy product forms (:66-70) ------
  *   lx_spec_gemv_f32        y[M, N] = x[M, K] @ w[N, K]^T + bias[N], all f32, M <= 8, a row's bits independent of M
+ *   lx_gemm_f32             the same product for any M (engine/cuda/kernels.h:72-76: the routers and the depth head,
+ *                           engine/model/metis.cpp:1314-1319,2095); a row's bits are lx_spec_gemv_f32's
  *   lx_router_route         that product on the router's weights w [E, K] into logits [M, E], then lx_moe_route on
  *                           them: every output has the bits of the two calls (it is the two calls, in two launches);
  *                           M <= 8, E <= 1024, K <= 2048, top_k <= 32; `ticket` (one zeroed int32 the fused CUDA
@@ -196,6 +198,8 @@ LX_API int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int to
  *   lx_gemm_bf16            y = alpha * (x @ w^T + bias) + beta * y, x and w bf16, bias bf16 or null, any M */
 LX_API int lx_spec_gemv_f32(const float* x, int ld_x, const float* w, const float* bias, float* y, int ld_y, int M, int N,
                             int K, void* stream);
+LX_API int lx_gemm_f32(const float* x, int ld_x, const float* w, const float* bias, float* y, int ld_y, int M, int N, int K,
+                       void* stream);
 LX_API int lx_router_route(const float* x, int ld_x, const float* w, const float* bias, float* logits,
                            const float* selection_bias, int32_t* ids, float* weights, float* entropy, float* confidence,
                            int32_t* ticket, int M, int E, int K, int top_k, void* stream);
@@ -248,6 +252,13 @@ LX_API int lx_rt_copy(void* dst, const void* src, int64_t bytes, lx_copy_kind ki
 LX_API int lx_rt_stream_create(void** stream);
 LX_API int lx_rt_stream_destroy(void* stream);
 LX_API int lx_rt_stream_sync(void* stream);
+/* No counterpart in the reference. A stream made by lx_rt_stream_create owns 64 MiB of device memory that some products
+ * of lx_gemm_w / lx_gemm_skinny (17 .. 64 rows on matrices of few tiles) keep their partial sums in; no product ever
+ * allocates. A host that brings streams of its own (or uses the null stream) calls lx_rt_stream_reserve once per stream
+ * (and device) to give it the same, and lx_rt_stream_release before it destroys the stream; without it those products
+ * take another kernel with the same results. */
+LX_API int lx_rt_stream_reserve(void* stream);
+LX_API int lx_rt_stream_release(void* stream);
 LX_API int lx_rt_event_create(void** event);
 LX_API int lx_rt_event_create_timed(void** event);
 LX_API int lx_rt_event_destroy(void* event);
@@ -316,7 +327,9 @@ LX_API int lx_probe_empty(void* stream);
 /* ---- architecture and kernel variants (replaces engine/cuda/tunable.h:37-55) -----------------------
  * lx_arch is 95 on gfx950. The GEMV registers its variants under gemv_w_<format>; a variant's name starts
  * with s<S>, its K split, and lx_tune_set admits a variant for a shape only when its split is the
- * shape's own (so the rows' bits never depend on the table). */
+ * shape's own (so the rows' bits never depend on the table). The matrix-core products (lx_gemm_w, lx_gemm_skinny)
+ * register theirs under gemm_w_<format>: which kernel family runs ("tiles", "walk1", "walk2", "walk4", "window",
+ * "slab"); none changes a sum, so every one is admitted. */
 LX_API int lx_arch(void);
 LX_API int lx_set_arch_override(int arch);
 LX_API int lx_tune_get(const char* kernel, int M, int N, int K);
@@ -326,6 +339,24 @@ LX_API void lx_tune_clear(void);
 LX_API int lx_tune_kernels(const char** names, int capacity);
 LX_API int lx_tune_variants(const char* kernel);
 LX_API const char* lx_tune_variant_name(const char* kernel, int variant);
+/* The autotuner's entry points (engine/cuda/tunable.h:57-75). A problem is one timed case: M rows against an N x K
+ * weight in format `weight` and math `math` (0 for both: the kernel's own), `experts` such weights (1 here).
+ *   lx_tune_run       runs variant `variant` of a registered kernel on inputs of its own making (seeded, kept per
+ *                     problem) and writes the result as f32 [M, N] to `out` (device memory); 801 when the kernel has no
+ *                     runner or the variant / problem cannot run (the tuner skips those)
+ *   lx_tune_runnable  1 when lx_tune_run can run the kernel's variants (gemv_w_<format>, gemm_w_<format>), else 0
+ *   lx_tune_key       the table key of a kernel's problem: the name, then "@w<weight>m<math>" when either is not 0,
+ *                     then "@e<experts>" when it is not 1 (engine/cuda/tunable.cu:180-185); writes it NUL-terminated
+ *                     into `out` (at most `capacity` bytes) and returns its length */
+typedef struct {
+  int M, N, K;
+  int experts;
+  int weight;
+  int math;
+} lx_tune_problem;
+LX_API int lx_tune_run(const char* kernel, int variant, const lx_tune_problem* problem, float* out, void* stream);
+LX_API int lx_tune_runnable(const char* kernel);
+LX_API int lx_tune_key(const char* kernel, const lx_tune_problem* problem, char* out, int capacity);
 
 #ifdef __cplusplus
 }

@@ -192,6 +192,20 @@ def spec_gemv_f32(lx, x, w, bias=None, M=None, status=False):
     return y[:M]
 
 
+def gemm_f32(lx, x, w, bias=None, pad=0, status=False):
+    """lx_gemm_f32 with `pad` unused columns behind the rows of x and y."""
+    M, K = x.shape
+    N = w.shape[0]
+    xb = torch.zeros(M, K + pad, device=lx.device)
+    xb[:, :K] = x
+    y = torch.full((max(M, 1), N + pad), float("nan"), device=lx.device)
+    args = (xb, K + pad, w, bias, y, N + pad, M, N, K)
+    if status:
+        return lx.status("gemm_f32", *args)
+    lx("gemm_f32", *args)
+    return y[:M]
+
+
 def router_route(lx, x, w, bias, selection_bias, top_k, status=False):
     M, K = x.shape
     E = w.shape[0]

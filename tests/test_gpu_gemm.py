@@ -295,21 +295,22 @@ def test_slab_shapes_give_the_bits_of_every_other_kernel(hip, fmt, M, N, K):
 @pytest.mark.parametrize("fmt", FMT)
 @pytest.mark.parametrize("M,N,K", [(17, 1027, 2048), (64, 300, 4096), (33, 4096, 1040), (48, 14336, 4096)])
 def test_slab_forced_equals_the_windowed_kernel(hip, fmt, M, N, K):
-    # The tuning knob sends any row count to the slab kernel where it fits (ragged N and K included): same bits as
-    # without it, for f32 and bf16 activations and beta != 0.
+    # The variant table sends any row count to the slab kernel where it fits (ragged N and K included), or keeps it
+    # away: same bits, for f32 and bf16 activations and beta != 0.
     g = torch.Generator().manual_seed(N)
     w = random_weight(FORMATS[fmt], N, K - K % 16, N).to("cuda")
     K = K - K % 16
     for x_dtype in (torch.bfloat16, torch.float32):
         x = torch.randn(M, K, generator=g).to(x_dtype).cuda()
         y0 = torch.randn(M, N, generator=g).cuda()
+        key = f"gemm_w_{fmt}".encode()
         try:
-            os.environ["LX_SLAB_MIN_ROWS"] = "1000"
+            assert hip.lib.lx_tune_force(key, M, N, K, 4) == 0  # "window": never the slab kernel
             a = ops.gemm_w(hip, x, w, MATH_BF16, y=y0.clone(), alpha=1.25, beta=-0.5)
-            os.environ["LX_SLAB_MIN_ROWS"] = "1"
+            assert hip.lib.lx_tune_force(key, M, N, K, 5) == 0  # "slab": wherever it fits
             b = ops.gemm_w(hip, x, w, MATH_BF16, y=y0.clone(), alpha=1.25, beta=-0.5)
         finally:
-            os.environ.pop("LX_SLAB_MIN_ROWS", None)
+            hip.lib.lx_tune_clear()
         assert torch.equal(a.view(torch.int32), b.view(torch.int32)), x_dtype
 
 

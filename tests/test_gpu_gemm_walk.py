@@ -1,7 +1,8 @@
 """GPU parity: the walk kernel of lx_gemm_w / lx_gemm_skinny (9 .. 64 bf16 activation rows, a wavefront walking a whole
 tile) against float64 on the decoded values, and bit for bit against the tile kernels it replaces on the shapes it
-takes: the variant table forces each family ("gemm_w_<format>": 0 = tiles, 1 .. 3 = walk with 1, 2, 4 tiles a
-workgroup), and no variant may change an output bit, a row's bits may not depend on the batch."""
+takes: the variant table forces each family ("gemm_w_<format>": 0 = the tile kernels, 1 .. 3 = walk with 1, 2, 4 tiles
+a workgroup, 4 / 5 = the tile kernels without / with the slab kernel), and no variant may change an output bit, a row's
+bits may not depend on the batch."""
 
 import pytest
 import torch
@@ -35,10 +36,10 @@ def test_variants_are_registered(hip):
     hip.lib.lx_tune_variant_name.restype = ctypes.c_char_p
     for fmt in FMT:
         key = f"gemm_w_{fmt}".encode()
-        assert hip.lib.lx_tune_variants(key) == 4
-        assert [hip.lib.lx_tune_variant_name(key, v).decode() for v in range(4)] == ["tiles", "walk1", "walk2", "walk4"]
-        assert all(hip.lib.lx_tune_set(key, 32, 4096, 4096, v) == 0 for v in range(4))  # none changes a sum: all admitted
-        assert hip.lib.lx_tune_set(key, 32, 4096, 4096, 4) == 803
+        assert hip.lib.lx_tune_variants(key) == 6
+        assert [hip.lib.lx_tune_variant_name(key, v).decode() for v in range(6)] == ["tiles", "walk1", "walk2", "walk4", "window", "slab"]
+        assert all(hip.lib.lx_tune_set(key, 32, 4096, 4096, v) == 0 for v in range(6))  # none changes a sum: all admitted
+        assert hip.lib.lx_tune_set(key, 32, 4096, 4096, 6) == 803
 
 
 @pytest.mark.parametrize("M", [9, 16, 17, 33, 48, 64])
@@ -52,7 +53,7 @@ def test_every_variant_gives_the_same_bits(hip, fmt, M):
         want = ops.gemv_reference(x, w.dense(), bias, 1.0, 0.0, None)
         wd, xd, bd = w.to("cuda"), x.cuda(), bias.cuda()
         outs = {}
-        for variant in (0, 1, 2, 3, None):
+        for variant in (0, 1, 2, 3, 4, 5, None):
             force(hip, fmt, M, N, K, variant)
             y = torch.full((M, N), float("nan"), device="cuda")
             outs[variant] = ops.gemm_w(hip, xd, wd, MATH_BF16, bias=bd, y=y).clone()
@@ -115,3 +116,37 @@ def test_walk_under_a_quantised_math(hip):
         force(hip, "nvfp4", M, N, K, variant)
         outs.append(ops.gemm_w(hip, x, w, MATH_FP8).clone())
     assert torch.equal(outs[0].view(torch.int32), outs[1].view(torch.int32))
+
+
+class TuneProblem(__import__("ctypes").Structure):
+    _fields_ = [(n, __import__("ctypes").c_int) for n in ("M", "N", "K", "experts", "weight", "math")]
+
+
+@pytest.mark.parametrize("fmt", FMT)
+def test_tune_run_times_what_the_table_would_pick(hip, fmt):
+    # engine/cuda/tunable.h:57-75: every variant of a runnable kernel runs on the kernel's own inputs and writes f32
+    # [M, N]; the products' variants agree bit for bit, the GEMV's K splits within the sums' rounding.
+    import ctypes
+
+    N, K = SHAPES[fmt][1]
+    for kernel, M, exact in ((f"gemm_w_{fmt}", 32, True), (f"gemv_w_{fmt}", 4, False)):
+        p = TuneProblem(M, N, K, 1, 0, 0)
+        outs = []
+        for v in range(hip.lib.lx_tune_variants(kernel.encode())):
+            out = torch.full((M, N), float("nan"), device="cuda")
+            assert hip.status("tune_run", kernel.encode(), v, ctypes.byref(p), out) == 0, (kernel, v)
+            torch.cuda.synchronize()
+            assert torch.isfinite(out).all() and out.abs().max() > 0
+            outs.append(out)
+        for v, out in enumerate(outs):
+            if exact:
+                assert torch.equal(out.view(torch.int32), outs[0].view(torch.int32)), (kernel, v)
+            else:
+                assert ((out - outs[0]).norm() / outs[0].norm()).item() < 1e-5, (kernel, v)
+        assert hip.lib.lx_tune_get(kernel.encode(), M, N, K) == -1  # running a variant leaves the table alone
+    p = TuneProblem(32, N, K, 1, 0, 0)
+    out = torch.zeros(32, N, device="cuda")
+    assert hip.status("tune_run", b"attention", 0, ctypes.byref(p), out) == 801
+    assert hip.status("tune_run", f"gemm_w_{fmt}".encode(), 99, ctypes.byref(p), out) == 801
+    assert hip.status("tune_run", f"gemm_w_{fmt}".encode(), 0, ctypes.byref(TuneProblem(32, N, K, 8, 0, 0)), out) == 801  # stacks
+    assert hip.status("tune_run", f"gemv_w_{fmt}".encode(), 0, ctypes.byref(TuneProblem(9, N, K, 1, 0, 0)), out) == 801  # M > 8

@@ -38,6 +38,33 @@ def test_spec_gemv_f32(hip, oracle, M, N, K):
         assert torch.equal(alone[0].view(torch.int32), y[m].view(torch.int32)), f"row {m}"
 
 
+@pytest.mark.parametrize("pad", [0, 3])
+@pytest.mark.parametrize("M,N,K", [(1, 64, 2048), (9, 128, 2048), (33, 64, 2304), (70, 37, 130), (64, 1, 2048)])
+def test_gemm_f32(hip, oracle, M, N, K, pad):
+    # engine/cuda/kernels.h:72-76 (the reference tests it against float64 with rtol 1e-5, tests/kernels/test_gemm.py:67-80).
+    x, w, bias, _ = router_inputs(M, N, K, M + N + pad)
+    y = ops.gemm_f32(hip, x.cuda(), w.cuda(), bias.cuda(), pad=pad)
+    want = ops.gemm_f32(oracle, x, w, bias, pad=pad)
+    assert rel_l2(y[:, :N], want[:, :N]) <= 1e-5  # f32 sums in another order
+    close(y[:, :N], x.double() @ w.double().T + bias.double(), atol=2e-6 * K**0.5 * max(want[:, :N].abs().max().item(), 1.0))
+    assert torch.isnan(y[:, N:]).all(), "wrote past the N columns of y"
+    # a row's bits are those of the decode-sized call, whatever the batch
+    for m in (0, M // 2, M - 1):
+        alone = ops.spec_gemv_f32(hip, x[m : m + 1].contiguous().cuda(), w.cuda(), bias.cuda())
+        assert torch.equal(alone[0].view(torch.int32), y[m, :N].contiguous().view(torch.int32)), f"row {m}"
+    no_bias = ops.gemm_f32(hip, x.cuda(), w.cuda(), None)
+    assert rel_l2(no_bias, x.double() @ w.double().T) <= 1e-5
+
+
+def test_gemm_f32_arguments(hip):
+    w = torch.zeros(16, 64, device="cuda")
+    assert ops.gemm_f32(hip, torch.zeros(0, 64, device="cuda"), w, None, status=True) == 0
+    y = torch.zeros(4, 16, device="cuda")
+    assert hip.status("gemm_f32", torch.zeros(4, 64, device="cuda"), 32, w, None, y, 16, 4, 16, 64) == 1  # ld_x < K
+    assert hip.status("gemm_f32", torch.zeros(4, 64, device="cuda"), 64, w, None, y, 8, 4, 16, 64) == 1  # ld_y < N
+    assert hip.status("gemm_f32", None, 64, w, None, y, 16, 4, 16, 64) == 1
+
+
 def test_spec_gemv_f32_arguments(hip):
     w = torch.zeros(16, 64, device="cuda")
     assert ops.spec_gemv_f32(hip, torch.zeros(9, 64, device="cuda"), w, None, status=True) == 1
