@@ -59,9 +59,13 @@ class JsonReader {
   }
 
  private:
+  // The files this reads nest three deep (header, tensor entry, shape); a value nested deeper than this is refused
+  // before the recursion that reads it can run the thread out of stack.
+  static constexpr int kMaxDepth = 64;
   const char* p_;
   const char* end_;
   std::string what_;
+  int depth_ = 0;
 
   [[noreturn]] void bad(const char* why) const { refuse(what_ + ": not valid JSON (" + why + ")"); }
   void space() {
@@ -118,6 +122,16 @@ class JsonReader {
   Json value() {
     space();
     if (p_ == end_) bad("the text ends early");
+    if (*p_ == '{' || *p_ == '[') {
+      if (depth_ >= kMaxDepth) bad("objects or arrays nested more than 64 deep");
+      ++depth_;
+      Json v = nested();
+      --depth_;
+      return v;
+    }
+    return scalar();
+  }
+  Json nested() {
     Json v;
     if (*p_ == '{') {
       ++p_;
@@ -137,7 +151,12 @@ class JsonReader {
       do v.items.push_back(value());
       while (take(','));
       if (!take(']')) bad("a ']' was expected");
-    } else if (*p_ == '"') {
+    }
+    return v;
+  }
+  Json scalar() {
+    Json v;
+    if (*p_ == '"') {
       v.kind = Json::kString;
       v.text = string();
     } else if (end_ - p_ >= 4 && !std::strncmp(p_, "true", 4)) {
@@ -254,6 +273,8 @@ class Folder {
     uint64_t header = 0;
     std::memcpy(&header, f.data(), 8);
     if (header > f.size() - 8) refuse(path + ": the header is longer than the file");
+    // The format's own limit on a header (100 MB): a longer one is no model's table of tensors.
+    if (header > 100u * 1000u * 1000u) refuse(path + ": the header is longer than 100 MB");
     const Json doc = JsonReader(reinterpret_cast<const char*>(f.data()) + 8, static_cast<size_t>(header), path).document();
     if (doc.kind != Json::kObject) refuse(path + ": the header is not an object");
     const uint8_t* base = f.data() + 8 + header;
@@ -411,6 +432,11 @@ class Loader {
  public:
   Loader(const Folder& f, int target, int stored, bool skip_experts, Model& out)
       : folder_(f), target_(target), stored_(stored), skip_experts_(skip_experts), out_(out) {}
+  Loader(const Loader&) = delete;
+  Loader& operator=(const Loader&) = delete;
+  // The conversion buffers go with the loader, also when run() leaves by an exception (a refused tensor, a failed
+  // allocation half way through a folder).
+  ~Loader() { release_scratch(); }
 
   void run() {
     std::vector<Projection> list = collect();  // the map's name order: the device layout does not depend on hash order
@@ -574,12 +600,17 @@ class Loader {
       data = std::max(data, static_cast<size_t>(p.shape.N) * data_row_bytes(p.src, p.shape.K));
       scale = std::max(scale, static_cast<size_t>(p.shape.N) * scale_row_bytes(p.src, p.shape.K));
     }
-    bf16_ = device(bf16), qdata_ = device(data), qscale_ = device(scale);
-    scratch_bytes_ = bf16 + data + scale;
+    bf16_ = device(bf16), scratch_bytes_ = bf16;
+    qdata_ = device(data), scratch_bytes_ += data;
+    qscale_ = device(scale), scratch_bytes_ += scale;
   }
   void release_scratch() {
-    for (void* p : {bf16_, qdata_, qscale_}) (void)lx_rt_free(p);
+    for (void** p : {&bf16_, &qdata_, &qscale_}) {
+      if (*p) (void)lx_rt_free(*p);
+      *p = nullptr;
+    }
     live_ -= scratch_bytes_;
+    scratch_bytes_ = 0;
   }
 
   // Expert e of a projection (the whole matrix of a plain one) as bf16 at `dst` on the device.

@@ -167,9 +167,23 @@ int lx_moe_experts_w8(const void* latent, const int32_t* ids, const float* weigh
   if (T <= 0) return kOk;
   if (!latent || !ids || !weights || !out || L <= 0 || I <= 0 || top_k < 1) return fail(kInvalid);
   if (!gate_up || !gate_up_scale || !down || !down_scale || !workspace) return fail(kInvalid);
-  if (top_k > 8) return fail(kNotSupported);
   const lx_weight gu{LX_W_INT8, gate_up, gate_up_scale, 1.0f, nullptr}, dn{LX_W_INT8, down, down_scale, 1.0f, nullptr};
   hipStream_t s = as_stream(stream);
+  if (top_k > 8) {
+    // More picks than the decode kernels take, and no expert count to group pairs by: the element-wise experts, every
+    // pair on its own, the intermediate rows [T * top_k, I] in the workspace (the reference takes any top_k here,
+    // engine/cpu/moe.cpp:460-476).
+    DecodeArgs d{};
+    d.latent = static_cast<const uint16_t*>(latent);
+    d.ids = ids;
+    d.weights = weights;
+    d.gu = as_stack(gu);
+    d.dn = as_stack(dn);
+    d.inter = static_cast<uint16_t*>(workspace);
+    d.out = out;
+    d.T = T, d.L = L, d.I = I, d.top_k = top_k;
+    return experts_plain(d, LX_W_INT8, LX_W_INT8, s);
+  }
   for (int t0 = 0; t0 < T; t0 += 8) {
     const int n = T - t0 < 8 ? T - t0 : 8;
     const int st = experts_decode(static_cast<const uint16_t*>(latent) + static_cast<int64_t>(t0) * L, ids + static_cast<int64_t>(t0) * top_k,

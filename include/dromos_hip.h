@@ -194,7 +194,8 @@ LX_API int64_t lx_moe_grouped_workspace_bytes(int T, int L, int I, int E, int to
  *   lx_moe_summary          summary[t, :] = sum_k weights[t, k] * expert_emb[ids[t, k], :], expert_emb bf16 [E, R],
  *                           summary f32 [T, R]; _history also history = a * history + b * summary in place
  *   lx_moe_experts_w8       lx_moe_experts on int8 stacks with per-row scales (gate_up_scale [E, 2I], down_scale
- *                           [E, L]), any T, top_k <= 8, workspace of lx_moe_workspace_bytes(T, I, top_k)
+ *                           [E, L]), any T and top_k (more than 8 picks take element-wise kernels), workspace of
+ *                           lx_moe_workspace_bytes(T, I, top_k)
  *   lx_gemm_bf16            y = alpha * (x @ w^T + bias) + beta * y, x and w bf16, bias bf16 or null, any M */
 LX_API int lx_spec_gemv_f32(const float* x, int ld_x, const float* w, const float* bias, float* y, int ld_y, int M, int N,
                             int K, void* stream);

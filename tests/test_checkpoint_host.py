@@ -84,6 +84,25 @@ def test_reader_refusals(lib, tmp_path):
         ModelWeights.stored_format(lib, folder("dtype", {"a": {"dtype": "F4", "shape": [8], "data_offsets": [0, 8]}}))
     with pytest.raises(RuntimeError, match="lacks dtype"):
         ModelWeights.stored_format(lib, folder("lacks", {"a": {"dtype": "F32", "shape": [2]}}))
+    # nesting the reader would have to recurse through: refused with a reason, in the header and in the index
+    for i, opener in enumerate((b"[", b"{\"a\":", b"[{\"a\":")):
+        with pytest.raises(RuntimeError, match="nested more than 64 deep"):
+            ModelWeights.stored_format(lib, folder(f"deep{i}", b'{"a": ' + opener * 100000))
+    deep = tmp_path / "deep_index"
+    folders.write(deep, "bf16", shards=2)
+    (deep / "model.safetensors.index.json").write_bytes(b'{"weight_map": ' + b"[" * 100000)
+    with pytest.raises(RuntimeError, match="nested more than 64 deep"):
+        ModelWeights.stored_format(lib, deep)
+    sixty = b'{"__metadata__": ' + b"[" * 62 + b"]" * 62 + b', "a.weight": {"dtype": "BF16", "shape": [2, 2], "data_offsets": [0, 8]}}'
+    assert ModelWeights.stored_format(lib, folder("sixty", sixty)) == W_BF16  # 63 levels are read
+    # a header past the format's 100 MB limit (a sparse file: only the length is real)
+    big = tmp_path / "big"
+    big.mkdir()
+    with open(big / "model.safetensors", "wb") as f:
+        f.write(struct.pack("<Q", 100_000_001) + b"{")
+        f.truncate(8 + 100_000_001 + 64)
+    with pytest.raises(RuntimeError, match="longer than 100 MB"):
+        ModelWeights.stored_format(lib, big)
     # metadata is skipped, escapes in names are read
     ok = folder("ok", {"__metadata__": {"format": "pt"}, "a\\u0041.weight": {"dtype": "BF16", "shape": [2, 2], "data_offsets": [0, 8]}})
     assert ModelWeights.stored_format(lib, ok) == W_BF16

@@ -73,6 +73,27 @@ def test_gemv_equals_the_bf16_gemv_bit_for_bit(hip, oracle, N, K, kind):
         assert rel_l2(got, want) <= 1e-5
 
 
+@pytest.mark.parametrize("variant", [0, 1, 2])
+def test_gemv_follows_the_bf16_kernels_forced_split(hip, variant):
+    # A K split forced for the bf16 GEMV is the encoded GEMV's too: the two keep equal bits under any variant table.
+    lib = hip.lib
+    g = torch.Generator().manual_seed(variant)
+    try:
+        for M, N, K in [(1, 300, 2048), (4, 512, 4096), (8, 96, 1024)]:
+            w = checks.bf16x_weights(N, K, N + K, "trained").cuda()
+            enc = ops.bf16x_encode(hip, w)
+            x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+            lib.lx_tune_clear()
+            default = ops.gemv_bf16x(hip, x, w, N, entry="gemv_decode_bf16")
+            assert lib.lx_tune_force(b"gemv_w_bf16", M, N, K, variant) == 0
+            got = ops.gemv_bf16x(hip, x, enc, N)
+            plain = ops.gemv_bf16x(hip, x, w, N, entry="gemv_decode_bf16")
+            assert torch.equal(bits(got), bits(plain)), (M, N, K)
+            assert rel_l2(plain, default) <= 1e-5
+    finally:
+        lib.lx_tune_clear()
+
+
 def test_gemv_arguments(hip):
     w = checks.bf16x_weights(16, 256, 3).cuda()
     enc = ops.bf16x_encode(hip, w)

@@ -1,9 +1,14 @@
 """GPU tests of the model-folder loader (lx_ckpt_*): folders in the bf16, compressed-tensors FP8 and GPTQ NVFP4 layouts
-loaded for every target. A projection held in the file's format has the file's bytes; a converted one has the bytes the
+loaded for every target, first against the fixture that records what the reference's own loader made of the same
+folders (tests/golden/ckpt_reference.json), then rule by rule: a projection held in the file's format has the file's bytes; a converted one has the bytes the
 library's own quantiser gives the same bf16 values (the quantisers are pinned bit for bit elsewhere), the lossless target
 the bytes of lx_bf16x_encode; the products on the loaded weights run."""
 
 import ctypes
+import hashlib
+import json
+import struct
+from pathlib import Path
 
 import pytest
 import torch
@@ -55,6 +60,59 @@ def as_bf16(hip, w, fmt):
         K = rows.shape[-1] * (2 if fmt == W_NVFP4 else 1)
         outs.append(ops.dequantize(hip, Weight(fmt, rows[e], scales[e], glob), rows.shape[-2], K))
     return torch.stack(outs).reshape(*lead, *outs[0].shape)
+
+
+GOLDEN = json.loads((Path(__file__).parent / "golden" / "ckpt_reference.json").read_text())
+TARGET_OF = {"bf16": W_BF16, "int8": W_INT8, "fp8": W_FP8, "nvfp4": W_NVFP4, "bf16x": W_BF16X}
+
+
+def sha_of_device(ptr, n):
+    return hashlib.sha256(device_bytes(ptr, n).numpy().tobytes()).hexdigest() if n else None
+
+
+@pytest.mark.parametrize("case", sorted(GOLDEN["cases"]))
+def test_the_reference_loaders_formats_and_bytes(hip, tmp_path, case):
+    """Against what the reference's own loader (engine/core/checkpoint.cpp, ModelWeights::load, compiled from its sources
+    and run over its CPU backend) made of the same folders: every projection's format, shape, data, scale and global
+    bytes, the plain tensors, what skip_experts leaves readable, and the refusals' words."""
+    want = GOLDEN["cases"][case]
+    layout, _, rest = case.partition("->")
+    target, skip = TARGET_OF[rest.split()[0]], rest.endswith("skip_experts")
+    tensors = folders.write(tmp_path, layout, seed=GOLDEN["seed"], shards=1, wide=GOLDEN["wide"])
+    assert folders.digest(tensors) == GOLDEN["inputs"][layout], "this folder is not the one the fixture was made from"
+    assert ModelWeights.stored_format(hip, tmp_path) == want["stored"]
+    if "error" in want:
+        with pytest.raises(RuntimeError) as err:
+            ModelWeights.load(hip, tmp_path, target, skip)
+        assert str(err.value) == want["error"]
+        return
+    mw = ModelWeights.load(hip, tmp_path, target, skip)
+    assert mw.format() == want["format"]
+    assert sorted(mw.projection_names()) == sorted(want["projections"])
+    for name, p in want["projections"].items():
+        w, shape = mw.projection(name), mw.projection_shape(name)
+        assert w is not None and w.type == p["type"] == mw.projection_format(name), name
+        assert (shape.E, shape.N, shape.K, int(shape.stack)) == (p["E"], p["N"], p["K"], p["stack"]), name
+        assert list(mw.expert_bytes(name)) == p["expert_bytes"], name
+        assert sha_of_device(w.data, p["data_bytes"]) == p["data"], name
+        assert (w.scale is None) == (p["scale"] is None), name
+        if p["scale"]:
+            assert sha_of_device(w.scale, p["scale_bytes"]) == p["scale"], name
+        assert struct.unpack("<I", struct.pack("<f", w.global_))[0] == p["global_bits"], name
+        assert (w.expert_global is None) == (p["globals"] is None), name
+        if p["globals"]:
+            assert sha_of_device(w.expert_global, 4 * p["E"]) == p["globals"], name
+    for name, t in want["plain"].items():
+        view = mw.find(name)
+        assert view is not None and view.dtype == t["dtype"] and list(view.shape) == t["shape"], name
+        n = (2 if t["dtype"] == 1 else 4) * int(torch.tensor(t["shape"]).prod())
+        assert sha_of_device(view.data, n) == t["bytes"], name
+    for name, p in want["skipped"].items():
+        shape = mw.projection_shape(name)
+        assert (mw.projection(name) is not None) == bool(p["held"]), name
+        assert (shape.E, shape.N, shape.K, int(shape.stack)) == (p["E"], p["N"], p["K"], p["stack"]), name
+        assert list(mw.expert_bytes(name)) == p["expert_bytes"], name
+    assert mw.device_bytes() == want["device_bytes"]
 
 
 @pytest.mark.parametrize("layout", ["bf16", "fp8", "nvfp4"])

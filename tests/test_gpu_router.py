@@ -128,6 +128,18 @@ def test_experts_w8(hip, oracle, T):
     assert int(hip.size("moe_workspace_bytes", T, I, top_k)) >= int(oracle.size("moe_workspace_bytes", T, I, top_k))
 
 
+@pytest.mark.parametrize("T", [1, 5, 19])
+def test_experts_w8_more_than_eight_picks(hip, oracle, T):
+    # engine/cpu/moe.cpp:460-476 takes any top_k.
+    E, L, I, top_k = 16, 512, 256, 12
+    gu, dn = random_stack(W_INT8, E, 2 * I, L, 91), random_stack(W_INT8, E, L, I, 92)
+    latent, ids, weights = checks.make_routing(T, E, L, top_k, 93 + T)
+    out = ops.experts_w8(hip, latent.cuda(), ids.cuda(), weights.cuda(), gu.to("cuda"), dn.to("cuda"), I, top_k)
+    want = ops.experts_w8(oracle, latent, ids, weights, gu, dn, I, top_k)
+    assert rel_l2(out, want) <= 2e-3
+    checks.experts_close(out, ops.experts_reference(latent, ids, weights, gu.dense(), dn.dense()))
+
+
 @pytest.mark.parametrize("M", [1, 8, 33, 64])
 @pytest.mark.parametrize("y_dtype", [torch.float32, torch.bfloat16])
 def test_gemm_bf16(hip, oracle, M, y_dtype):
