@@ -156,23 +156,27 @@ def make_moe_case(lx, torch, fmt, T, E, L, I, top_k, seed, steps_total):
     from dromos_amd.formats import Weight
 
     g = torch.Generator(device="cpu").manual_seed(seed)
-    copies = 2 if fmt == "bf16" else 3
-    stacks = []
-    for _ in range(copies):
-        gu = (torch.randn(E, 2 * I, L, generator=g) * 0.02).to(torch.bfloat16).cuda()
-        dn = (torch.randn(E, L, I, generator=g) * 0.02).to(torch.bfloat16).cuda()
-        if fmt == "bf16":
-            stacks.append((Weight(0, gu), Weight(0, dn)))
-        else:
-            from dromos_amd.formats import alloc_quantized
+    gu = (torch.randn(E, 2 * I, L, generator=g) * 0.02).to(torch.bfloat16).cuda()
+    dn = (torch.randn(E, L, I, generator=g) * 0.02).to(torch.bfloat16).cuda()
+    if fmt == "bf16":
+        first = (Weight(0, gu), Weight(0, dn))
+    else:
+        from dromos_amd.formats import alloc_quantized
 
-            pair = []
-            for w, n, k in ((gu, 2 * I, L), (dn, L, I)):
-                out = alloc_quantized(FORMATS[fmt], E * n, k, "cuda")
-                s = out.lx()
-                lx("quantize_weight", w.view(E * n, k), ctypes.pointer(s), ctypes.c_int64(E * n), k)
-                pair.append(out)
-            stacks.append(tuple(pair))
+        pair = []
+        for w, n, k in ((gu, 2 * I, L), (dn, L, I)):
+            out = alloc_quantized(FORMATS[fmt], E * n, k, "cuda")
+            s = out.lx()
+            lx("quantize_weight", w.view(E * n, k), ctypes.pointer(s), ctypes.c_int64(E * n), k)
+            pair.append(out)
+        first = tuple(pair)
+        del gu, dn
+    # Rotating copies of the stacks at other addresses: at least four, and enough that the steps between two uses of one
+    # copy stream more than 640 MB (the Infinity Cache holds 256 MB), however few experts a step touches.
+    step_bytes = min(E, T * top_k) * (first[0].nbytes() + first[1].nbytes()) // E
+    copies = max(4, -(-(640 << 20) // step_bytes))
+    clone = lambda w: Weight(w.fmt, w.data.clone(), None if w.scale is None else w.scale.clone(), w.glob)  # noqa: E731
+    stacks = [first] + [(clone(first[0]), clone(first[1])) for _ in range(copies - 1)]
     per_expert = (stacks[0][0].nbytes() + stacks[0][1].nbytes()) // E
     n_routings = max(8, steps_total)
     logits = torch.randn(n_routings, T, E, generator=g).cuda()
@@ -269,7 +273,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--cases", default="all", choices=["headline", "gemv", "all", "layer"])
+    ap.add_argument("--cases", default="all", choices=["headline", "gemv", "all", "layer", "moe"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="no timing: one 256 MiB device copy (the counters' yardstick), then eager launches of the headline "
@@ -404,6 +408,7 @@ def main():
         run_gemv("C2 int8 M=4", "int8", 4, 14336, 4096, 1004)
         run_gemv("C2 fp8 M=4", "fp8", 4, 14336, 4096, 1004)
         run_gemv("C3 nvfp4 M=8", "nvfp4", 8, 4096, 14336, 2008)
+        run_gemv("C3 nvfp4 M=8 invariant", "nvfp4", 8, 4096, 14336, 2008, invariant=True)
     if args.cases == "all":
         for fmt in ("int8", "fp8"):
             for M in (16, 64):
@@ -438,6 +443,9 @@ def main():
         run_moe("C4 moe bf16 T=1", "bf16", 1, 64, 2048, 1024, 8, 3001)
     elif args.cases == "layer":
         run_layer()
+    elif args.cases == "moe":
+        for T in (1, 8, 32, 64):
+            run_moe(f"C4 moe bf16 T={T}", "bf16", T, 64, 2048, 1024, 8, 3000 + T)
 
     result = {
         "metric": "weight-stream GB/s and % of HBM peak: M=1 GEMV and top-8 MoE decode",
