@@ -222,7 +222,9 @@ def cpu_baseline(torch, fmt, M, N, K, seed, seconds=12.0):
     from dromos_amd.abi import DTYPE, F32, FORMATS, Kernels
     from dromos_amd.formats import Weight, master_weight, quantize_with
 
-    threads = min(16, os.cpu_count() or 1)
+    # One thread per physical core, at most the 16 a one-GPU box is given.
+    physical = physical_cores()
+    threads = min(16, physical)
     os.environ.setdefault("LX_THREADS", str(threads))
     os.environ.setdefault("OMP_NUM_THREADS", str(threads))
     ref = ROOT / "oracle" / "_ref" / "libdromos_cpu.so"
@@ -264,8 +266,22 @@ def cpu_baseline(torch, fmt, M, N, K, seed, seconds=12.0):
         "cores": threads,
         "kind": kind,
         "sample": f"{len(times)} calls of lx_gemv_w {fmt} {N}x{K} M={M} on {copies} rotated weight copies, median {med * 1e6:.0f} us/call, "
-                  f"host has {os.cpu_count()} logical cpus",
+                  f"{threads} threads; the host has {physical_cores()} physical cores ({os.cpu_count()} logical cpus)",
     }
+
+
+def physical_cores():
+    """Distinct (package, core) pairs of /proc/cpuinfo; the logical count where that file does not say."""
+    seen, package = set(), None
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("physical id"):
+                package = line.split(":")[1].strip()
+            elif line.startswith("core id"):
+                seen.add((package, line.split(":")[1].strip()))
+    except OSError:
+        pass
+    return len(seen) or (os.cpu_count() or 1)
 
 
 def main():
@@ -468,7 +484,15 @@ def main():
         "cases": cases,
     }
     if not args.no_cpu:
+        # The headline shape for about 12 s, then the other formats' M = 1 configurations for about 4 s each.
         result["cpu_baseline"] = cpu_baseline(torch, "int8", 1, 14336, 4096, 1001)
+        if result["cpu_baseline"] and args.cases in ("gemv", "all"):
+            others = {}
+            for name, fmt, N, K, seed in (("C1 bf16 M=1", "bf16", 4096, 4096, 0), ("C2 fp8 M=1", "fp8", 14336, 4096, 1001),
+                                          ("C3 nvfp4 M=1", "nvfp4", 4096, 14336, 2001)):
+                c = cpu_baseline(torch, fmt, 1, N, K, seed, seconds=4.0)
+                others[name] = {"value": c["value"], "unit": c["unit"], "sample": c["sample"]}
+            result["cpu_baseline"]["other_formats"] = others
     print(json.dumps(result))
 
 

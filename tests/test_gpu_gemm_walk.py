@@ -150,3 +150,19 @@ def test_tune_run_times_what_the_table_would_pick(hip, fmt):
     assert hip.status("tune_run", f"gemm_w_{fmt}".encode(), 99, ctypes.byref(p), out) == 801
     assert hip.status("tune_run", f"gemm_w_{fmt}".encode(), 0, ctypes.byref(TuneProblem(32, N, K, 8, 0, 0)), out) == 801  # stacks
     assert hip.status("tune_run", f"gemv_w_{fmt}".encode(), 0, ctypes.byref(TuneProblem(9, N, K, 1, 0, 0)), out) == 801  # M > 8
+
+
+def test_the_tuner_times_checks_and_stores(hip):
+    # dromos_amd/tune.py drives lx_tune_run / lx_tune_set as the engine's autotuner does (engine/cuda/tunable.h:57-75).
+    from dromos_amd import tune
+
+    try:
+        got = tune.tune(hip, "gemm_w_fp8", 32, 2048, 4096, repeats=3)
+        names = tune.variants(hip, "gemm_w_fp8")
+        assert set(got["us"]) == set(names) and all(us > 0 for us in got["us"].values())
+        assert got["pick"] in names and hip.lib.lx_tune_get(b"gemm_w_fp8", 32, 2048, 4096) == names.index(got["pick"])
+        assert got["key"].startswith("gemm_w_fp8 ")
+        split = tune.tune(hip, "gemv_w_int8", 4, 2048, 4096, repeats=3)  # the order-class rule admits one split for the shape
+        assert split["pick"] in tune.variants(hip, "gemv_w_int8")
+    finally:
+        hip.lib.lx_tune_clear()
