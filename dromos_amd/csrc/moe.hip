@@ -2,9 +2,9 @@
 // (contract: engine/cuda/kernels.h:203-209,495-507,606-611; CPU behaviour: engine/cpu/moe.cpp:163-329,343-397).
 //
 // Decode experts (T <= 8, top_k <= 8, so at most 64 (token, slot) pairs), two launches, no host round trip:
-//   gate/up   every workgroup sorts the pairs by expert in LDS (64 ids: a rank sort), takes one expert
-//             group and a block of intermediate rows, and streams gate row i and up row I + i of that
-//             expert once for all the group's tokens (stream_dot.h): inter[pair, i] = bf16(silu(g) * u).
+//   gate/up   a workgroup takes one expert's pairs (found from the step's ids with a ballot) and a block of
+//             intermediate rows, and streams gate row i and up row I + i of that expert once for all the
+//             group's tokens (stream_dot.h): inter[pair, i] = bf16(silu(g) * u).
 //   down      one workgroup per (block of output rows, token): for the token's slots in order it streams
 //             the expert's down rows against inter[pair] and adds w_k * c_k in slot order, so each output
 //             is written once and its bits depend on nothing but the token.
@@ -168,49 +168,6 @@ __global__ void __launch_bounds__(kThreads) route_kernel(const float* __restrict
   if (lane < top_k) weights[t * top_k + lane] = ex / esum;
 }
 
-// The pairs of a step with more than one token, sorted by expert (stable), as the gate/up stage reads them:
-//   table[0]                  number of groups (distinct experts)
-//   table[1 + g], g <= groups first sorted position of group g (table[1 + groups] = P)
-//   table[kTableOrder + p]    the pair at sorted position p
-//   table[kTableExpert + p]   its expert
-constexpr int kTableOrder = 2 + kMaxPairs, kTableExpert = kTableOrder + kMaxPairs, kTableInts = kTableExpert + kMaxPairs;
-constexpr int64_t kTableBytes = 1024;
-static_assert(kTableInts * 4 <= kTableBytes, "the sort table fits its part of the workspace");
-
-// One wavefront sorts the P <= 64 pairs: a pair's rank is the number of pairs with a smaller expert id, or the same
-// id and a smaller index.
-__global__ void __launch_bounds__(kWave) decode_sort_kernel(const int32_t* __restrict__ ids, int P, int* __restrict__ table) {
-  __shared__ int s_ids[kMaxPairs], s_order[kMaxPairs];
-  const int p = threadIdx.x;
-  // A lane past P holds an id above every other: it ranks behind all pairs and is never written.
-  const int mine = p < P ? ids[p] : 0x7fffffff;
-  // (id, index) as one 64-bit number: one compare a pair, all 64 lanes' numbers unrolled.
-  const uint64_t mine64 = static_cast<uint64_t>(static_cast<uint32_t>(mine)) << 32 | static_cast<uint32_t>(p);
-  int rank = 0;
-#pragma unroll
-  for (int q = 0; q < kWave; ++q) {
-    const uint64_t other = static_cast<uint64_t>(static_cast<uint32_t>(__builtin_amdgcn_readlane(mine, q))) << 32 | static_cast<uint32_t>(q);
-    rank += other < mine64;
-  }
-  if (p < P) {
-    s_ids[p] = mine;
-    s_order[rank] = p;
-  }
-  __syncthreads();
-  const bool starts = p < P && (p == 0 || s_ids[s_order[p]] != s_ids[s_order[p - 1]]);
-  const uint64_t mask = __ballot(starts);
-  const int groups = __popcll(mask);
-  if (starts) table[1 + __popcll(mask & ((1ull << p) - 1))] = p;
-  if (p == 0) {
-    table[0] = groups;
-    table[1 + groups] = P;
-  }
-  if (p < P) {
-    table[kTableOrder + p] = s_order[p];
-    table[kTableExpert + p] = s_ids[s_order[p]];
-  }
-}
-
 // One intermediate row i per wavefront (i = blockIdx.x * waves + wave) of expert e for the cnt <= MT pairs at
 // sorted positions first..: the pair (gate row i, up row I + i) is the wavefront's two streamed rows, all of
 // their loads in flight before the activations are waited for. MT only sets how many activation rows share
@@ -278,8 +235,8 @@ __device__ __forceinline__ void gate_up_rows(const DecodeArgs& a, float* lds, in
 }
 
 // grid = (I / wavefronts per workgroup, group slots); mt_cap (a power of two, the LDS image's rows) bounds a
-// pass's pairs. One token: every slot is its own group and nothing is sorted; more: the groups come from the
-// table decode_sort_kernel wrote.
+// pass's pairs. One token: every slot is its own group; more: a slot whose pair is the first of its expert takes all
+// of that expert's pairs, the other slots' workgroups leave at once.
 // ONE: a row's steps fit one batch of U.
 // SINGLE: one token (its own kernel: the many-row paths would set the registers of all).
 template <int F, int U, bool ONE, bool SINGLE>
@@ -291,21 +248,29 @@ __global__ void __launch_bounds__(kThreads) decode_gate_up_kernel(const DecodeAr
     gate_up_rows<F, U, 1, ONE>(a, lds, e, blockIdx.y, 1, nullptr, nullptr);
     return;
   }
-  __shared__ int s_rows[8];
-  if (static_cast<int>(blockIdx.y) >= a.table[0]) return;
-  const int begin = a.table[1 + blockIdx.y], end = a.table[2 + blockIdx.y];
-  const int e = a.table[kTableExpert + begin];
-  const int* const order = a.table + kTableOrder;
+  // Slot blockIdx.y of the grid is pair blockIdx.y: the workgroup goes on if no earlier pair has that pair's expert, and
+  // then takes every pair of the expert, in pair order. Each wavefront finds that from the step's ids (64 at most, one
+  // per lane) with one comparison and a ballot; nothing is sorted and no table is read.
+  __shared__ int s_rows[8], s_order[kMaxPairs];
+  const int P = a.T * a.top_k, slot = blockIdx.y;
+  if (slot >= P) return;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int id = lane < P ? a.ids[lane] : -1 - lane;  // a lane past the pairs matches nothing
+  const int e = __builtin_amdgcn_readlane(id, slot);
+  const uint64_t members = __ballot(id == e);
+  if (__ffsll(static_cast<unsigned long long>(members)) - 1 != slot) return;
+  const int total = __popcll(members);
+  if (threadIdx.x < kWave && ((members >> lane) & 1)) s_order[__popcll(members & ((1ull << lane) - 1))] = lane;
   // A group larger than the image (an expert repeated within a token) runs mt_cap pairs at a time.
-  for (int first = begin; first < end; first += mt_cap) {
-    const int cnt = min(mt_cap, end - first);
+  for (int first = 0; first < total; first += mt_cap) {
+    const int cnt = min(mt_cap, total - first);
     __syncthreads();
-    if (threadIdx.x < 8) s_rows[threadIdx.x] = static_cast<int>(threadIdx.x) < cnt ? order[first + threadIdx.x] / a.top_k : 0;
+    if (threadIdx.x < 8) s_rows[threadIdx.x] = static_cast<int>(threadIdx.x) < cnt ? s_order[first + threadIdx.x] / a.top_k : 0;
     __syncthreads();
-    if (cnt <= 1) gate_up_rows<F, U, 1, ONE>(a, lds, e, first, cnt, order, s_rows);
-    else if (cnt <= 2) gate_up_rows<F, U, 2, ONE>(a, lds, e, first, cnt, order, s_rows);
-    else if (cnt <= 4) gate_up_rows<F, U, 4, ONE>(a, lds, e, first, cnt, order, s_rows);
-    else gate_up_rows<F, U, 8, ONE>(a, lds, e, first, cnt, order, s_rows);
+    if (cnt <= 1) gate_up_rows<F, U, 1, ONE>(a, lds, e, first, cnt, s_order, s_rows);
+    else if (cnt <= 2) gate_up_rows<F, U, 2, ONE>(a, lds, e, first, cnt, s_order, s_rows);
+    else if (cnt <= 4) gate_up_rows<F, U, 4, ONE>(a, lds, e, first, cnt, s_order, s_rows);
+    else gate_up_rows<F, U, 8, ONE>(a, lds, e, first, cnt, s_order, s_rows);
   }
 }
 
@@ -506,7 +471,6 @@ int experts_decode(const void* latent, const int32_t* ids, const float* weights,
   a.gu = as_stack(gate_up);
   a.dn = as_stack(down);
   a.inter = static_cast<uint16_t*>(inter);
-  a.table = reinterpret_cast<const int*>(static_cast<const char*>(inter) + round256(2 * static_cast<int64_t>(T) * top_k * I));
   a.out = out;
   a.T = T;
   a.L = L;
@@ -522,10 +486,6 @@ int experts_decode(const void* latent, const int32_t* ids, const float* weights,
     }
   };
   int st;
-  if (T > 1 && can_stream(gate_up.type, a.gu, L)) {
-    hipLaunchKernelGGL(decode_sort_kernel, dim3(1), dim3(kWave), 0, s, ids, T * top_k, const_cast<int*>(a.table));
-    if ((st = status_of(hipGetLastError()))) return st;
-  }
   if (!can_stream(gate_up.type, a.gu, L)) {
     st = gate_up_plain(a, gate_up.type, s);
   } else {
@@ -598,8 +558,7 @@ int lx_moe_experts_decode(const void* latent, const int32_t* ids, const float* w
 
 int64_t lx_moe_decode_workspace_bytes(int T, int I, int top_k) {
   if (T <= 0 || I <= 0 || top_k <= 0) return 0;
-  // The intermediate rows, and behind them the table of the pairs sorted by expert.
-  return round256(2 * static_cast<int64_t>(T) * top_k * I) + kTableBytes;
+  return round256(2 * static_cast<int64_t>(T) * top_k * I);  // the intermediate rows
 }
 
 int64_t lx_moe_bf16x_workspace_bytes(int T, int I, int top_k) { return lx_moe_decode_workspace_bytes(T, I, top_k); }

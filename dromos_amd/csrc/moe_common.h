@@ -18,7 +18,6 @@ struct DecodeArgs {
   const float* weights;    // [T, top_k]
   Stack gu, dn;
   uint16_t* inter;  // bf16 [T * top_k, I], by pair
-  const int* table;  // the pairs sorted by expert (more than one token): see decode_sort_kernel
   float* out;       // f32 [T, L]
   int T, L, I, top_k;
 };
@@ -46,7 +45,7 @@ inline bool valid_stack(const lx_weight& w, int64_t K) {
 }
 
 // moe.hip: routing behind lx_moe_route, and the decode experts (T <= 8, top_k <= 8) on two stacks of any formats with
-// the intermediate rows and the sort table in `inter` (lx_moe_decode_workspace_bytes).
+// the intermediate rows in `inter` (lx_moe_decode_workspace_bytes).
 int route(const float* logits, const float* selection_bias, int32_t* ids, float* weights, float* entropy, float* confidence, int T,
           int E, int top_k, hipStream_t s);
 int experts_decode(const void* latent, const int32_t* ids, const float* weights, const lx_weight& gate_up, const lx_weight& down,

@@ -159,8 +159,8 @@ int lx_moe_summary_history(const int32_t* ids, const float* weights, const void*
 }
 
 // The int8 experts of the legacy entry (weight-only, any T): the decode experts' kernels, eight tokens at a time (a
-// token's bits do not depend on the tokens beside it). The workspace holds the intermediate rows and the sort table of
-// one such step.
+// token's bits do not depend on the tokens beside it). The workspace holds the intermediate rows of one such
+// step.
 int lx_moe_experts_w8(const void* latent, const int32_t* ids, const float* weights, const int8_t* gate_up, const float* gate_up_scale,
                       const int8_t* down, const float* down_scale, float* out, void* workspace, int T, int L, int I, int top_k,
                       void* stream) {
