@@ -124,132 +124,6 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) skinny_kernel(const GemmArgs
   });
 }
 
-// More than 16 activation rows: a workgroup's wavefronts own consecutive 16-row weight tiles and walk K together, one
-// weight batch (kLoadsInFlight steps) at a time. The batch's activations (M rows of the batch's k values, as bf16,
-// zero past K) are staged in LDS once for all the tiles, so they cost the memory system a fraction of the weights
-// instead of a multiple; the next batch's weights and activations are asked for before the present batch is
-// multiplied. The sums keep the order of the split kernels: each K slice (steps_per_wave steps) is an ascending
-// chain from zero, and the slices are added in ascending order, so a row's bits are those of any other M.
-constexpr int kPanelThreads = 512;
-constexpr int kPanelItems = 8;  // 16-byte pieces of x a thread stages per batch at most
-
-template <int F, int MT, bool XF32>
-__global__ void __launch_bounds__(kPanelThreads) panel_kernel(const GemmArgs a) {
-  extern __shared__ __align__(16) f32x4 lds4[];
-  constexpr int E = Fmt<F>::kElems, WU = kLoadsInFlight;
-  constexpr int kBatchElems = WU * 4 * E, kBatchVecs = kBatchElems / 8, kPitch = kBatchElems + 8;
-  const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int waves = blockDim.x / kWave;
-  const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
-  const int tile_raw = blockIdx.x * waves + wave;
-  const bool tile_live = tile_raw < n_tiles;
-  const int n0 = min(tile_raw, n_tiles - 1) * kTileRows;
-  const TileRows tiles[1] = {{a.w + n0 * a.row_bytes, a.scale + n0 * a.scale_row_bytes, min(kTileRows, a.N - n0)}};
-  uint8_t* const lds_bytes = reinterpret_cast<uint8_t*>(lds4);
-  uint16_t* const ximg = reinterpret_cast<uint16_t*>(lds_bytes + waves * kStageBytes);
-  const TileStream<F, 1> ts(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, lds_bytes + wave * kStageBytes);
-
-  // A thread's pieces of a batch's activations: item = thread + u * blockDim -> (row item / kBatchVecs, vector
-  // item % kBatchVecs). Addresses are clamped; what lies past M or K is dropped or zeroed when it is stored.
-  u32x4 xr[kPanelItems][XF32 ? 2 : 1];
-  auto x_load = [&](int tb) {
-    const int k0 = tb * 4 * E;
-#pragma unroll
-    for (int u = 0; u < kPanelItems; ++u) {
-      if (u < a.x_iters) {
-        const int item = threadIdx.x + u * blockDim.x;
-        const int m = min(item / kBatchVecs, a.M - 1), k = min(k0 + (item % kBatchVecs) * 8, a.K - 8);
-        const char* src = static_cast<const char*>(a.xs.x) + (static_cast<int64_t>(m) * a.xs.ld + k) * (XF32 ? 4 : 2);
-        xr[u][0] = *reinterpret_cast<const u32x4*>(src);
-        if constexpr (XF32) xr[u][1] = *reinterpret_cast<const u32x4*>(src + 16);
-      }
-    }
-  };
-  auto x_store = [&](int tb) {
-    const int k0 = tb * 4 * E;
-#pragma unroll
-    for (int u = 0; u < kPanelItems; ++u) {
-      if (u < a.x_iters) {
-        const int item = threadIdx.x + u * blockDim.x;
-        const int m = item / kBatchVecs, v = item % kBatchVecs;
-        if (m < a.M) {
-          u32x4 val = xr[u][0];
-          if constexpr (XF32) {
-            bf16x2 q[4] = {pack_bf16(__uint_as_float(xr[u][0].x), __uint_as_float(xr[u][0].y)),
-                           pack_bf16(__uint_as_float(xr[u][0].z), __uint_as_float(xr[u][0].w)),
-                           pack_bf16(__uint_as_float(xr[u][1].x), __uint_as_float(xr[u][1].y)),
-                           pack_bf16(__uint_as_float(xr[u][1].z), __uint_as_float(xr[u][1].w))};
-            val = __builtin_bit_cast(u32x4, q);
-          }
-          if (k0 + v * 8 >= a.K) val = u32x4{0u, 0u, 0u, 0u};
-          *reinterpret_cast<u32x4*>(ximg + m * kPitch + v * 8) = val;
-        }
-      }
-    }
-  };
-
-  x_load(0);
-  WeightBatch<F, 1> wa, wb;
-  ts.issue(wa, 0);
-  // The epilogue's row factors and f32 biases: a lane always finishes the same four weight rows.
-  const bool bias_f32 = a.bias && a.bias_dtype == LX_F32;
-  float rf[4], bs[4];
-  {
-    const int nq = n0 + 4 * (lane >> 4);
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-      const int n = min(nq + r, a.N - 1);
-      rf[r] = row_factor(F, a.scale, a.global, n);
-      bs[r] = bias_f32 ? static_cast<const float*>(a.bias)[n] : 0.0f;
-    }
-  }
-  const uint16_t* xrow0[MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) xrow0[mt] = ximg + min(mt * 16 + (lane & 15), a.M - 1) * kPitch;
-
-  f32x4 total[1][MT], acc[1][MT];
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) total[0][mt] = acc[0][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  const int steps = a.steps, spw = a.steps_per_wave;
-  // One batch: store its activations, ask for the next batch's, multiply.
-  auto half = [&](const WeightBatch<F, 1>& cur, WeightBatch<F, 1>& next, int tb) {
-    __syncthreads();  // every wavefront has read the previous image
-    x_store(tb);
-    if (tb + WU < steps) {
-      x_load(tb + WU);
-      ts.issue(next, tb + WU);
-    }
-    __syncthreads();
-    const void* xrow[MT];
-#pragma unroll
-    for (int mt = 0; mt < MT; ++mt) xrow[mt] = xrow0[mt] - tb * 4 * E;  // the image starts at the batch's first k
-    ts.template consume<MT, kXLds>(cur, tb, xrow, a.K, a.K, acc);
-    if ((tb + WU) % spw == 0 || tb + WU >= steps) {  // the slice ends: add it to the slices before it
-      const bool first = tb + WU <= spw;
-#pragma unroll
-      for (int mt = 0; mt < MT; ++mt) {
-        total[0][mt] = first ? acc[0][mt] : total[0][mt] + acc[0][mt];
-        acc[0][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-      }
-    }
-  };
-  for (int tb = 0; tb < steps; tb += 2 * WU) {
-    half(wa, wb, tb);
-    if (tb + WU < steps) half(wb, wa, tb + WU);
-  }
-  if (!tile_live) return;
-#pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    const int m = mt * 16 + (lane & 15), nq = n0 + 4 * (lane >> 4);
-    if (m < a.M) {
-#pragma unroll
-      for (int r = 0; r < 4; ++r)
-        if (nq + r < a.N)
-          write_out(a, m, nq + r, total[0][mt][r], rf[r], bias_f32 || !a.bias ? bs[r] : load_as_f32(a.bias, a.bias_dtype, nq + r));
-    }
-  }
-}
-
 // ---- up to 16 activation rows: the lean tile kernel ------------------------------------------------------
 //
 // The same arithmetic as skinny_kernel (one 16 x 16 tile per S wavefronts, contiguous K slices of
@@ -1315,15 +1189,27 @@ bool try_walk(const GemmArgs& a, int* status, hipStream_t stream) {
   if (tuned >= 1 && tuned <= 3) {
     W = 1 << (tuned - 1);
   } else {
-    // A walk of 32 groups (bf16 at K = 4096) pays only at the largest batches: 14336 x 4096 bf16 at 64 rows 39.3 -> 35.3 us,
-    // at 32 rows 29.8 -> 31.5.
-    if (a.M <= 8 || n_tiles < 192 || a.steps > (a.M > 48 && n_tiles >= 512 ? 128 : 64)) return false;
-    W = n_tiles >= 512 ? 4 : 2;
+    // From sweeps of every variant (16 / 32 / 48 / 64 rows): a walk of at most 16 groups wins from 9 rows on; longer walks
+    // (bf16, K >= 8192) win once the batch is large, where the tile kernels' activation reads grow with every row tile:
+    // 8192 x 8192 fp8 at 32 / 64 rows 28.4 -> 24.6 / 50.4 -> 39.4 us, bf16 40.6 -> 36.7 / 58.8 -> 43.4 us, 14336 x 4096 bf16
+    // at 64 rows 39.3 -> 35.3 us, 14336 x 8192 fp8 at 48 rows 47.5 -> 41.6 us. Few tiles (4096 rows) stay with the tile kernels.
+    const int walk_groups = a.steps >> 2;
+    if (a.M <= 8 || n_tiles < 192) return false;
+    if (walk_groups > 16) {
+      if (n_tiles < 512 || walk_groups > 64) return false;
+      if (a.M <= (n_tiles >= 768 ? 32 + 8 : 24)) return false;  // many tiles: the windowed kernel holds on to 40 rows
+    }
+    W = n_tiles >= (walk_groups <= 16 ? 512 : 768) ? 4 : 2;
   }
-  if constexpr (F == LX_W_BF16) return launch_walk_bf16(a, W, status, stream);
-  else if constexpr (F == LX_W_INT8) return launch_walk_int8(a, W, status, stream);
-  else if constexpr (F == LX_W_FP8) return launch_walk_fp8(a, W, status, stream);
-  else return launch_walk_nvfp4(a, W, status, stream);
+  auto launch = [&](int w) {
+    if constexpr (F == LX_W_BF16) return launch_walk_bf16(a, w, status, stream);
+    else if constexpr (F == LX_W_INT8) return launch_walk_int8(a, w, status, stream);
+    else if constexpr (F == LX_W_FP8) return launch_walk_fp8(a, w, status, stream);
+    else return launch_walk_nvfp4(a, w, status, stream);
+  };
+  if (launch(W)) return true;
+  // The rule's two tiles a workgroup can be too many staging registers a lane (NVFP4 from 33 rows): four tiles then.
+  return tuned < 0 && W == 2 && launch(4);
 }
 
 template <int F, int MT>
@@ -1362,31 +1248,6 @@ int launch_skinny(GemmArgs a, hipStream_t stream) {
       const unsigned grid = (n_tiles + tiles_per_wg - 1) / tiles_per_wg;
       return a.xs.dtype == LX_F32 ? launch_skinny_x<F, 1, true, true>(a, lds, grid, threads, stream)
                                   : launch_skinny_x<F, 1, false, true>(a, lds, grid, threads, stream);
-    }
-  }
-  if constexpr (MT > 1) {
-    // The panel kernel, when a batch's activations fit LDS and a thread's share of them its registers.
-    constexpr int kBatchElems = kLoadsInFlight * 4 * Fmt<F>::kElems;
-    const int waves = kPanelThreads / kWave;
-    const size_t lds = static_cast<size_t>(waves) * kStageBytes + static_cast<size_t>(a.M) * (kBatchElems + 8) * 2;
-    a.x_iters = (a.M * (kBatchElems / 8) + kPanelThreads - 1) / kPanelThreads;
-    // It needs many tiles: with fewer than 96 workgroups most compute units would idle and the split kernel, one tile
-    // to a workgroup, does better.
-    if (lds <= kLdsMax && a.x_iters <= kPanelItems && a.steps_per_wave % kLoadsInFlight == 0 && n_tiles >= 96u * waves) {
-      const unsigned grid = (n_tiles + waves - 1) / waves;
-      auto launch = [&](auto kernel) {
-        if (lds > 48 * 1024) {
-          static thread_local bool raised = false;
-          if (!raised) {
-            if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, kLdsMax) != hipSuccess)
-              (void)hipGetLastError();
-            raised = true;
-          }
-        }
-        hipLaunchKernelGGL(kernel, dim3(grid), dim3(kPanelThreads), lds, stream, a);
-        return status_of(hipGetLastError());
-      };
-      return a.xs.dtype == LX_F32 ? launch(panel_kernel<F, MT, true>) : launch(panel_kernel<F, MT, false>);
     }
   }
   const size_t lds = tile_lds_bytes(S, 1, MT);

@@ -28,7 +28,7 @@ struct GemmArgs {
   float alpha, beta;
   int chunks, steps, steps_per_wave, S;
   int64_t row_bytes, scale_row_bytes;
-  int tiles_per_wg, x_vecs, x_row_vecs, x_pitch, x_iters;  // the LDS activation image (XL and panel kernels)
+  int tiles_per_wg, x_vecs, x_row_vecs, x_pitch, x_iters;  // the LDS activation image (XL kernels)
   int x_phased;  // lean kernel with two slices a wavefront: the image holds half of K at a time
   int win;       // windowed kernel: load steps of every slice the image holds at a time (2, 4 or 8)
   int win_steps_shift, win_shift, row_shift;  // log2 of win, of the 16-byte pieces in a window, and in an image row

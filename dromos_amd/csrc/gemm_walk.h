@@ -35,7 +35,10 @@ namespace walk {
 template <int N>
 using Tag = std::integral_constant<int, N>;
 
-template <int F, int MT, int W>
+// ROT: the workgroups start at different slices (see above) and a wavefront keeps every slice's sum in LDS until the end;
+// without it every workgroup starts at slice 0 and the sums are added as the slices end, in registers: the form for
+// shapes whose images leave no room for the sums.
+template <int F, int MT, int W, bool ROT>
 __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
   constexpr int E = Fmt<F>::kElems, J = E / 8;
@@ -54,7 +57,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   uint8_t* const img = lds + W * 4096;  // + buffer * kImage
   const int groups = a.steps >> 2, last = groups - 1;  // groups of four load steps in a row
   const int gps = a.steps_per_wave >> 2;               // groups of a slice
-  const int first_slice = blockIdx.x % a.S, rot = first_slice * gps;
+  const int first_slice = ROT ? blockIdx.x % a.S : 0, rot = first_slice * gps;
   // The l-th group this workgroup takes (l past the end repeats the last one).
   auto group_of = [&](int l) {
     const int gq = min(l, last) + rot;
@@ -153,6 +156,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   f32x4* const sums = reinterpret_cast<f32x4*>(img + 2 * kImage) + wave * (a.S * MT * kWave) + lane;  // [slice][mt][lane]
+  f32x4 total[MT];
   int slice_end = gps, slice = first_slice;
 
   // The gamma-th group the workgroup takes (its fragments are in wv).
@@ -210,7 +214,8 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
     if (gamma + 1 == slice_end) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        sums[(slice * MT + mt) * kWave] = acc[mt];
+        if constexpr (ROT) sums[(slice * MT + mt) * kWave] = acc[mt];
+        else total[mt] = slice == 0 ? acc[mt] : total[mt] + acc[mt];
         acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
       slice_end += gps;
@@ -226,11 +231,12 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
 
   // The slices' sums in ascending order (the wavefront reads what it wrote itself: LDS keeps its order).
   asm volatile("" ::: "memory");
-  f32x4 total[MT];
+  if constexpr (ROT) {
 #pragma unroll
-  for (int mt = 0; mt < MT; ++mt) {
-    total[mt] = sums[mt * kWave];
-    for (int sl = 1; sl < a.S; ++sl) total[mt] += sums[(sl * MT + mt) * kWave];
+    for (int mt = 0; mt < MT; ++mt) {
+      total[mt] = sums[mt * kWave];
+      for (int sl = 1; sl < a.S; ++sl) total[mt] += sums[(sl * MT + mt) * kWave];
+    }
   }
 
   if (tile >= n_tiles) return;
@@ -270,18 +276,27 @@ template <int F, int W>
 int launch_w(const GemmArgs& a, unsigned grid, hipStream_t stream) {
   constexpr int J = Fmt<F>::kElems / 8, PB = 4 * J;
   const int MT = (a.M + 15) / 16;
-  const size_t lds = static_cast<size_t>(W) * 4096 + 2 * static_cast<size_t>(MT) * 4 * PB * 256 + static_cast<size_t>(W) * a.S * MT * kWave * 16;
+  // A lane holds 2 MT 4 J / W staging pieces of 16 bytes: past 32 of them the kernel spills (measured 4 .. 20 x slower).
+  if (MT * 4 * J / W > 16) return kNotSupported;
+  const size_t images = static_cast<size_t>(W) * 4096 + 2 * static_cast<size_t>(MT) * 4 * PB * 256;
+  const size_t with_sums = images + static_cast<size_t>(W) * a.S * MT * kWave * 16;
+  const bool rot = with_sums <= kLdsMax;
+  const size_t lds = rot ? with_sums : images;
   if (lds > kLdsMax) return kNotSupported;
   auto launch = [&](auto kernel) {
     if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), kLdsMax);
     hipLaunchKernelGGL(kernel, dim3(grid), dim3(W * kWave), lds, stream, a);
     return status_of(hipGetLastError());
   };
-  switch (MT) {
-    case 1: return launch(walk_kernel<F, 1, W>);
-    case 2: return launch(walk_kernel<F, 2, W>);
-    case 3: return launch(walk_kernel<F, 3, W>);
-    default: return launch(walk_kernel<F, 4, W>);
+  switch (MT * 2 + (rot ? 1 : 0)) {
+    case 3: return launch(walk_kernel<F, 1, W, true>);
+    case 5: return launch(walk_kernel<F, 2, W, true>);
+    case 7: return launch(walk_kernel<F, 3, W, true>);
+    case 9: return launch(walk_kernel<F, 4, W, true>);
+    case 2: return launch(walk_kernel<F, 1, W, false>);
+    case 4: return launch(walk_kernel<F, 2, W, false>);
+    case 6: return launch(walk_kernel<F, 3, W, false>);
+    default: return launch(walk_kernel<F, 4, W, false>);
   }
 }
 
