@@ -602,7 +602,8 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
   using Acc = typename std::conditional<MATH == LX_MATH_INT8, i32x4, f32x4>::type;
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
   const int waves = blockDim.x / kWave;
-  const int S = a.S, w = blockIdx.y, spw = a.steps_per_wave, t_begin = w * spw;
+  // This launch takes steps [pass_begin, pass_begin + pass_steps) of every slice (the whole slice where its image fits).
+  const int S = a.S, w = blockIdx.y, spw = a.pass_steps, t_begin = w * a.steps_per_wave + a.pass_begin;
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
   const int tile_first = blockIdx.x * a.tiles_per_wg, tile_end = min(n_tiles, tile_first + a.tiles_per_wg);
   const int g = lane >> 4, i = lane & 15;
@@ -699,9 +700,11 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
   for (; tile < tile_end; tile += waves) {
     const int next_tile = tile + waves;
     const TilePtrs next = ptrs_of(next_tile < tile_end ? next_tile : tile);
+    // A slice taken in several launches goes on from where the launch before left its chain (the partial tile).
+    Acc* const part = static_cast<Acc*>(a.partial) + ((static_cast<int64_t>(w) * n_tiles + tile) * MT) * kWave + lane;
     Acc acc[MT];
 #pragma unroll
-    for (int mt = 0; mt < MT; ++mt) acc[mt] = Acc{0, 0, 0, 0};
+    for (int mt = 0; mt < MT; ++mt) acc[mt] = a.pass_continues ? part[mt * kWave] : Acc{0, 0, 0, 0};
     for (int off = 0; off < spw; off += 8) {
 #pragma unroll
       for (int grp = 0; grp < 2; ++grp) {
@@ -743,13 +746,12 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) slab_kernel(const GemmArgs a
     }
     // The tile's slice is done: the partial tile, or with one slice the result itself.
     const int nq = tile * kTileRows + 4 * g;
-    if (S > 1) {
+    if (a.partial) {
       // Partial tiles lie as the wavefront holds them: [slice][tile][16 activation rows][lane] vectors of four words, so a
       // store instruction writes 1 KB of whole cache lines (rows of the output would be 64-byte halves of lines, which
       // the cache has to fetch first).
-      Acc* const out = static_cast<Acc*>(a.partial) + ((static_cast<int64_t>(w) * n_tiles + tile) * MT) * kWave + lane;
 #pragma unroll
-      for (int mt = 0; mt < MT; ++mt) out[mt * kWave] = acc[mt];
+      for (int mt = 0; mt < MT; ++mt) part[mt * kWave] = acc[mt];
     } else {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
@@ -867,7 +869,14 @@ bool launch_slab(GemmArgs a, int* status, hipStream_t stream) {
   if (spw % 8 != 0 || S < 1) return false;
   const bool xf32 = !I8 && a.xs.dtype == LX_F32;
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
-  const size_t pitch = static_cast<size_t>(spw) * SB + 16;
+  // A slice whose image does not fit LDS is taken in several launches of `part` steps each (whole batches of eight): a
+  // launch leaves its chains in the partial tiles and the next one goes on from them, so the sums are those of one pass.
+  int part = spw;
+  while (part > 8 && static_cast<size_t>(a.M) * (static_cast<size_t>(part) * SB + 16) + 16 > kLdsMax - 1024) part -= 8;
+  const int passes = (spw + part - 1) / part;
+  if (passes > 1 && S == 1) return false;  // the chain is handed on through the partial tiles, which one slice has none of
+  if (passes > 3) return false;
+  const size_t pitch = static_cast<size_t>(part) * SB + 16;
   const size_t image = static_cast<size_t>(a.M) * pitch + 16;
   // One slab per compute unit and slice round: tiles_per_wg tiles of one slice, up to sixteen wavefronts on them.
   const int slabs = compute_units() / S > 0 ? compute_units() / S : 1;
@@ -886,10 +895,6 @@ bool launch_slab(GemmArgs a, int* status, hipStream_t stream) {
   a.tiles_per_wg = tpw;
   a.x_vecs = a.K * (I8 ? 1 : 2) / 16;
   a.x_pitch = static_cast<int>(pitch);
-  const int row_pieces = spw * (SB / 16);
-  a.row_shift = -1;
-  for (int sh = 0; sh < 20; ++sh)
-    if ((1 << sh) == row_pieces) a.row_shift = sh;
   const dim3 grid((n_tiles + tpw - 1) / tpw, S);
   auto launch = [&](auto kernel) {
     if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), kLdsMax);
@@ -901,12 +906,21 @@ bool launch_slab(GemmArgs a, int* status, hipStream_t stream) {
     if constexpr (I8) return launch(slab_kernel<F, MATH, false, MT>);
     else return xf32 ? launch(slab_kernel<F, MATH, true, MT>) : launch(slab_kernel<F, MATH, false, MT>);
   };
-  int st;
-  switch ((a.M + 15) / 16) {
-    case 1: st = with_mt(std::integral_constant<int, 1>{}); break;
-    case 2: st = with_mt(std::integral_constant<int, 2>{}); break;
-    case 3: st = with_mt(std::integral_constant<int, 3>{}); break;
-    default: st = with_mt(std::integral_constant<int, 4>{}); break;
+  int st = kOk;
+  for (int begin = 0; begin < spw && !st; begin += part) {
+    a.pass_begin = begin;
+    a.pass_steps = spw - begin < part ? spw - begin : part;
+    a.pass_continues = begin > 0;
+    const int row_pieces = a.pass_steps * (SB / 16);
+    a.row_shift = -1;
+    for (int sh = 0; sh < 20; ++sh)
+      if ((1 << sh) == row_pieces) a.row_shift = sh;
+    switch ((a.M + 15) / 16) {
+      case 1: st = with_mt(std::integral_constant<int, 1>{}); break;
+      case 2: st = with_mt(std::integral_constant<int, 2>{}); break;
+      case 3: st = with_mt(std::integral_constant<int, 3>{}); break;
+      default: st = with_mt(std::integral_constant<int, 4>{}); break;
+    }
   }
   if (!st && S > 1) {
     const int mts = (a.M + 15) / 16;

@@ -35,6 +35,7 @@ struct GemmArgs {
   const int8_t* xq;     // the INT8 math: quantised activations [M, K], rows K bytes apart
   const float* xscale;  // and their per-row scales
   const float* act_scale;  // BF16-math kernels on a quantised math's activation images: the rows' scales (else null)
+  int pass_begin, pass_steps, pass_continues;  // slab kernel: the part of every slice this launch takes, and whether it goes on from `partial`
   void* partial;  // slab kernel with S > 1: the slices' partial tiles, [S][tile][16 rows][lane] x 4 words (f32, or i32 for the INT8 math)
 };
 

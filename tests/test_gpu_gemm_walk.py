@@ -166,3 +166,26 @@ def test_the_tuner_times_checks_and_stores(hip):
         assert split["pick"] in tune.variants(hip, "gemv_w_int8")
     finally:
         hip.lib.lx_tune_clear()
+
+
+@pytest.mark.parametrize("fmt,N,K", [("fp8", 4096, 14336), ("nvfp4", 4096, 14336), ("bf16", 4096, 14336)])
+def test_long_slices_in_several_slab_passes(hip, fmt, N, K):
+    # Rows whose slices are too long for one LDS image: the slab kernel takes a slice in two or three launches, each going
+    # on from the partial tiles of the one before; the sums are the one-pass chain's, bit for bit the other kernels'.
+    w = random_weight(FORMATS[fmt], N, K, N + K)
+    g = torch.Generator().manual_seed(K)
+    wd = w.to("cuda")
+    dense = w.dense()
+    for M in (33, 64):
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        outs = {}
+        for variant in (0, 4, 5, None):
+            force(hip, fmt, M, N, K, variant)
+            outs[variant] = ops.gemm_w(hip, x.cuda(), wd, MATH_BF16).clone()
+        checks.check_product(outs[5].cpu(), ops.gemv_reference(x, dense, None, 1.0, 0.0, None))
+        for variant, out in outs.items():
+            assert torch.equal(out.view(torch.int32), outs[4].view(torch.int32)), f"variant {variant} at {fmt} M={M}"
+        # a row's bits are those of the row alone
+        force(hip, fmt, 1, N, K, None)
+        alone = ops.gemm_skinny(hip, x[M - 1 : M].cuda(), wd)
+        assert torch.equal(alone[0].view(torch.int32), outs[None][M - 1].view(torch.int32))
