@@ -293,7 +293,7 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="no timing: one 256 MiB device copy (the counters' yardstick), then eager launches of the headline "
-                         "GEMV, the 16- and 64-row products, the one-token experts and the 32-token grouped experts")
+                         "GEMV, the 16- and 64-row products, the one- and eight-token experts and the 32-token grouped experts")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this path runs on one GPU; --gpus N with N > 1 is not supported (one MI355X per box)")
@@ -324,7 +324,7 @@ def main():
         del keep
         for M in (16, 64):
             step, nbytes, keep = make_gemv_case(lx, torch, "int8", M, 14336, 4096, 1000 + M, "gemm_w")
-            launches(f"C2 int8 M={M} (window_kernel)", step, nbytes, 10)
+            launches(f"C2 int8 M={M} (walk_kernel)", step, nbytes, 10)
             del keep
         os.environ["LX_BATCH_INVARIANT"] = "1"
         step, nbytes, keep = make_gemv_case(lx, torch, "int8", 4, 14336, 4096, 1004, "gemv_w")
@@ -337,6 +337,10 @@ def main():
         torch.cuda.empty_cache()
         step, nbytes, keep, _ = make_moe_case(lx, torch, "bf16", 1, 64, 2048, 1024, 8, 3001, 16)
         launches("C4 moe bf16 T=1 (route + decode_gate_up + decode_down)", step, nbytes, 16)
+        del keep
+        torch.cuda.empty_cache()
+        step, nbytes, keep, _ = make_moe_case(lx, torch, "bf16", 8, 64, 2048, 1024, 8, 3008, 8)
+        launches("C4 moe bf16 T=8 (route + decode_gate_up + decode_down)", step, nbytes, 8)
         del keep
         torch.cuda.empty_cache()
         step, nbytes, keep, _ = make_moe_case(lx, torch, "fp8", 32, 128, 4096, 1536, 8, 5032, 8)
