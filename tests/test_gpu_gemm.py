@@ -314,6 +314,62 @@ def test_slab_forced_equals_the_windowed_kernel(hip, fmt, M, N, K):
         assert torch.equal(a.view(torch.int32), b.view(torch.int32)), x_dtype
 
 
+def test_streams_with_and_without_the_partial_sum_buffer(hip):
+    """The slab kernel's partial tiles belong to the stream (lx_rt_stream_create makes them, a host with its own streams
+    calls lx_rt_stream_reserve): a product allocates nothing, and a stream without the buffer takes another kernel with
+    the same bits, eagerly and under graph capture alike."""
+    import ctypes
+
+    M, N, K = 64, 4096, 8192  # a shape the rule sends to the slab kernel
+    g = torch.Generator().manual_seed(31)
+    w = random_weight(FORMATS["fp8"], N, K, 7).to("cuda")
+    x = torch.randn(M, K, generator=g).to(torch.bfloat16).cuda()
+    lib = hip.lib
+    plain, owned = torch.cuda.Stream(), torch.cuda.Stream()
+    assert lib.lx_rt_stream_reserve(ctypes.c_void_p(owned.cuda_stream)) == 0
+    assert lib.lx_rt_stream_reserve(ctypes.c_void_p(owned.cuda_stream)) == 0  # once is enough, twice is no error
+    made = ctypes.c_void_p()
+    assert lib.lx_rt_stream_create(ctypes.byref(made)) == 0
+    try:
+        y = torch.full((M, N), float("nan"), device="cuda")
+        wl = w.lx()
+        # Once before the memory is looked at: torch's allocator takes its blocks for the outputs and the runtime sets up
+        # each stream's queue on its first launch.
+        for s in (plain, owned):
+            with torch.cuda.stream(s):
+                ops.gemm_w(hip, x, w, MATH_BF16)
+        assert lib.lx_gemm_w(x.data_ptr(), 1, K, ctypes.byref(wl), MATH_BF16, None, 0, y.data_ptr(), 0, N, M, N, K, 1.0, 0.0, None, made) == 0
+        torch.cuda.synchronize()
+        y.fill_(float("nan"))
+        torch.cuda.synchronize()
+        free0 = torch.cuda.mem_get_info()[0]
+        outs = []
+        for s in (plain, owned):
+            with torch.cuda.stream(s):
+                outs.append(ops.gemm_w(hip, x, w, MATH_BF16))
+        assert lib.lx_gemm_w(x.data_ptr(), 1, K, ctypes.byref(wl), MATH_BF16, None, 0, y.data_ptr(), 0, N, M, N, K, 1.0, 0.0, None, made) == 0
+        assert lib.lx_rt_stream_sync(made) == 0
+        assert torch.equal(outs[0].view(torch.int32), outs[1].view(torch.int32)) and torch.equal(y.view(torch.int32), outs[0].view(torch.int32))
+        assert torch.cuda.mem_get_info()[0] == free0, "a product allocated device memory"
+        # under capture on the stream that owns a buffer: the same result on every replay
+        graph = ctypes.c_void_p()
+        y2 = torch.zeros(M, N, device="cuda")
+        assert lib.lx_rt_capture_begin(made) == 0
+        assert lib.lx_gemm_w(x.data_ptr(), 1, K, ctypes.byref(wl), MATH_BF16, None, 0, y2.data_ptr(), 0, N, M, N, K, 1.0, 0.0, None, made) == 0
+        assert lib.lx_rt_capture_end(made, ctypes.byref(graph)) == 0
+        for _ in range(3):
+            y2.zero_()
+            torch.cuda.synchronize()
+            assert lib.lx_rt_graph_launch(graph, made) == 0 and lib.lx_rt_stream_sync(made) == 0
+            assert torch.equal(y2.view(torch.int32), outs[0].view(torch.int32))
+        assert lib.lx_rt_graph_destroy(graph) == 0
+    finally:
+        torch.cuda.synchronize()
+        assert lib.lx_rt_stream_release(ctypes.c_void_p(owned.cuda_stream)) == 0
+        assert lib.lx_rt_stream_release(ctypes.c_void_p(owned.cuda_stream)) == 0  # nothing left: no error
+        assert lib.lx_rt_stream_destroy(made) == 0
+
+
 @pytest.mark.parametrize("math,fmt", [(MATH_INT8, "int8"), (MATH_FP8, "fp8")])
 def test_slab_under_the_byte_maths(hip, oracle, math, fmt):
     M, N, K = 64, 6144, 4096
