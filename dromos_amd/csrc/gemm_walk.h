@@ -66,16 +66,28 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
 
   // Staging: item idx = (tile of rows * 4 + step of the window) * J + quad of pieces; wavefront tw takes
   // items tw, tw + W, ... A lane's piece of an item: row 4 (lane / 16) + (lane % 16) / 4, piece lane % 4 of the quad.
+  // (J == 2, the one-byte formats: an item is instead eight rows of a whole step, lane (g, i) holding row 8 h + i / 2,
+  // piece 2 g + i % 2, and a piece's rows are rotated by eight slots on odd pieces: writes and reads both touch every
+  // bank once, and the four 16-lane groups of a fragment read, whose pieces are all even or all odd, share one rotation,
+  // which is what the LDS serves at full rate.)
   const int r = 4 * g + (i >> 2), e3 = i & 3;
   const uint32_t lds_lane = e3 * 256 + ((r + 4 * e3) & 15) * 16;
   const char* const xbase = static_cast<const char*>(a.xs.x);
   const uint32_t ld_bytes = static_cast<uint32_t>(a.xs.ld) * 2u;
   uint32_t x_off[Q];  // byte offset of this lane's piece of item `it` within window 0
+  uint32_t x_lds[J == 2 ? Q : 1];  // J == 2: where it goes in an image
 #pragma unroll
   for (int it = 0; it < Q; ++it) {
     const int idx = tw + it * W;
-    const int pq = idx & (J - 1), u = (idx / J) & 3, mt = idx / (4 * J);
-    x_off[it] = static_cast<uint32_t>(min(16 * mt + r, a.M - 1)) * ld_bytes + static_cast<uint32_t>(u * 4 * E + pq * 32 + e3 * 8) * 2u;
+    if constexpr (J == 2) {
+      const int h = idx & 1, u = (idx >> 1) & 3, mt = idx >> 3;
+      const int row = 8 * h + (i >> 1), piece = 2 * g + (i & 1);
+      x_off[it] = static_cast<uint32_t>(min(16 * mt + row, a.M - 1)) * ld_bytes + static_cast<uint32_t>(u * 4 * E + piece * 8) * 2u;
+      x_lds[it] = static_cast<uint32_t>(((mt * 4 + u) * PB + piece) * 256 + ((row + 8 * (piece & 1)) & 15) * 16);
+    } else {
+      const int pq = idx & (J - 1), u = (idx / J) & 3, mt = idx / (4 * J);
+      x_off[it] = static_cast<uint32_t>(min(16 * mt + r, a.M - 1)) * ld_bytes + static_cast<uint32_t>(u * 4 * E + pq * 32 + e3 * 8) * 2u;
+    }
   }
   u32x4 xr[2][Q];  // two windows on their way
   auto stage_load = [&](auto set, int gamma) {
@@ -84,9 +96,15 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
     for (int it = 0; it < Q; ++it) xr[decltype(set)::value][it] = *reinterpret_cast<const u32x4*>(src + x_off[it]);
   };
   auto stage_store = [&](auto set, int gamma) {
-    uint8_t* const dst = img + (gamma & 1) * kImage + tw * 1024 + lds_lane;
+    if constexpr (J == 2) {
+      uint8_t* const dst = img + (gamma & 1) * kImage;
 #pragma unroll
-    for (int it = 0; it < Q; ++it) *reinterpret_cast<u32x4*>(dst + it * (W * 1024)) = xr[decltype(set)::value][it];
+      for (int it = 0; it < Q; ++it) *reinterpret_cast<u32x4*>(dst + x_lds[it]) = xr[decltype(set)::value][it];
+    } else {
+      uint8_t* const dst = img + (gamma & 1) * kImage + tw * 1024 + lds_lane;
+#pragma unroll
+      for (int it = 0; it < Q; ++it) *reinterpret_cast<u32x4*>(dst + it * (W * 1024)) = xr[decltype(set)::value][it];
+    }
   };
 
   // This lane's weight loads: rows 4 q + g of the tile, chunk i of a group (256 contiguous bytes per 16 lanes).
@@ -149,7 +167,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   // A fragment read: piece g * J + j of the step, this lane's row i of the activation tile.
   uint32_t rd_lane[J];
 #pragma unroll
-  for (int j = 0; j < J; ++j) rd_lane[j] = (g * J + j) * 256 + ((i + 4 * ((g * J + j) & 3)) & 15) * 16;
+  for (int j = 0; j < J; ++j) rd_lane[j] = (g * J + j) * 256 + ((i + (J == 2 ? 8 * j : 4 * ((g * J + j) & 3))) & 15) * 16;
 
   // The slice at hand; a finished slice's sum waits in the wavefront's own area behind the images.
   f32x4 acc[MT];
