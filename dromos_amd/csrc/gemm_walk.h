@@ -240,12 +240,26 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
       slice = slice + 1 == a.S ? 0 : slice + 1;
     }
   };
-  for (int gamma = 0; gamma < groups; gamma += 4) {
+  for (int gamma = 0; gamma < groups - 4; gamma += 4) {
     one_group(Tag<0>{}, gamma);
     one_group(Tag<1>{}, gamma + 1);
     one_group(Tag<2>{}, gamma + 2);
     one_group(Tag<3>{}, gamma + 3);
   }
+  // The last four groups, with the epilogue's row factors and biases asked for one group before the end: at the end they
+  // would be a memory latency nothing hides, and asked for at the start they would hold registers through the walk.
+  one_group(Tag<0>{}, groups - 4);
+  one_group(Tag<1>{}, groups - 3);
+  one_group(Tag<2>{}, groups - 2);
+  const int nq = n0 + 4 * g;
+  float rf[4], bs[4];
+#pragma unroll
+  for (int rr = 0; rr < 4; ++rr) {
+    const int n = min(nq + rr, a.N - 1);
+    rf[rr] = row_factor(F, a.scale, a.global, n);
+    bs[rr] = a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f;
+  }
+  one_group(Tag<3>{}, groups - 1);
 
   // The slices' sums in ascending order (the wavefront reads what it wrote itself: LDS keeps its order).
   asm volatile("" ::: "memory");
@@ -259,15 +273,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
 
   if (tile >= n_tiles) return;
   // A lane holds four consecutive outputs of one activation row: one 16-byte store where y allows it.
-  const int nq = n0 + 4 * g;
   const bool wide = a.y_dtype == LX_F32 && a.beta == 0.0f && nq + 3 < a.N && (a.ld_y & 3) == 0 && (reinterpret_cast<uintptr_t>(a.y) & 15) == 0;
-  float rf[4], bs[4];
-#pragma unroll
-  for (int rr = 0; rr < 4; ++rr) {
-    const int n = min(nq + rr, a.N - 1);
-    rf[rr] = row_factor(F, a.scale, a.global, n);
-    bs[rr] = a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f;
-  }
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) {
     const int m = mt * 16 + i;
