@@ -841,7 +841,7 @@ void* slab_scratch(hipStream_t stream, size_t bytes) {
 
 // Which of the tile kernels' own choices the variant table fixes ("gemm_w_<format>": 4 = never the slab kernel,
 // 5 = the slab kernel wherever it fits); anything else leaves the measured rule.
-constexpr int kVariantWindow = 4, kVariantSlab = 5;
+constexpr int kVariantWindow = 4, kVariantSlab = 5, kVariantWalkParts = 6;
 
 template <int F>
 const char* gemm_key() {
@@ -1199,7 +1199,7 @@ bool try_walk(const GemmArgs& a, int* status, hipStream_t stream) {
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
   const int tuned = tuned_variant(gemm_key<F>(), a.M, a.N, a.K);
   int W;
-  if (tuned == 0 || tuned == kVariantWindow || tuned == kVariantSlab) return false;
+  if (tuned == 0 || tuned >= kVariantWindow) return false;
   if (tuned >= 1 && tuned <= 3) {
     W = 1 << (tuned - 1);
   } else {
@@ -1226,19 +1226,72 @@ bool try_walk(const GemmArgs& a, int* status, hipStream_t stream) {
   return tuned < 0 && W == 2 && launch(4);
 }
 
+// The walk kernel for a matrix of few tiles and long rows: a workgroup of eight tiles (four where eight do not divide the
+// window's pieces or do not fit LDS) walks one slice (two where a slice's groups are not fours), the slices' sums go
+// through the stream's partial-tile buffer, and the slab kernel's second half adds them and runs the epilogue. False
+// when it does not apply (one slice, ragged slices, a stream without the buffer).
+template <int F>
+bool launch_walk_parts(GemmArgs a, int* status, hipStream_t stream) {
+  if (a.xs.dtype != LX_BF16) return false;
+  const int spw = a.steps_per_wave;
+  if (spw < 8 || spw % 8 != 0) return false;
+  const int slices = (a.steps + spw - 1) / spw, gps = spw >> 2;
+  if (slices < 2 || slices > a.S) return false;
+  // A walk is groups in fours: two slices to a workgroup where one is not (then the row must be whole slices).
+  const int per_wg = gps % 4 == 0 ? 1 : 2;
+  if (per_wg == 2 && (a.steps % spw != 0 || slices % 2 != 0)) return false;
+  const int n_tiles = (a.N + kTileRows - 1) / kTileRows, mts = (a.M + 15) / 16;
+  void* const partial = slab_scratch(stream, sizeof(float) * 4 * kWave * mts * n_tiles * slices);
+  if (!partial) return false;
+  a.partial = partial;
+  a.walk_slices = per_wg;
+  auto launch = [&](int w, int* st) {
+    if constexpr (F == LX_W_BF16) return launch_walk_bf16(a, w, st, stream);
+    else if constexpr (F == LX_W_INT8) return launch_walk_int8(a, w, st, stream);
+    else if constexpr (F == LX_W_FP8) return launch_walk_fp8(a, w, st, stream);
+    else return launch_walk_nvfp4(a, w, st, stream);
+  };
+  int st = kOk;
+  if (!launch(8, &st) && !launch(4, &st)) return false;
+  if (!st) {
+    a.S = slices;  // the reducer adds the slices that were written
+    const int64_t items = static_cast<int64_t>(n_tiles) * mts * kWave;
+    hipLaunchKernelGGL((slab_reduce_kernel<F, LX_MATH_BF16>), dim3(static_cast<unsigned>((items + 255) / 256)), dim3(256), 0, stream, a, mts);
+    st = status_of(hipGetLastError());
+  }
+  *status = st;
+  return true;
+}
+
+// Where the single-slice walks are taken without a table entry. From sweeps of every variant over 2048 .. 8192 rows of
+// 4096 .. 28672 values at 16 / 32 / 64 activation rows: they win where the activations weigh most against the weights
+// (many rows, long K; NVFP4 earlier, whose values are half a byte), by up to 2 x (4096 x 14336 fp8 at 64 rows
+// 44.9 -> 28.0 us, 8192 x 28672 112 -> 66 us; nvfp4 4096 x 28672 at 32 rows 75 -> 41 us), and lose 5 .. 30 % on short rows.
+template <int F>
+bool walk_parts_wanted(int M, int n_tiles, int64_t K, int tuned) {
+  if (tuned >= 0) return tuned == kVariantWalkParts;
+  if (M <= 8) return false;
+  const int mts = (M + 15) / 16;
+  if (mts >= 3) return F == LX_W_NVFP4 || K >= 8192;
+  if (F == LX_W_NVFP4 && mts == 2 && K >= 8192) return true;
+  return K >= 28672 || (K >= 14336 && n_tiles <= 256);
+}
+
 template <int F, int MT>
 int launch_skinny(GemmArgs a, hipStream_t stream) {
   const int S = a.S;
   const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
   {
     int st = kOk;
+    if (walk_parts_wanted<F>(a.M, static_cast<int>(n_tiles), a.K, tuned_variant(gemm_key<F>(), a.M, a.N, a.K)) && launch_walk_parts<F>(a, &st, stream)) return st;
     if (try_walk<F>(a, &st, stream)) return st;
   }
   // More than eight rows: the windowed kernel (for 9 .. 16 rows where the matrix has the tiles to fill its
   // sixteen-wavefront workgroups; the lean kernel's image of all of K leaves too few of them resident there).
-  if (MT > 1 || (a.M > 8 && n_tiles >= 320)) {
+  const int tuned = tuned_variant(gemm_key<F>(), a.M, a.N, a.K);
+  if (MT > 1 || (a.M > 8 && n_tiles >= 320) || tuned == kVariantWindow || tuned == kVariantSlab) {
     int st = kOk;
-    if (slab_wanted(a.M, static_cast<int>(n_tiles), a.K, tuned_variant(gemm_key<F>(), a.M, a.N, a.K)) && launch_slab<F, LX_MATH_BF16>(a, &st, stream)) return st;
+    if (slab_wanted(a.M, static_cast<int>(n_tiles), a.K, tuned) && launch_slab<F, LX_MATH_BF16>(a, &st, stream)) return st;
     if (launch_window<F, LX_MATH_BF16>(a, &st, stream)) return st;
   }
   if constexpr (MT == 1) {

@@ -38,11 +38,16 @@ namespace walk {
 template <int N>
 using Tag = std::integral_constant<int, N>;
 
-// ROT: the workgroups start at different slices (see above) and a wavefront keeps every slice's sum in LDS until the end;
-// without it every workgroup starts at slice 0 and the sums are added as the slices end, in registers: the form for
-// shapes whose images leave no room for the sums.
-template <int F, int MT, int W, bool ROT>
+// MODE kRot: the workgroups start at different slices (see above) and a wavefront keeps every slice's sum in LDS until the
+// end. kPlain: every workgroup starts at slice 0 and the sums are added as the slices end, in registers: the form for
+// shapes whose images leave no room for the sums. kPart: the matrix has too few tiles to fill the device with whole
+// walks, so workgroup (bx, by) walks only slices [by * walk_slices, (by + 1) * walk_slices) of its tiles and leaves every
+// slice's sum in a.partial ([slice][tile][16 rows][lane] x 4 floats); the caller's second kernel adds them in ascending
+// order and runs the epilogue, so the sums are the same.
+constexpr int kPlain = 0, kRot = 1, kPart = 2;
+template <int F, int MT, int W, int MODE>
 __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
+  constexpr bool ROT = MODE == kRot, PART = MODE == kPart;
   extern __shared__ __align__(16) f32x4 lds4[];
   constexpr int E = Fmt<F>::kElems, J = E / 8;
   constexpr int PB = 4 * J;          // 16-byte pieces of an image row under one load step
@@ -58,13 +63,15 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   uint8_t* const lds = reinterpret_cast<uint8_t*>(lds4);
   uint8_t* const stage = lds + wave * 4096;
   uint8_t* const img = lds + W * 4096;  // + buffer * kImage
-  const int groups = a.steps >> 2, last = groups - 1;  // groups of four load steps in a row
-  const int gps = a.steps_per_wave >> 2;               // groups of a slice
-  const int first_slice = ROT ? blockIdx.x % a.S : 0, rot = first_slice * gps;
+  const int gps = a.steps_per_wave >> 2;  // groups of four load steps in a slice (the row's last slice may be shorter)
+  const int row_groups = a.steps >> 2;    // and in a row
+  const int slices = (row_groups + gps - 1) / gps;  // the slices that hold steps (a.S may count empty ones behind them: their sums are zero)
+  const int first_slice = ROT ? blockIdx.x % slices : PART ? blockIdx.y * a.walk_slices : 0, rot = first_slice * gps;
+  const int groups = PART ? min(a.walk_slices * gps, row_groups - rot) : row_groups, last = groups - 1;  // the groups this workgroup walks
   // The l-th group this workgroup takes (l past the end repeats the last one).
   auto group_of = [&](int l) {
     const int gq = min(l, last) + rot;
-    return gq >= groups ? gq - groups : gq;
+    return !PART && gq >= row_groups ? gq - row_groups : gq;
   };
 
   // Staging: item idx = (tile of rows * 4 + step of the window) * J + quad of pieces; wavefront tw takes
@@ -176,13 +183,16 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   f32x4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  f32x4* const sums = reinterpret_cast<f32x4*>(img + 2 * kImage) + wave * (a.S * MT * kWave) + lane;  // [slice][mt][lane]
+  f32x4* const sums = reinterpret_cast<f32x4*>(img + 2 * kImage) + wave * (a.S * MT * kWave) + lane;  // kRot: [slice][mt][lane]
   f32x4 total[MT];
-  int slice_end = gps, slice = first_slice;
+  // Where the walk is in the row: group `at` of slice `slice`, which ends before group `slice_end`.
+  int slice = first_slice, at = rot, slice_end = min(rot + gps, row_groups);
 
-  // The gamma-th group the workgroup takes (its fragments are in wv).
-  auto one_group = [&](auto phase, int gamma) {
+  // The gamma-th group the workgroup takes (its fragments are in wv). TAIL: one of the walk's last four groups, which ask
+  // for nothing past the walk's end (a 16-group walk would otherwise load 5 groups and 3 windows more than it uses).
+  auto one_group = [&](auto phase, int gamma, auto tail) {
     constexpr int P = decltype(phase)::value;  // gamma % 4
+    constexpr bool TAIL = decltype(tail)::value;
     __syncthreads();  // every wavefront has left window gamma - 1, and window gamma is complete
     const uint8_t* const xb = img + (P & 1) * kImage;
     // The products of the group, pair by pair (a pair = load step s, matrix instruction j of the step). A pair's
@@ -208,17 +218,17 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, b[p % (kAhead + 1)][mt], acc[mt], 0, 0, 0);
       if (p + 1 < kPairs) wf = weight_fragment<F>(wv[(p + 1) / J], scales[(p + 1) / J], (p + 1) % J);
-      if (p == 0) {
+      if (p == 0 && !(TAIL && P == 3)) {
         // The next window goes into the other image, the window after the next is asked for.
         stage_store(Tag<(P + 1) & 1>{}, gamma + 1);
-        stage_load(Tag<(P + 1) & 1>{}, gamma + 3);
+        if (!TAIL || P == 0) stage_load(Tag<(P + 1) & 1>{}, gamma + 3);
       }
-      if (p == 1) {
+      if (p == 1 && !(TAIL && P == 3)) {
         // The next group goes into the wavefront's image; its registers take the group four ahead of it.
         to_image(Tag<(P + 1) & 3>{});
-        issue_group(Tag<(P + 1) & 3>{}, gamma + 5);
+        if (!TAIL) issue_group(Tag<(P + 1) & 3>{}, gamma + 5);
       }
-      if (p == kPairs - 1) {
+      if (p == kPairs - 1 && !(TAIL && P == 3)) {
         asm volatile("" ::: "memory");
 #pragma unroll
         for (int s = 0; s < 4; ++s) wv_next[s] = *reinterpret_cast<const u32x4*>(stage + get_at[s]);
@@ -226,34 +236,42 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
       }
       __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (!(TAIL && P == 3)) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      scales[u] = wsc[u];
-      wv[u] = wv_next[u];
+      for (int u = 0; u < 4; ++u) {
+        scales[u] = wsc[u];
+        wv[u] = wv_next[u];
+      }
     }
     // A slice ends.
-    if (gamma + 1 == slice_end) {
+    if (++at == slice_end) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
         if constexpr (ROT) sums[(slice * MT + mt) * kWave] = acc[mt];
-        else total[mt] = slice == 0 ? acc[mt] : total[mt] + acc[mt];
+        else if constexpr (PART) {
+          if (tile < n_tiles) static_cast<f32x4*>(a.partial)[((static_cast<int64_t>(slice) * n_tiles + tile) * MT + mt) * kWave + lane] = acc[mt];
+        } else total[mt] = slice == 0 ? acc[mt] : total[mt] + acc[mt];
         acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
-      slice_end += gps;
-      slice = slice + 1 == a.S ? 0 : slice + 1;
+      if (at == row_groups) at = 0, slice = 0, slice_end = min(gps, row_groups);  // round to the row's start
+      else ++slice, slice_end = min(slice_end + gps, row_groups);
     }
   };
   for (int gamma = 0; gamma < groups - 4; gamma += 4) {
-    one_group(Tag<0>{}, gamma);
-    one_group(Tag<1>{}, gamma + 1);
-    one_group(Tag<2>{}, gamma + 2);
-    one_group(Tag<3>{}, gamma + 3);
+    one_group(Tag<0>{}, gamma, std::false_type{});
+    one_group(Tag<1>{}, gamma + 1, std::false_type{});
+    one_group(Tag<2>{}, gamma + 2, std::false_type{});
+    one_group(Tag<3>{}, gamma + 3, std::false_type{});
   }
   // The last four groups, with the epilogue's row factors and biases asked for one group before the end: at the end they
   // would be a memory latency nothing hides, and asked for at the start they would hold registers through the walk.
-  one_group(Tag<0>{}, groups - 4);
-  one_group(Tag<1>{}, groups - 3);
-  one_group(Tag<2>{}, groups - 2);
+  one_group(Tag<0>{}, groups - 4, std::true_type{});
+  one_group(Tag<1>{}, groups - 3, std::true_type{});
+  one_group(Tag<2>{}, groups - 2, std::true_type{});
+  if constexpr (PART) {
+    one_group(Tag<3>{}, groups - 1, std::true_type{});
+    return;
+  }
   const int nq = n0 + 4 * g;
   float rf[4], bs[4];
 #pragma unroll
@@ -262,7 +280,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
     rf[rr] = row_factor(F, a.scale, a.global, n);
     bs[rr] = a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f;
   }
-  one_group(Tag<3>{}, groups - 1);
+  one_group(Tag<3>{}, groups - 1, std::true_type{});
 
   // The slices' sums in ascending order (the wavefront reads what it wrote itself: LDS keeps its order).
   asm volatile("" ::: "memory");
@@ -270,7 +288,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       total[mt] = sums[mt * kWave];
-      for (int sl = 1; sl < a.S; ++sl) total[mt] += sums[(sl * MT + mt) * kWave];
+      for (int sl = 1; sl < slices; ++sl) total[mt] += sums[(sl * MT + mt) * kWave];
     }
   }
 
@@ -305,25 +323,42 @@ int launch_w(const GemmArgs& a, unsigned grid, hipStream_t stream) {
   const int MT = (a.M + 15) / 16;
   // A lane holds 2 MT 4 J / W staging pieces of 16 bytes: past 32 of them the kernel spills (measured 4 .. 20 x slower).
   if (MT * 4 * J / W > 16) return kNotSupported;
+  // Eight wavefronts a workgroup have 256 registers each: room for four pieces (NVFP4 from 33 rows spills with six).
+  if (W == 8 && MT * 4 * J / W > 4) return kNotSupported;
+  if (MT * 4 * J % W != 0) return kNotSupported;  // the wavefronts share a window's pieces evenly
   const size_t images = static_cast<size_t>(W) * 4096 + 2 * static_cast<size_t>(MT) * 4 * PB * 256;
   const size_t with_sums = images + static_cast<size_t>(W) * a.S * MT * kWave * 16;
-  const bool rot = with_sums <= kLdsMax;
+  const bool part = a.partial != nullptr;
+  const bool rot = !part && with_sums <= kLdsMax;
   const size_t lds = rot ? with_sums : images;
   if (lds > kLdsMax) return kNotSupported;
+  unsigned parts = 1;
+  if (part) {
+    // Whole slices to a workgroup, their groups in fours.
+    const int gps = a.steps_per_wave >> 2, slices = (a.steps + a.steps_per_wave - 1) / a.steps_per_wave;
+    const bool ragged = a.steps % a.steps_per_wave != 0;
+    if (a.walk_slices < 1 || (a.walk_slices * gps) % 4 != 0 || (ragged ? gps % 4 != 0 : slices % a.walk_slices != 0)) return kNotSupported;
+    parts = static_cast<unsigned>((slices + a.walk_slices - 1) / a.walk_slices);
+  }
   auto launch = [&](auto kernel) {
     if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), kLdsMax);
-    hipLaunchKernelGGL(kernel, dim3(grid), dim3(W * kWave), lds, stream, a);
+    hipLaunchKernelGGL(kernel, dim3(grid, parts), dim3(W * kWave), lds, stream, a);
     return status_of(hipGetLastError());
   };
-  switch (MT * 2 + (rot ? 1 : 0)) {
-    case 3: return launch(walk_kernel<F, 1, W, true>);
-    case 5: return launch(walk_kernel<F, 2, W, true>);
-    case 7: return launch(walk_kernel<F, 3, W, true>);
-    case 9: return launch(walk_kernel<F, 4, W, true>);
-    case 2: return launch(walk_kernel<F, 1, W, false>);
-    case 4: return launch(walk_kernel<F, 2, W, false>);
-    case 6: return launch(walk_kernel<F, 3, W, false>);
-    default: return launch(walk_kernel<F, 4, W, false>);
+  auto with_mt = [&](auto mt_tag) {
+    constexpr int M16 = decltype(mt_tag)::value;
+    if constexpr (M16 * 4 * J % W != 0) return static_cast<int>(kNotSupported);
+    else if constexpr (W == 8) return part ? launch(walk_kernel<F, M16, W, kPart>) : static_cast<int>(kNotSupported);
+    else if (part) {
+      if constexpr (W == 4) return launch(walk_kernel<F, M16, W, kPart>);
+      else return static_cast<int>(kNotSupported);
+    } else return rot ? launch(walk_kernel<F, M16, W, kRot>) : launch(walk_kernel<F, M16, W, kPlain>);
+  };
+  switch (MT) {
+    case 1: return with_mt(Tag<1>{});
+    case 2: return with_mt(Tag<2>{});
+    case 3: return with_mt(Tag<3>{});
+    default: return with_mt(Tag<4>{});
   }
 }
 
@@ -332,14 +367,16 @@ bool launch_format(const GemmArgs& a, int W, int* status, hipStream_t stream) {
   constexpr int E = Fmt<F>::kElems;
   const int S = a.S, spw = a.steps_per_wave;
   if (a.M < 1 || a.M > 64 || S < 1 || spw % 8 != 0) return false;
-  // Whole slices, and groups in fours.
-  if (S * spw != a.steps || static_cast<int64_t>(a.steps) * 4 * E != a.K || a.steps % 16 != 0) return false;
+  // Slices of whole batches, the row's last one as long as the row reaches (S may count empty ones behind it: a zero
+  // added last changes no sum), and groups in fours.
+  if ((a.steps + spw - 1) / spw > S || static_cast<int64_t>(a.steps) * 4 * E != a.K || a.steps % 16 != 0) return false;
   if (static_cast<int64_t>(a.M) * a.xs.ld * 2 + static_cast<int64_t>(a.K) * 2 >= (int64_t{1} << 31)) return false;
   if (static_cast<int64_t>(kTileRows) * a.row_bytes >= (int64_t{1} << 31)) return false;
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
   const unsigned grid = static_cast<unsigned>((n_tiles + W - 1) / W);
   int st;
   switch (W) {
+    case 8: st = launch_w<F, 8>(a, grid, stream); break;
     case 4: st = launch_w<F, 4>(a, grid, stream); break;
     case 2: st = launch_w<F, 2>(a, grid, stream); break;
     case 1: st = launch_w<F, 1>(a, grid, stream); break;

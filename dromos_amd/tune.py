@@ -47,6 +47,9 @@ def time_variants(lx, kernel, M, N, K, repeats=7):
         events.append(e)
     flush = torch.empty(FLUSH_BYTES, dtype=torch.uint8, device="cuda")
     stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    # The variants that keep partial sums in the stream's buffer run only on a stream that has one; the stream keeps it
+    # afterwards (reserving twice is harmless, and releasing here would take away a buffer the caller had reserved).
+    assert lib.lx_rt_stream_reserve(stream) == 0
     first, result = None, {}
     try:
         for v, vname in enumerate(variants(lx, kernel)):

@@ -254,7 +254,7 @@ LX_API int lx_rt_stream_create(void** stream);
 LX_API int lx_rt_stream_destroy(void* stream);
 LX_API int lx_rt_stream_sync(void* stream);
 /* No counterpart in the reference. A stream made by lx_rt_stream_create owns 64 MiB of device memory that some products
- * of lx_gemm_w / lx_gemm_skinny (17 .. 64 rows on matrices of few tiles) keep their partial sums in; no product ever
+ * of lx_gemm_w / lx_gemm_skinny (9 .. 64 rows on matrices of few tiles or long rows) keep their partial sums in; no product ever
  * allocates. A host that brings streams of its own (or uses the null stream) calls lx_rt_stream_reserve once per stream
  * (and device) to give it the same, and lx_rt_stream_release before it destroys the stream; without it those products
  * take another kernel with the same results. */
@@ -330,7 +330,7 @@ LX_API int lx_probe_empty(void* stream);
  * with s<S>, its K split, and lx_tune_set admits a variant for a shape only when its split is the
  * shape's own (so the rows' bits never depend on the table). The matrix-core products (lx_gemm_w, lx_gemm_skinny)
  * register theirs under gemm_w_<format>: which kernel family runs ("tiles", "walk1", "walk2", "walk4", "window",
- * "slab"); none changes a sum, so every one is admitted. */
+ * "slab", "walkparts"); none changes a sum, so every one is admitted. */
 LX_API int lx_arch(void);
 LX_API int lx_set_arch_override(int arch);
 LX_API int lx_tune_get(const char* kernel, int M, int N, int K);

@@ -1,8 +1,8 @@
 """GPU parity: the walk kernel of lx_gemm_w / lx_gemm_skinny (9 .. 64 bf16 activation rows, a wavefront walking a whole
 tile) against float64 on the decoded values, and bit for bit against the tile kernels it replaces on the shapes it
 takes: the variant table forces each family ("gemm_w_<format>": 0 = the tile kernels, 1 .. 3 = walk with 1, 2, 4 tiles
-a workgroup, 4 / 5 = the tile kernels without / with the slab kernel), and no variant may change an output bit, a row's
-bits may not depend on the batch."""
+a workgroup, 4 / 5 = the tile kernels without / with the slab kernel, 6 = walks of single slices whose sums meet in the
+stream's partial-tile buffer), and no variant may change an output bit, a row's bits may not depend on the batch."""
 
 import pytest
 import torch
@@ -36,10 +36,10 @@ def test_variants_are_registered(hip):
     hip.lib.lx_tune_variant_name.restype = ctypes.c_char_p
     for fmt in FMT:
         key = f"gemm_w_{fmt}".encode()
-        assert hip.lib.lx_tune_variants(key) == 6
-        assert [hip.lib.lx_tune_variant_name(key, v).decode() for v in range(6)] == ["tiles", "walk1", "walk2", "walk4", "window", "slab"]
-        assert all(hip.lib.lx_tune_set(key, 32, 4096, 4096, v) == 0 for v in range(6))  # none changes a sum: all admitted
-        assert hip.lib.lx_tune_set(key, 32, 4096, 4096, 6) == 803
+        assert hip.lib.lx_tune_variants(key) == 7
+        assert [hip.lib.lx_tune_variant_name(key, v).decode() for v in range(7)] == ["tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts"]
+        assert all(hip.lib.lx_tune_set(key, 32, 4096, 4096, v) == 0 for v in range(7))  # none changes a sum: all admitted
+        assert hip.lib.lx_tune_set(key, 32, 4096, 4096, 7) == 803
 
 
 @pytest.mark.parametrize("M", [9, 16, 17, 33, 48, 64])
@@ -53,7 +53,7 @@ def test_every_variant_gives_the_same_bits(hip, fmt, M):
         want = ops.gemv_reference(x, w.dense(), bias, 1.0, 0.0, None)
         wd, xd, bd = w.to("cuda"), x.cuda(), bias.cuda()
         outs = {}
-        for variant in (0, 1, 2, 3, 4, 5, None):
+        for variant in (0, 1, 2, 3, 4, 5, 6, None):
             force(hip, fmt, M, N, K, variant)
             y = torch.full((M, N), float("nan"), device="cuda")
             outs[variant] = ops.gemm_w(hip, xd, wd, MATH_BF16, bias=bd, y=y).clone()
@@ -176,16 +176,38 @@ def test_long_slices_in_several_slab_passes(hip, fmt, N, K):
     g = torch.Generator().manual_seed(K)
     wd = w.to("cuda")
     dense = w.dense()
-    for M in (33, 64):
+    for M in (12, 33, 64):
         x = torch.randn(M, K, generator=g).to(torch.bfloat16)
         outs = {}
-        for variant in (0, 4, 5, None):
+        for variant in (0, 4, 5, 6, None):
             force(hip, fmt, M, N, K, variant)
             outs[variant] = ops.gemm_w(hip, x.cuda(), wd, MATH_BF16).clone()
         checks.check_product(outs[5].cpu(), ops.gemv_reference(x, dense, None, 1.0, 0.0, None))
         for variant, out in outs.items():
             assert torch.equal(out.view(torch.int32), outs[4].view(torch.int32)), f"variant {variant} at {fmt} M={M}"
         # a row's bits are those of the row alone
+        force(hip, fmt, 1, N, K, None)
+        alone = ops.gemm_skinny(hip, x[M - 1 : M].cuda(), wd)
+        assert torch.equal(alone[0].view(torch.int32), outs[None][M - 1].view(torch.int32))
+
+
+@pytest.mark.parametrize("fmt,N,K", [("fp8", 8192, 7168), ("int8", 8192, 7168), ("nvfp4", 8192, 14336), ("bf16", 8192, 3584)])
+def test_a_short_last_slice(hip, fmt, N, K):
+    # 112 load steps in four slices of 32: the last slice is half as long as the others. Every walk takes it as the tile
+    # kernels do (whole walks that start anywhere in the row, and walks of single slices).
+    w = random_weight(FORMATS[fmt], N, K, N + K)
+    g = torch.Generator().manual_seed(K)
+    wd = w.to("cuda")
+    dense = w.dense()
+    for M in (16, 40, 64):
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        outs = {}
+        for variant in (0, 1, 2, 3, 4, 6, None):
+            force(hip, fmt, M, N, K, variant)
+            outs[variant] = ops.gemm_w(hip, x.cuda(), wd, MATH_BF16).clone()
+        checks.check_product(outs[0].cpu(), ops.gemv_reference(x, dense, None, 1.0, 0.0, None))
+        for variant, out in outs.items():
+            assert torch.equal(out.view(torch.int32), outs[0].view(torch.int32)), f"variant {variant} at {fmt} M={M}"
         force(hip, fmt, 1, N, K, None)
         alone = ops.gemm_skinny(hip, x[M - 1 : M].cuda(), wd)
         assert torch.equal(alone[0].view(torch.int32), outs[None][M - 1].view(torch.int32))
