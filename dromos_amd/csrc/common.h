@@ -111,6 +111,51 @@ __device__ __forceinline__ float wave_sum(float v) {
   return a + b;
 }
 
+// N wave sums at once (N = 2, 4, 8 or 16): lane l ends with the sum of v[l % N] over the wavefront, by wave_sum's
+// tree. Where wave_sum adds a value and its partner's in every lane, two sums share the step: the lanes whose bit d is
+// clear keep the first sum's pair, the others the second's, so the registers halve at every step and sixteen sums cost
+// about fifty instructions instead of a hundred and sixty. The operands of every addition are those of wave_sum (a + b
+// or b + a), so each sum has wave_sum's bits. (Partners are true xor partners here: lane ^ 4 through the LDS crossbar,
+// lane ^ 8 by a rotation of the 16-lane row; wave_sum's mirrors pair the same partial sums only while every lane of a
+// quad holds the same one.)
+template <int N>
+__device__ __forceinline__ float wave_sum_many(const float (&in)[N]) {
+  static_assert(N == 2 || N == 4 || N == 8 || N == 16, "a power of two up to 16");
+  const unsigned lane = threadIdx.x & (kWave - 1);
+  float v[N];
+#pragma unroll
+  for (int i = 0; i < N; ++i) v[i] = in[i];
+  auto xor1 = [](float x) { return dpp_move<0xB1>(x); };
+  auto xor2 = [](float x) { return dpp_move<0x4E>(x); };
+  auto xor4 = [](float x) { return __int_as_float(__builtin_amdgcn_ds_swizzle(__float_as_int(x), 0x101F)); };
+  auto xor8 = [](float x) { return dpp_move<0x128>(x); };  // row_ror:8
+  int n = N;
+  auto step = [&](bool upper, auto partner) {
+    if (n > 1) {
+      // v[i] <- the pair sums of v[2 i] (lanes with the bit clear) and of v[2 i + 1] (lanes with it set)
+#pragma unroll
+      for (int i = 0; i < N / 2; ++i) {
+        if (i < n / 2) {
+          const float keep = upper ? v[2 * i + 1] : v[2 * i], send = upper ? v[2 * i] : v[2 * i + 1];
+          v[i] = keep + partner(send);
+        }
+      }
+      n /= 2;
+    } else {
+      v[0] += partner(v[0]);
+    }
+  };
+  step((lane & 1u) != 0, xor1);
+  step((lane & 2u) != 0, xor2);
+  step((lane & 4u) != 0, xor4);
+  step((lane & 8u) != 0, xor8);
+  float a, b;
+  swap_halves<true>(v[0], a, b);
+  const float w = a + b;
+  swap_halves<false>(w, a, b);
+  return a + b;
+}
+
 __device__ __forceinline__ float wave_max(float v) {
   v = fmaxf(v, dpp_move<0xB1>(v));
   v = fmaxf(v, dpp_move<0x4E>(v));

@@ -83,36 +83,30 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs
       x_image[r] = xs;
     }
   };
+  // A group's MT * R lane sums become wave sums sixteen at a time: lane j of a round ends with the sum of output j
+  // (activation row j / R, weight row j % R of the group), so the S > 1 exchange and the epilogue run once across the
+  // lanes instead of once per output.
   auto done_fn = [&](int g, float (&acc)[MT][R]) {
+    constexpr int NO = MT * R, PER = NO < 16 ? NO : 16;
 #pragma unroll
-    for (int m = 0; m < MT; ++m)
+    for (int o0 = 0; o0 < NO; o0 += PER) {
+      float sum;
+      if constexpr (PER == 1) {
+        sum = wave_sum(acc[0][0]);
+      } else {
+        float v[PER];
 #pragma unroll
-      for (int r = 0; r < R; ++r) acc[m][r] = wave_sum(acc[m][r]);
-    if (S > 1) {
-      if (lane == 0) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-#pragma unroll
-          for (int r = 0; r < R; ++r) partial[wave * (MT * R) + m * R + r] = acc[m][r];
+        for (int j = 0; j < PER; ++j) v[j] = acc[(o0 + j) / R][(o0 + j) % R];
+        sum = wave_sum_many<PER>(v);
       }
-      __syncthreads();
-      if (part == 0) {
-#pragma unroll
-        for (int m = 0; m < MT; ++m)
-#pragma unroll
-          for (int r = 0; r < R; ++r) {
-            float s = acc[m][r];
-            for (int p = 1; p < S; ++p) s += partial[(wave + p) * (MT * R) + m * R + r];
-            acc[m][r] = s;
-          }
+      const int o = o0 + (lane & (PER - 1)), m = o / R, r = o % R;
+      if (S > 1) {
+        if (lane < PER) partial[wave * NO + o] = sum;
+        __syncthreads();
+        if (part == 0 && lane < PER)
+          for (int p = 1; p < S; ++p) sum += partial[(wave + p) * NO + o];
       }
-    }
-    if (lane == 0 && part == 0) {
-#pragma unroll
-      for (int m = 0; m < MT; ++m)
-#pragma unroll
-        for (int r = 0; r < R; ++r)
-          if (m < a.M && g * R + r < a.N) write_out(a, F, m, static_cast<int64_t>(g) * R + r, acc[m][r]);
+      if (lane < PER && part == 0 && m < a.M && g * R + r < a.N) write_out(a, F, m, static_cast<int64_t>(g) * R + r, sum);
     }
   };
 
