@@ -38,18 +38,23 @@ struct GemvArgs {
   int64_t row_bytes;
   int64_t scale_row_bytes;  // NVFP4: bytes of block scales per row; BF16X: a whole record
   int phase_steps;  // > 0: the activation image holds this many steps at a time (two images in turn), else all
+  int rounds;       // ROLL kernels: the consecutive row groups a workgroup takes (at least one per wavefront)
 };
 
 namespace {
 
-// The epilogue's operation order (engine/cpu/gemm.cpp:21-34).
-__device__ __forceinline__ void write_out(const GemvArgs& a, int wtype, int m, int64_t n, float sum) {
-  float t = row_factor(wtype, a.scale, a.global, n) * sum;
-  if (a.bias) t += load_as_f32(a.bias, a.bias_dtype, n);
+// The epilogue's operation order (engine/cpu/gemm.cpp:21-34); rf is the row factor, b the bias (unused without one).
+__device__ __forceinline__ void write_out(const GemvArgs& a, int m, int64_t n, float sum, float rf, float b) {
+  float t = rf * sum;
+  if (a.bias) t += b;
   float v = a.alpha * t;
   const int64_t at = m * a.ld_y + n;
   if (a.beta != 0.0f) v = a.beta * load_as_f32(a.y, a.y_dtype, at) + v;
   store_from_f32(a.y, a.y_dtype, at, v);
+}
+
+__device__ __forceinline__ void write_out(const GemvArgs& a, int wtype, int m, int64_t n, float sum) {
+  write_out(a, m, n, sum, row_factor(wtype, a.scale, a.global, n), a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f);
 }
 
 // One workgroup takes blockDim / 64 / S groups of R rows, one group per wavefront (S wavefronts share a
@@ -58,8 +63,14 @@ __device__ __forceinline__ void write_out(const GemvArgs& a, int wtype, int m, i
 // memory system busier than a few long-lived ones.
 // XB: the activations are bf16 and go into the packed image (two products per instruction); otherwise the f32 image.
 // ONE: a wavefront's share of a row's steps fits one batch of U (the usual case at decode sizes).
-template <int F, int MT, int R, int U, bool XB, bool ONE>
+// ROLL (several bf16 activation rows, one-batch rows, no K split): the products of several rows cost about as many
+// vector instructions as the weights take to arrive, and with a workgroup per set of rows the device holds only part of
+// the workgroups at a time: all ask, all wait, all multiply, and only then do the others ask. Here the grid is what the
+// device holds at once and a wavefront streams `rounds` groups through its one batch of registers (run_rolling), so the
+// memory and the vector units work at the same time; the image is staged once per workgroup.
+template <int F, int MT, int R, int U, bool XB, bool ONE, bool ROLL = false>
 __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs a) {
+  static_assert(!ROLL || (ONE && XB && MT > 1 && F != LX_W_BF16X), "rolling: one batch, the packed image, several activation rows");
   extern __shared__ __align__(16) float lds[];
   const int steps = a.steps;
   const int per_row = x_row_words<F, XB>(a.phase_steps > 0 ? a.phase_steps : steps);
@@ -86,8 +97,20 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs
   // A group's MT * R lane sums become wave sums sixteen at a time: lane j of a round ends with the sum of output j
   // (activation row j / R, weight row j % R of the group), so the S > 1 exchange and the epilogue run once across the
   // lanes instead of once per output.
-  auto done_fn = [&](int g, float (&acc)[MT][R]) {
-    constexpr int NO = MT * R, PER = NO < 16 ? NO : 16;
+  constexpr int NO = MT * R, PER = NO < 16 ? NO : 16;
+  // What lane j's outputs of group g need besides their sums: the weight row's factor and bias (the same weight row in
+  // every round of sixteen when there are several, as 16 is a multiple of R).
+  struct Epilogue {
+    float rf, bias;
+  };
+  auto pre_fn = [&](int g) {
+    const int64_t n = min(static_cast<int64_t>(g) * R + (lane & (PER - 1)) % R, static_cast<int64_t>(a.N) - 1);
+    Epilogue e;
+    e.rf = row_factor(F, a.scale, a.global, n);
+    e.bias = a.bias ? load_as_f32(a.bias, a.bias_dtype, n) : 0.0f;
+    return e;
+  };
+  auto finish = [&](int g, float (&acc)[MT][R], const Epilogue& e) {
 #pragma unroll
     for (int o0 = 0; o0 < NO; o0 += PER) {
       float sum;
@@ -106,12 +129,29 @@ __global__ void __launch_bounds__(kMaxThreads) gemv_stream_kernel(const GemvArgs
         if (part == 0 && lane < PER)
           for (int p = 1; p < S; ++p) sum += partial[(wave + p) * NO + o];
       }
-      if (lane < PER && part == 0 && m < a.M && g * R + r < a.N) write_out(a, F, m, static_cast<int64_t>(g) * R + r, sum);
+      if (lane < PER && part == 0 && m < a.M && g * R + r < a.N) write_out(a, m, static_cast<int64_t>(g) * R + r, sum, e.rf, e.bias);
     }
   };
+  auto done_fn = [&](int g, float (&acc)[MT][R]) { finish(g, acc, pre_fn(g)); };
 
   RowStreamer<F, MT, R, U, XB, ONE> st(a.chunks, s_begin, s_end, per_row);
   if constexpr (F == LX_W_BF16X) st.set_bf16x(static_cast<int>(a.K));
+  if constexpr (ROLL) {
+    // The workgroup's a.rounds consecutive groups go round its wavefronts (the first ones take one more when they do not
+    // divide: the device's share of groups per SIMD is then the same everywhere). A group past the last streams the last
+    // rows again and writes nothing.
+    const int waves_per_wg = blockDim.x / kWave;
+    const int group = blockIdx.x * a.rounds + wave;
+    // Ask for the activation rows, then for the first group's weights, and only then wait for the rows.
+    XRowRegsN<MT> xr;
+    stage_rows_load<F>(xr, static_cast<const uint16_t*>(a.x), a.ld_x, nullptr, a.M, a.K, steps);
+    st.prefetch(rows_fn, group, 0, 1);
+    if (xr.ready) stage_rows_store<F, MT>(xr, reinterpret_cast<uint32_t*>(xs), a.M, a.K, steps);
+    else stage_x_pairs<F, MT>(reinterpret_cast<uint32_t*>(xs), static_cast<const uint16_t*>(a.x), a.ld_x, nullptr, a.M, a.K, steps);
+    __syncthreads();
+    st.run_rolling(rows_fn, pre_fn, finish, group, waves_per_wg, (a.rounds - wave + waves_per_wg - 1) / waves_per_wg);
+    return;
+  }
   auto stage_all = [&] {
     if constexpr (XB) stage_x_pairs<F, MT>(reinterpret_cast<uint32_t*>(xs), static_cast<const uint16_t*>(a.x), a.ld_x, nullptr, a.M, a.K, steps);
     else stage_x<F, MT>(xs, a.x, a.x_dtype, a.ld_x, nullptr, a.M, a.K, steps);
@@ -222,7 +262,7 @@ int launch_stream(GemvArgs a, const Shape& shape, hipStream_t stream) {
   const size_t lds = sizeof(float) * (static_cast<size_t>(MT) * x_row_words<F, XB>(a.phase_steps > 0 ? a.phase_steps : a.steps) + waves * MT * R);
   const int groups_per_wg = waves / a.split;
   const int64_t n_groups = (a.N + R - 1) / R;
-  const int64_t grid = (n_groups + groups_per_wg - 1) / groups_per_wg;
+  int64_t grid = (n_groups + groups_per_wg - 1) / groups_per_wg;
   auto launch = [&](auto kernel) {
     if (lds > 48 * 1024) {
       static thread_local bool raised = false;  // one per kernel: the lambda is instantiated per kernel type
@@ -236,6 +276,29 @@ int launch_stream(GemvArgs a, const Shape& shape, hipStream_t stream) {
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(grid)), dim3(shape.threads), lds, stream, a);
     return status_of(hipGetLastError());
   };
+  a.rounds = 1;
+  if constexpr (MT > 1 && XB && F != LX_W_BF16X) {
+    if (a.phase_steps == 0 && a.split == 1 && a.steps_per_part <= U) {
+      // The workgroups the device holds at once (asked once per kernel and workgroup shape).
+      static thread_local int held_for_lds = -1, held = 0;
+      if (held_for_lds != static_cast<int>(lds)) {
+        int per_cu = 0;
+        if (lds > 48 * 1024) (void)hipFuncSetAttribute(reinterpret_cast<const void*>(gemv_stream_kernel<F, MT, R, U, XB, true, true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 256);
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, gemv_stream_kernel<F, MT, R, U, XB, true, true>, shape.threads, lds) != hipSuccess) {
+          (void)hipGetLastError();
+          per_cu = 0;
+        }
+        held = per_cu * compute_units();
+        held_for_lds = static_cast<int>(lds);
+      }
+      if (held > 0 && grid > held) {
+        a.rounds = static_cast<int>((n_groups + held - 1) / held);  // groups per workgroup
+        if (a.rounds < waves) a.rounds = waves;
+        grid = (n_groups + a.rounds - 1) / a.rounds;
+        return launch(gemv_stream_kernel<F, MT, R, U, XB, true, true>);
+      }
+    }
+  }
   return a.steps_per_part <= U ? launch(gemv_stream_kernel<F, MT, R, U, XB, true>) : launch(gemv_stream_kernel<F, MT, R, U, XB, false>);
 }
 

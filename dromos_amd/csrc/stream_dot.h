@@ -832,6 +832,74 @@ struct RowStreamer {
     }
   }
 
+  // ONE, several groups a wavefront (first_group, first_group + stride, ..., n_groups of them; prefetch() has asked for
+  // the first): as soon as a step's chunks have been multiplied, their registers take the same step of the next group,
+  // so a wavefront keeps a whole batch on its way while it multiplies, in the registers of one. Every load sits outside
+  // any branch (the last group, which asks for nothing, is a copy of its own): a load under a condition would turn every
+  // later wait into a wait for all of them. Not for BF16X (its exceptions ride on a batch's first chunk).
+  // pre_fn(g) asks for what group g's epilogue needs and finish_fn(g, acc, that) uses it: asked for before the next
+  // group's chunks, it is there when the sums are (loads return in order: asked for at the end, it would wait for all
+  // of the next group).
+  template <class RowsFn, class PreFn, class FinishFn>
+  __device__ __forceinline__ void run_rolling(RowsFn& rows_fn, PreFn& pre_fn, FinishFn& finish_fn, int first_group, int stride, int n_groups) {
+    static_assert(ONE && F != LX_W_BF16X, "one buffer, plain chunks");
+    float acc[MT][R];
+    auto zero = [&] {
+#pragma unroll
+      for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[m][r] = 0.0f;
+    };
+    zero();
+    const int last_step = s_end > s_begin ? s_end - 1 : s_begin;
+    const uint8_t* rows[R];
+    const uint8_t* scales[R];
+    const float* xs[R];
+    rows_fn(first_group, rows, scales, xs);
+    int g = first_group;
+    auto step = [&](int u) {
+      if (s_begin + u < s_end) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) consume_one<false>(buf_a[u][r], NoExceptions{}, rows[r], xs[r], s_begin + u, u, 0, r, acc);
+      }
+    };
+    // A row pointer is the same in every lane: said so, the loads take it from scalar registers.
+    auto uniform = [](const uint8_t* p) {
+      const uint64_t v = reinterpret_cast<uint64_t>(p);
+      const uint32_t lo = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v)), hi = __builtin_amdgcn_readfirstlane(static_cast<uint32_t>(v >> 32));
+      return reinterpret_cast<const uint8_t*>((static_cast<uint64_t>(hi) << 32) | lo);
+    };
+    for (int t = 1; t < n_groups; ++t) {
+      const uint8_t* next_rows[R];
+      const uint8_t* next_scales[R];
+      const float* next_xs[R];
+      rows_fn(g + stride, next_rows, next_scales, next_xs);
+#pragma unroll
+      for (int r = 0; r < R; ++r) next_rows[r] = uniform(next_rows[r]), next_scales[r] = uniform(next_scales[r]);
+      const auto epilogue = pre_fn(g);
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        step(u);
+        // The scheduler is held to this order: left alone it asks for the next group's chunks early, in registers of
+        // their own, and the kernel loses the wavefronts those registers would have held.
+        __builtin_amdgcn_sched_barrier(0);
+        const int chunk = min(min(s_begin + u, last_step) * kWave + lane, chunks - 1);
+#pragma unroll
+        for (int r = 0; r < R; ++r) load_chunk<F>(buf_a[u][r], next_rows[r], next_scales[r], chunk);
+        __builtin_amdgcn_sched_barrier(0);
+      }
+      finish_fn(g, acc, epilogue);
+      zero();
+      g += stride;
+#pragma unroll
+      for (int r = 0; r < R; ++r) rows[r] = next_rows[r], scales[r] = next_scales[r], xs[r] = next_xs[r];
+    }
+    const auto epilogue = pre_fn(g);
+#pragma unroll
+    for (int u = 0; u < U; ++u) step(u);
+    finish_fn(g, acc, epilogue);
+  }
+
   // Groups first_group, first_group + stride, ... (n_groups of them); prefetch() has asked for the first two
   // batches.
   template <class RowsFn, class DoneFn>

@@ -192,3 +192,14 @@ def test_rows_do_not_depend_on_the_batch_long_rows(hip, fmt, N, K):
     # Rows long enough that eight activation rows do not fit one LDS image: the image then holds half of K at a time
     # (or the weights are passed over twice), and a row's bits must still be those of the row alone.
     checks.gemv_rows_do_not_depend_on_batch(hip, fmt, N, K, seed=N + K)
+
+
+@pytest.mark.parametrize("fmt,N,K", [("int8", 14335, 4096), ("fp8", 14336, 4096), ("bf16", 9001, 4096), ("nvfp4", 14336, 4096), ("int8", 12000, 1024)])
+def test_more_rows_than_the_device_holds_at_once(hip, fmt, N, K):
+    # With several bf16 activation rows and more weight rows than the device's wavefronts hold in one go, a wavefront
+    # streams several row groups in turn (the workgroup's groups go round its wavefronts; the last workgroup's run past N).
+    # A row's bits are those of the row alone, the values the reference's, the bias and factors the row's own.
+    checks.gemv_rows_do_not_depend_on_batch(hip, fmt, N, K, seed=N + K)
+    for M in (2, 4, 8):
+        checks.gemv_case(hip, fmt, M, N, K, seed=M + N, x_dtype=torch.bfloat16, bias_dtype=torch.float32, alpha=0.5)
+    checks.gemv_case(hip, fmt, 8, N, K, seed=N, x_dtype=torch.bfloat16, bias_dtype=torch.bfloat16, y_dtype=torch.bfloat16, alpha=-1.5, beta=1.0, pad=8)
