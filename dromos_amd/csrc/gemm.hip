@@ -841,7 +841,7 @@ void* slab_scratch(hipStream_t stream, size_t bytes) {
 
 // Which of the tile kernels' own choices the variant table fixes ("gemm_w_<format>": 4 = never the slab kernel,
 // 5 = the slab kernel wherever it fits); anything else leaves the measured rule.
-constexpr int kVariantWindow = 4, kVariantSlab = 5, kVariantWalkParts = 6;
+constexpr int kVariantWindow = 4, kVariantSlab = 5, kVariantWalkParts = 6, kVariantWalkSplit = 7;
 
 template <int F>
 const char* gemm_key() {
@@ -1263,6 +1263,38 @@ bool launch_walk_parts(GemmArgs a, int* status, hipStream_t stream) {
   return true;
 }
 
+// The walk kernel with a tile's slices split over the four (or two) wavefronts of a workgroup; false when it does not
+// apply (slices that do not divide, a short last slice, windows that do not fit).
+template <int F>
+bool launch_walk_split(GemmArgs a, int* status, hipStream_t stream) {
+  if (a.xs.dtype != LX_BF16) return false;
+  const int spw = a.steps_per_wave;
+  if (spw < 8 || spw % 8 != 0 || a.steps % spw != 0) return false;
+  const int slices = a.steps / spw;
+  auto launch = [&](int w, int* st) {
+    if (slices % w != 0) return false;
+    a.walk_split = w;
+    a.walk_slices = slices / w;
+    if constexpr (F == LX_W_BF16) return launch_walk_bf16(a, w, st, stream);
+    else if constexpr (F == LX_W_INT8) return launch_walk_int8(a, w, st, stream);
+    else if constexpr (F == LX_W_FP8) return launch_walk_fp8(a, w, st, stream);
+    else return launch_walk_nvfp4(a, w, st, stream);
+  };
+  return launch(4, status) || launch(2, status);
+}
+
+// Where a tile's slices are split over a workgroup's wavefronts without a table entry: a tile per compute unit at most
+// (the windows of four wavefronts fill a unit's LDS, so a second workgroup waits for the first: 5120 x 4096 fp8 at 16 / 32
+// rows 9.6 / 12.1 -> 12.3 / 18.1 us) and up to 32 rows of short K, where the whole walk is a few wavefronts' long chains:
+// 4096 x 4096 at 16 / 32 rows fp8 9.3 / 12.1 -> 7.3 / 10.2 us, int8 11.4 / 14.2 -> 7.7 / 10.6, bf16 10.6 / 14.4 -> 9.0 / 11.7,
+// nvfp4 at 16 rows 12.6 -> 9.6; 2048 x 4096 fp8 8.3 / 11.7 -> 6.5 / 9.7; 4096 x 8192 fp8 at 16 rows 13.3 -> 11.2 (at 32 rows
+// the single-slice walks and the slab kernel do better there). Two wavefronts a tile, whose windows leave room for two
+// workgroups a unit, do not carry it to 257 .. 512 tiles (6144 x 4096 fp8 at 32 rows 12.2 -> 15.0 us).
+inline bool walk_split_wanted(int M, int n_tiles, int64_t K, int tuned) {
+  if (tuned >= 0) return tuned == kVariantWalkSplit;
+  return M > 8 && M <= 32 && n_tiles <= compute_units() && (K <= 4096 || (M <= 16 && K <= 8192));
+}
+
 // Where the single-slice walks are taken without a table entry. From sweeps of every variant over 2048 .. 8192 rows of
 // 4096 .. 28672 values at 16 / 32 / 64 activation rows: they win where the activations weigh most against the weights
 // (many rows, long K; NVFP4 earlier, whose values are half a byte), by up to 2 x (4096 x 14336 fp8 at 64 rows
@@ -1284,6 +1316,7 @@ int launch_skinny(GemmArgs a, hipStream_t stream) {
   {
     int st = kOk;
     if (walk_parts_wanted<F>(a.M, static_cast<int>(n_tiles), a.K, tuned_variant(gemm_key<F>(), a.M, a.N, a.K)) && launch_walk_parts<F>(a, &st, stream)) return st;
+    if (walk_split_wanted(a.M, static_cast<int>(n_tiles), a.K, tuned_variant(gemm_key<F>(), a.M, a.N, a.K)) && launch_walk_split<F>(a, &st, stream)) return st;
     if (try_walk<F>(a, &st, stream)) return st;
   }
   // More than eight rows: the windowed kernel (for 9 .. 16 rows where the matrix has the tiles to fill its

@@ -37,7 +37,8 @@ struct GemmArgs {
   const float* act_scale;  // BF16-math kernels on a quantised math's activation images: the rows' scales (else null)
   int pass_begin, pass_steps, pass_continues;  // slab kernel: the part of every slice this launch takes, and whether it goes on from `partial`
   void* partial;  // slab kernel with S > 1: the slices' partial tiles, [S][tile][16 rows][lane] x 4 words (f32, or i32 for the INT8 math)
-  int walk_slices;  // walk kernel with partial tiles: the slices a workgroup walks
+  int walk_slices;  // walk kernel with partial tiles: the slices a workgroup walks; split over a workgroup's wavefronts: the slices a wavefront walks
+  int walk_split;   // walk kernel: the wavefronts of a workgroup take one tile between them (two or four of them)
 };
 
 // The epilogue's operation order (engine/cpu/gemm.cpp:21-34); rf is the row factor, b the bias (0 without one).
@@ -55,7 +56,8 @@ __device__ __forceinline__ void write_out(const GemmArgs& a, int wtype, int m, i
 }
 
 // gemm_walk_<format>.hip: the walk kernel (gemm_walk.h) for up to 64 bf16 activation rows with W tiles a workgroup
-// (1, 2 or 4; with a.partial set, 4 or 8, and a workgroup walks a.walk_slices slices and leaves their sums there); false when it does not apply to the call (the caller then takes another kernel), otherwise *status holds
+// (1, 2 or 4; with a.partial set, 4 or 8, and a workgroup walks a.walk_slices slices and leaves their sums there; with a.walk_split
+// set, W = 2 or 4 wavefronts on one tile); false when it does not apply to the call (the caller then takes another kernel), otherwise *status holds
 // the launch's status.
 bool launch_walk_bf16(const GemmArgs& a, int W, int* status, hipStream_t stream);
 bool launch_walk_int8(const GemmArgs& a, int W, int* status, hipStream_t stream);

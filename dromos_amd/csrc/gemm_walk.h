@@ -43,35 +43,40 @@ using Tag = std::integral_constant<int, N>;
 // shapes whose images leave no room for the sums. kPart: the matrix has too few tiles to fill the device with whole
 // walks, so workgroup (bx, by) walks only slices [by * walk_slices, (by + 1) * walk_slices) of its tiles and leaves every
 // slice's sum in a.partial ([slice][tile][16 rows][lane] x 4 floats); the caller's second kernel adds them in ascending
-// order and runs the epilogue, so the sums are the same.
-constexpr int kPlain = 0, kRot = 1, kPart = 2;
+// order and runs the epilogue, so the sums are the same. kSplit, for the same matrices while they are small (few tiles
+// and short rows: a whole walk is then a few wavefronts' long chains of dependent steps, and single slices pay a second
+// launch): the W wavefronts of a workgroup take one tile between them, wavefront w slices [w * walk_slices,
+// (w + 1) * walk_slices), each with windows of its own (no barrier until the end: a wavefront stages what it reads), and
+// the slices' sums meet in LDS, where the first wavefront adds them in ascending order.
+constexpr int kPlain = 0, kRot = 1, kPart = 2, kSplit = 3;
 template <int F, int MT, int W, int MODE>
 __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
-  constexpr bool ROT = MODE == kRot, PART = MODE == kPart;
+  constexpr bool ROT = MODE == kRot, PART = MODE == kPart, SPLIT = MODE == kSplit;
   extern __shared__ __align__(16) f32x4 lds4[];
   constexpr int E = Fmt<F>::kElems, J = E / 8;
   constexpr int PB = 4 * J;          // 16-byte pieces of an image row under one load step
-  constexpr int Q = MT * 4 * J / W;  // staging pieces a lane holds per window
-  static_assert(Q * W == MT * 4 * J && Q >= 1, "the wavefronts share a window's pieces evenly");
+  constexpr int WS = SPLIT ? 1 : W;  // the wavefronts that share a window
+  constexpr int Q = MT * 4 * J / WS;  // staging pieces a lane holds per window
+  static_assert(Q * WS == MT * 4 * J && Q >= 1, "the wavefronts share a window's pieces evenly");
   constexpr int kImage = MT * 4 * PB * 256;  // one window
   const int lane = threadIdx.x & (kWave - 1), wave = __builtin_amdgcn_readfirstlane(threadIdx.x / kWave);
-  const int tw = wave;  // tile of the workgroup
+  const int tw = SPLIT ? 0 : wave;  // tile of the workgroup, and the wavefront's place among those that share its windows
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
-  const int tile = blockIdx.x * W + tw;
+  const int tile = SPLIT ? blockIdx.x : blockIdx.x * W + tw;
   const int n0 = min(tile, n_tiles - 1) * kTileRows, valid = min(kTileRows, a.N - n0);  // a tile past the last repeats it
   const int g = lane >> 4, i = lane & 15;
   uint8_t* const lds = reinterpret_cast<uint8_t*>(lds4);
   uint8_t* const stage = lds + wave * 4096;
-  uint8_t* const img = lds + W * 4096;  // + buffer * kImage
+  uint8_t* const img = lds + W * 4096 + (SPLIT ? wave * 2 * kImage : 0);  // + buffer * kImage
   const int gps = a.steps_per_wave >> 2;  // groups of four load steps in a slice (the row's last slice may be shorter)
   const int row_groups = a.steps >> 2;    // and in a row
   const int slices = (row_groups + gps - 1) / gps;  // the slices that hold steps (a.S may count empty ones behind them: their sums are zero)
-  const int first_slice = ROT ? blockIdx.x % slices : PART ? blockIdx.y * a.walk_slices : 0, rot = first_slice * gps;
-  const int groups = PART ? min(a.walk_slices * gps, row_groups - rot) : row_groups, last = groups - 1;  // the groups this workgroup walks
-  // The l-th group this workgroup takes (l past the end repeats the last one).
+  const int first_slice = ROT ? blockIdx.x % slices : PART ? blockIdx.y * a.walk_slices : SPLIT ? wave * a.walk_slices : 0, rot = first_slice * gps;
+  const int groups = PART || SPLIT ? min(a.walk_slices * gps, row_groups - rot) : row_groups, last = groups - 1;  // the groups this wavefront walks
+  // The l-th group this wavefront takes (l past the end repeats the last one).
   auto group_of = [&](int l) {
     const int gq = min(l, last) + rot;
-    return !PART && gq >= row_groups ? gq - row_groups : gq;
+    return !PART && !SPLIT && gq >= row_groups ? gq - row_groups : gq;
   };
 
   // Staging: item idx = (tile of rows * 4 + step of the window) * J + quad of pieces; wavefront tw takes
@@ -88,7 +93,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   uint32_t x_lds[J == 2 ? Q : 1];  // J == 2: where it goes in an image
 #pragma unroll
   for (int it = 0; it < Q; ++it) {
-    const int idx = tw + it * W;
+    const int idx = tw + it * WS;
     if constexpr (J == 2) {
       const int h = idx & 1, u = (idx >> 1) & 3, mt = idx >> 3;
       const int row = 8 * h + (i >> 1), piece = 2 * g + (i & 1);
@@ -113,7 +118,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
     } else {
       uint8_t* const dst = img + (gamma & 1) * kImage + tw * 1024 + lds_lane;
 #pragma unroll
-      for (int it = 0; it < Q; ++it) *reinterpret_cast<u32x4*>(dst + it * (W * 1024)) = xr[decltype(set)::value][it];
+      for (int it = 0; it < Q; ++it) *reinterpret_cast<u32x4*>(dst + it * (WS * 1024)) = xr[decltype(set)::value][it];
     }
   };
 
@@ -183,7 +188,9 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   f32x4 acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
-  f32x4* const sums = reinterpret_cast<f32x4*>(img + 2 * kImage) + wave * (a.S * MT * kWave) + lane;  // kRot: [slice][mt][lane]
+  // kRot: the wavefront's own [slice][mt][lane] behind the images; kSplit: the tile's, behind every wavefront's images.
+  f32x4* const sums = SPLIT ? reinterpret_cast<f32x4*>(lds + W * 4096 + W * 2 * kImage) + lane
+                            : reinterpret_cast<f32x4*>(img + 2 * kImage) + wave * (a.S * MT * kWave) + lane;
   f32x4 total[MT];
   // Where the walk is in the row: group `at` of slice `slice`, which ends before group `slice_end`.
   int slice = first_slice, at = rot, slice_end = min(rot + gps, row_groups);
@@ -193,7 +200,10 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   auto one_group = [&](auto phase, int gamma, auto tail) {
     constexpr int P = decltype(phase)::value;  // gamma % 4
     constexpr bool TAIL = decltype(tail)::value;
-    __syncthreads();  // every wavefront has left window gamma - 1, and window gamma is complete
+    // Every wavefront has left window gamma - 1, and window gamma is complete (kSplit: the wavefront's own window, which
+    // its own LDS instructions, run in order, have written).
+    if constexpr (SPLIT) asm volatile("" ::: "memory");
+    else __syncthreads();
     const uint8_t* const xb = img + (P & 1) * kImage;
     // The products of the group, pair by pair (a pair = load step s, matrix instruction j of the step). A pair's
     // activation fragments are asked for two pairs ahead, the next pair's weights are expanded under this pair's matrix
@@ -247,7 +257,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
     if (++at == slice_end) {
 #pragma unroll
       for (int mt = 0; mt < MT; ++mt) {
-        if constexpr (ROT) sums[(slice * MT + mt) * kWave] = acc[mt];
+        if constexpr (ROT || SPLIT) sums[(slice * MT + mt) * kWave] = acc[mt];
         else if constexpr (PART) {
           if (tile < n_tiles) static_cast<f32x4*>(a.partial)[((static_cast<int64_t>(slice) * n_tiles + tile) * MT + mt) * kWave + lane] = acc[mt];
         } else total[mt] = slice == 0 ? acc[mt] : total[mt] + acc[mt];
@@ -282,9 +292,13 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   }
   one_group(Tag<3>{}, groups - 1, std::true_type{});
 
-  // The slices' sums in ascending order (the wavefront reads what it wrote itself: LDS keeps its order).
+  // The slices' sums in ascending order (kRot: the wavefront reads what it wrote itself: LDS keeps its order).
   asm volatile("" ::: "memory");
-  if constexpr (ROT) {
+  if constexpr (SPLIT) {
+    __syncthreads();
+    if (wave != 0) return;
+  }
+  if constexpr (ROT || SPLIT) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
       total[mt] = sums[mt * kWave];
@@ -317,10 +331,43 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   }
 }
 
+// kSplit: W wavefronts on one tile, a.walk_slices slices each; every slice taken, none short, groups in fours.
+template <int F, int W>
+int launch_split(const GemmArgs& a, hipStream_t stream) {
+  constexpr int J = Fmt<F>::kElems / 8, PB = 4 * J;
+  const int MT = (a.M + 15) / 16;
+  if (MT * 4 * J > 16) return kNotSupported;  // a lane holds every piece of its wavefront's window twice: past 32 the kernel spills
+  const int gps = a.steps_per_wave >> 2;
+  if (a.steps % a.steps_per_wave != 0 || a.steps / a.steps_per_wave != W * a.walk_slices || (a.walk_slices * gps) % 4 != 0) return kNotSupported;
+  const size_t lds = static_cast<size_t>(W) * 4096 + static_cast<size_t>(W) * 2 * MT * 4 * PB * 256 + static_cast<size_t>(W) * a.walk_slices * MT * kWave * 16;
+  if (lds > kLdsMax) return kNotSupported;
+  const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
+  auto launch = [&](auto kernel) {
+    if (lds > 48 * 1024) allow_lds(reinterpret_cast<const void*>(kernel), kLdsMax);
+    hipLaunchKernelGGL(kernel, dim3(n_tiles), dim3(W * kWave), lds, stream, a);
+    return status_of(hipGetLastError());
+  };
+  auto with_mt = [&](auto mt_tag) {
+    constexpr int M16 = decltype(mt_tag)::value;
+    if constexpr (M16 * 4 * J > 16) return static_cast<int>(kNotSupported);
+    else return launch(walk_kernel<F, M16, W, kSplit>);
+  };
+  switch (MT) {
+    case 1: return with_mt(Tag<1>{});
+    case 2: return with_mt(Tag<2>{});
+    case 3: return with_mt(Tag<3>{});
+    default: return with_mt(Tag<4>{});
+  }
+}
+
 template <int F, int W>
 int launch_w(const GemmArgs& a, unsigned grid, hipStream_t stream) {
   constexpr int J = Fmt<F>::kElems / 8, PB = 4 * J;
   const int MT = (a.M + 15) / 16;
+  if (a.walk_split) {
+    if constexpr (W == 2 || W == 4) return launch_split<F, W>(a, stream);
+    else return kNotSupported;
+  }
   // A lane holds 2 MT 4 J / W staging pieces of 16 bytes: past 32 of them the kernel spills (measured 4 .. 20 x slower).
   if (MT * 4 * J / W > 16) return kNotSupported;
   // Eight wavefronts a workgroup have 256 registers each: room for four pieces (NVFP4 from 33 rows spills with six).

@@ -87,10 +87,10 @@ const std::map<std::string, Registered>& registry() {
       {"gemv_w_int8", {{"s1", "s2", "s4"}, LX_W_INT8}},
       {"gemv_w_fp8", {{"s1", "s2", "s4"}, LX_W_FP8}},
       {"gemv_w_nvfp4", {{"s1", "s2", "s4"}, LX_W_NVFP4}},
-      {"gemm_w_bf16", {{"tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts"}, -1}},
-      {"gemm_w_int8", {{"tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts"}, -1}},
-      {"gemm_w_fp8", {{"tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts"}, -1}},
-      {"gemm_w_nvfp4", {{"tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts"}, -1}},
+      {"gemm_w_bf16", {{"tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts", "walksplit"}, -1}},
+      {"gemm_w_int8", {{"tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts", "walksplit"}, -1}},
+      {"gemm_w_fp8", {{"tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts", "walksplit"}, -1}},
+      {"gemm_w_nvfp4", {{"tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts", "walksplit"}, -1}},
   };
   return *r;
 }

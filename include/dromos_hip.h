@@ -330,7 +330,7 @@ LX_API int lx_probe_empty(void* stream);
  * with s<S>, its K split, and lx_tune_set admits a variant for a shape only when its split is the
  * shape's own (so the rows' bits never depend on the table). The matrix-core products (lx_gemm_w, lx_gemm_skinny)
  * register theirs under gemm_w_<format>: which kernel family runs ("tiles", "walk1", "walk2", "walk4", "window",
- * "slab", "walkparts"); none changes a sum, so every one is admitted. */
+ * "slab", "walkparts", "walksplit"); none changes a sum, so every one is admitted. */
 LX_API int lx_arch(void);
 LX_API int lx_set_arch_override(int arch);
 LX_API int lx_tune_get(const char* kernel, int M, int N, int K);

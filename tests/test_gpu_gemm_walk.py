@@ -2,7 +2,7 @@
 tile) against float64 on the decoded values, and bit for bit against the tile kernels it replaces on the shapes it
 takes: the variant table forces each family ("gemm_w_<format>": 0 = the tile kernels, 1 .. 3 = walk with 1, 2, 4 tiles
 a workgroup, 4 / 5 = the tile kernels without / with the slab kernel, 6 = walks of single slices whose sums meet in the
-stream's partial-tile buffer), and no variant may change an output bit, a row's bits may not depend on the batch."""
+stream's partial-tile buffer, 7 = a tile's slices split over the wavefronts of a workgroup), and no variant may change an output bit, a row's bits may not depend on the batch."""
 
 import pytest
 import torch
@@ -36,10 +36,10 @@ def test_variants_are_registered(hip):
     hip.lib.lx_tune_variant_name.restype = ctypes.c_char_p
     for fmt in FMT:
         key = f"gemm_w_{fmt}".encode()
-        assert hip.lib.lx_tune_variants(key) == 7
-        assert [hip.lib.lx_tune_variant_name(key, v).decode() for v in range(7)] == ["tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts"]
-        assert all(hip.lib.lx_tune_set(key, 32, 4096, 4096, v) == 0 for v in range(7))  # none changes a sum: all admitted
-        assert hip.lib.lx_tune_set(key, 32, 4096, 4096, 7) == 803
+        assert hip.lib.lx_tune_variants(key) == 8
+        assert [hip.lib.lx_tune_variant_name(key, v).decode() for v in range(8)] == ["tiles", "walk1", "walk2", "walk4", "window", "slab", "walkparts", "walksplit"]
+        assert all(hip.lib.lx_tune_set(key, 32, 4096, 4096, v) == 0 for v in range(8))  # none changes a sum: all admitted
+        assert hip.lib.lx_tune_set(key, 32, 4096, 4096, 8) == 803
 
 
 @pytest.mark.parametrize("M", [9, 16, 17, 33, 48, 64])
@@ -53,7 +53,7 @@ def test_every_variant_gives_the_same_bits(hip, fmt, M):
         want = ops.gemv_reference(x, w.dense(), bias, 1.0, 0.0, None)
         wd, xd, bd = w.to("cuda"), x.cuda(), bias.cuda()
         outs = {}
-        for variant in (0, 1, 2, 3, 4, 5, 6, None):
+        for variant in (0, 1, 2, 3, 4, 5, 6, 7, None):
             force(hip, fmt, M, N, K, variant)
             y = torch.full((M, N), float("nan"), device="cuda")
             outs[variant] = ops.gemm_w(hip, xd, wd, MATH_BF16, bias=bd, y=y).clone()
@@ -71,7 +71,7 @@ def test_walk_rows_do_not_depend_on_the_batch(hip, fmt):
     force(hip, fmt, 64, N, K, 3)
     full = ops.gemm_skinny(hip, x, w)
     for M in (1, 8, 9, 16, 31, 40):
-        for variant in (2, 3):
+        for variant in (2, 3, 7):
             force(hip, fmt, M, N, K, variant)
             part = ops.gemm_skinny(hip, x[:M].contiguous(), w)
             assert torch.equal(part, full[:M]), f"rows of an M={M} call (variant {variant}) differ from the rows of the M=64 call"
@@ -91,7 +91,7 @@ def test_walk_epilogue_matrix(hip, fmt, bias_dtype, y_dtype, alpha, beta):
     bias = None if bias_dtype is None else torch.randn(N, generator=g).to(bias_dtype)
     y0 = torch.randn(M, N + pad, generator=g).to(y_dtype)
     want = ops.gemv_reference(xb[:, :K], w.dense(), bias, alpha, beta, y0[:, :N])
-    for variant in (0, 3):
+    for variant in (0, 3, 7):
         force(hip, fmt, M, N, K, variant)
         y = y0.clone().cuda()
         ops.gemm_w(hip, xb.cuda(), w.to("cuda"), MATH_BF16, bias=None if bias is None else bias.cuda(), y=y, alpha=alpha, beta=beta,
@@ -112,10 +112,11 @@ def test_walk_under_a_quantised_math(hip):
     w = random_weight(FORMATS["nvfp4"], N, K, 4).to("cuda")
     x = torch.randn(M, K, generator=torch.Generator().manual_seed(2)).to(torch.bfloat16).cuda()
     outs = []
-    for variant in (0, 3):
-        force(hip, "nvfp4", M, N, K, variant)
-        outs.append(ops.gemm_w(hip, x, w, MATH_FP8).clone())
+    for variant in (0, 3, 7):
+        force(hip, "nvfp4", M if variant != 7 else 16, N, K, variant)  # the split form takes NVFP4 up to 16 rows
+        outs.append(ops.gemm_w(hip, x if variant != 7 else x[:16].contiguous(), w, MATH_FP8).clone())
     assert torch.equal(outs[0].view(torch.int32), outs[1].view(torch.int32))
+    assert torch.equal(outs[0][:16].view(torch.int32), outs[2].view(torch.int32))
 
 
 class TuneProblem(__import__("ctypes").Structure):
@@ -179,7 +180,7 @@ def test_long_slices_in_several_slab_passes(hip, fmt, N, K):
     for M in (12, 33, 64):
         x = torch.randn(M, K, generator=g).to(torch.bfloat16)
         outs = {}
-        for variant in (0, 4, 5, 6, None):
+        for variant in (0, 4, 5, 6, 7, None):
             force(hip, fmt, M, N, K, variant)
             outs[variant] = ops.gemm_w(hip, x.cuda(), wd, MATH_BF16).clone()
         checks.check_product(outs[5].cpu(), ops.gemv_reference(x, dense, None, 1.0, 0.0, None))
@@ -211,3 +212,27 @@ def test_a_short_last_slice(hip, fmt, N, K):
         force(hip, fmt, 1, N, K, None)
         alone = ops.gemm_skinny(hip, x[M - 1 : M].cuda(), wd)
         assert torch.equal(alone[0].view(torch.int32), outs[None][M - 1].view(torch.int32))
+
+
+@pytest.mark.parametrize("fmt,N,K", [("fp8", 4096, 4096), ("int8", 4000, 4096), ("bf16", 2048, 2048), ("nvfp4", 4096, 4096), ("fp8", 4096, 8192)])
+def test_a_tile_split_over_a_workgroup(hip, fmt, N, K):
+    # Matrices of at most a tile per compute unit at 9 .. 32 rows: the rule takes the split form by itself (variant None),
+    # and its bits are the tile kernels' (variant 0) and the whole walk's (variant 2), a row's those of the row alone.
+    w = random_weight(FORMATS[fmt], N, K, N + K)
+    g = torch.Generator().manual_seed(K + 1)
+    wd = w.to("cuda")
+    dense = w.dense()
+    bias = torch.randn(N, generator=g)
+    for M in (9, 16, 17, 32):
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        outs = {}
+        for variant in (0, 2, 7, None):
+            force(hip, fmt, M, N, K, variant)
+            outs[variant] = ops.gemm_w(hip, x.cuda(), wd, MATH_BF16, bias=bias.cuda()).clone()
+        checks.check_product(outs[None].cpu(), ops.gemv_reference(x, dense, bias, 1.0, 0.0, None))
+        for variant, out in outs.items():
+            assert torch.equal(out.view(torch.int32), outs[0].view(torch.int32)), f"variant {variant} at {fmt} M={M}"
+        force(hip, fmt, 1, N, K, None)
+        alone = ops.gemm_skinny(hip, x[M - 1 : M].cuda(), wd)
+        force(hip, fmt, M, N, K, None)
+        assert torch.equal(alone[0].view(torch.int32), ops.gemm_skinny(hip, x.cuda(), wd)[M - 1].view(torch.int32))
