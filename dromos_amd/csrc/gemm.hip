@@ -1272,9 +1272,8 @@ bool launch_walk_split(GemmArgs a, int* status, hipStream_t stream) {
   if (spw < 8 || spw % 8 != 0 || a.steps % spw != 0) return false;
   const int slices = a.steps / spw;
   auto launch = [&](int w, int* st) {
-    if (slices % w != 0) return false;
     a.walk_split = w;
-    a.walk_slices = slices / w;
+    a.walk_slices = (slices + w - 1) / w;  // the last wavefront takes what is left
     if constexpr (F == LX_W_BF16) return launch_walk_bf16(a, w, st, stream);
     else if constexpr (F == LX_W_INT8) return launch_walk_int8(a, w, st, stream);
     else if constexpr (F == LX_W_FP8) return launch_walk_fp8(a, w, st, stream);
@@ -1288,7 +1287,8 @@ bool launch_walk_split(GemmArgs a, int* status, hipStream_t stream) {
 // rows 9.6 / 12.1 -> 12.3 / 18.1 us) and up to 32 rows of short K, where the whole walk is a few wavefronts' long chains:
 // 4096 x 4096 at 16 / 32 rows fp8 9.3 / 12.1 -> 7.3 / 10.2 us, int8 11.4 / 14.2 -> 7.7 / 10.6, bf16 10.6 / 14.4 -> 9.0 / 11.7,
 // nvfp4 at 16 rows 12.6 -> 9.6; 2048 x 4096 fp8 8.3 / 11.7 -> 6.5 / 9.7; 4096 x 8192 fp8 at 16 rows 13.3 -> 11.2 (at 32 rows
-// the single-slice walks and the slab kernel do better there). Two wavefronts a tile, whose windows leave room for two
+// the single-slice walks and the slab kernel do better there, as they do on long rows: 4096 x 14336 fp8 at 16 / 32 rows 16.8 /
+// 24.2 us split against 16.9 / 19.0). Two wavefronts a tile, whose windows leave room for two
 // workgroups a unit, do not carry it to 257 .. 512 tiles (6144 x 4096 fp8 at 32 rows 12.2 -> 15.0 us).
 inline bool walk_split_wanted(int M, int n_tiles, int64_t K, int tuned) {
   if (tuned >= 0) return tuned == kVariantWalkSplit;

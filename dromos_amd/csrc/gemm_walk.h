@@ -331,15 +331,18 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   }
 }
 
-// kSplit: W wavefronts on one tile, a.walk_slices slices each; every slice taken, none short, groups in fours.
+// kSplit: W wavefronts on one tile, a.walk_slices slices each (the last wavefront what is left, at least one); every
+// slice taken, none short, every wavefront's groups in fours.
 template <int F, int W>
 int launch_split(const GemmArgs& a, hipStream_t stream) {
   constexpr int J = Fmt<F>::kElems / 8, PB = 4 * J;
   const int MT = (a.M + 15) / 16;
   if (MT * 4 * J > 16) return kNotSupported;  // a lane holds every piece of its wavefront's window twice: past 32 the kernel spills
   const int gps = a.steps_per_wave >> 2;
-  if (a.steps % a.steps_per_wave != 0 || a.steps / a.steps_per_wave != W * a.walk_slices || (a.walk_slices * gps) % 4 != 0) return kNotSupported;
-  const size_t lds = static_cast<size_t>(W) * 4096 + static_cast<size_t>(W) * 2 * MT * 4 * PB * 256 + static_cast<size_t>(W) * a.walk_slices * MT * kWave * 16;
+  if (a.steps % a.steps_per_wave != 0 || a.walk_slices < 1) return kNotSupported;
+  const int slices = a.steps / a.steps_per_wave, left = slices - (W - 1) * a.walk_slices;
+  if (left < 1 || left > a.walk_slices || (a.walk_slices * gps) % 4 != 0 || (left * gps) % 4 != 0) return kNotSupported;
+  const size_t lds = static_cast<size_t>(W) * 4096 + static_cast<size_t>(W) * 2 * MT * 4 * PB * 256 + static_cast<size_t>(slices) * MT * kWave * 16;
   if (lds > kLdsMax) return kNotSupported;
   const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
   auto launch = [&](auto kernel) {
