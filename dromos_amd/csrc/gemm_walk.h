@@ -49,6 +49,13 @@ using Tag = std::integral_constant<int, N>;
 // (w + 1) * walk_slices), each with windows of its own (no barrier until the end: a wavefront stages what it reads), and
 // the slices' sums meet in LDS, where the first wavefront adds them in ascending order.
 constexpr int kPlain = 0, kRot = 1, kPart = 2, kSplit = 3;
+// A wavefront's own image: 4 KB of weights (16 rows x 256 bytes) and, for NVFP4, the group's block scales behind them
+// (16 rows x 32 bytes, the rows 40 bytes apart).
+constexpr int kScalePitch = 40;
+template <int F>
+constexpr int stage_bytes() {
+  return F == LX_W_NVFP4 ? 4096 + 16 * kScalePitch : 4096;
+}
 template <int F, int MT, int W, int MODE>
 __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   constexpr bool ROT = MODE == kRot, PART = MODE == kPart, SPLIT = MODE == kSplit;
@@ -66,8 +73,9 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   const int n0 = min(tile, n_tiles - 1) * kTileRows, valid = min(kTileRows, a.N - n0);  // a tile past the last repeats it
   const int g = lane >> 4, i = lane & 15;
   uint8_t* const lds = reinterpret_cast<uint8_t*>(lds4);
-  uint8_t* const stage = lds + wave * 4096;
-  uint8_t* const img = lds + W * 4096 + (SPLIT ? wave * 2 * kImage : 0);  // + buffer * kImage
+  constexpr int kStage = stage_bytes<F>();
+  uint8_t* const stage = lds + wave * kStage;
+  uint8_t* const img = lds + W * kStage + (SPLIT ? wave * 2 * kImage : 0);  // + buffer * kImage
   const int gps = a.steps_per_wave >> 2;  // groups of four load steps in a slice (the row's last slice may be shorter)
   const int row_groups = a.steps >> 2;    // and in a row
   const int slices = (row_groups + gps - 1) / gps;  // the slices that hold steps (a.S may count empty ones behind them: their sums are zero)
@@ -129,18 +137,17 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
 #pragma unroll
   for (int q = 0; q < 4; ++q) row_off[q] = static_cast<uint32_t>(min(4 * q + g, valid - 1)) * static_cast<uint32_t>(a.row_bytes) + i * 16u;
   u32x4 raw[4][4];
-  uint32_t sc[4][4];
+  // NVFP4: a group's block scales of the lane's row i, the eight bytes under piece group g (one load a group and lane,
+  // 32 contiguous bytes a row; a lane's fragments need bytes 8 u + 2 g, 8 u + 2 g + 1 of the row's 32 for step u, which
+  // the wavefront's image hands round).
+  u32x2 sc[4];
   auto issue_group = [&](auto slot, int gamma) {
     constexpr int SL = decltype(slot)::value;
     const int gq = group_of(gamma);
     const uint32_t c = static_cast<uint32_t>(gq) * 256u;  // a group is 256 bytes of a row
 #pragma unroll
     for (int q = 0; q < 4; ++q) raw[SL][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tile_w + (row_off[q] + c)));
-    if constexpr (F == LX_W_NVFP4) {
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-        sc[SL][u] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale) + (16 * gq + 4 * u + g));
-    }
+    if constexpr (F == LX_W_NVFP4) sc[SL] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(own_scale + 32 * gq + 8 * g));
   };
   // Row 4 q + g, chunk i goes into the wavefront's image; row i, chunk 4 s + g comes out.
   uint32_t put_at[4], get_at[4];
@@ -155,8 +162,16 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
     constexpr int SL = decltype(slot)::value;
 #pragma unroll
     for (int q = 0; q < 4; ++q) *reinterpret_cast<u32x4*>(stage + put_at[q]) = raw[SL][q];
+    if constexpr (F == LX_W_NVFP4) {
+      uint8_t* const srow = stage + 4096 + i * kScalePitch;
+      *reinterpret_cast<u32x2*>(srow + 8 * g) = sc[SL];
+      asm volatile("" ::: "memory");  // the wavefront's LDS instructions run in order: the reads see the writes
 #pragma unroll
-    for (int u = 0; u < 4; ++u) wsc[u] = F == LX_W_NVFP4 ? sc[SL][u] : 0u;
+      for (int u = 0; u < 4; ++u) wsc[u] = *reinterpret_cast<const uint16_t*>(srow + 8 * u + 2 * g);
+    } else {
+#pragma unroll
+      for (int u = 0; u < 4; ++u) wsc[u] = 0u;
+    }
   };
 
   // The activations first, then the weights: what is asked for first comes back first.
@@ -189,7 +204,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   // kRot: the wavefront's own [slice][mt][lane] behind the images; kSplit: the tile's, behind every wavefront's images.
-  f32x4* const sums = SPLIT ? reinterpret_cast<f32x4*>(lds + W * 4096 + W * 2 * kImage) + lane
+  f32x4* const sums = SPLIT ? reinterpret_cast<f32x4*>(lds + W * kStage + W * 2 * kImage) + lane
                             : reinterpret_cast<f32x4*>(img + 2 * kImage) + wave * (a.S * MT * kWave) + lane;
   f32x4 total[MT];
   // Where the walk is in the row: group `at` of slice `slice`, which ends before group `slice_end`.
@@ -342,7 +357,7 @@ int launch_split(const GemmArgs& a, hipStream_t stream) {
   if (a.steps % a.steps_per_wave != 0 || a.walk_slices < 1) return kNotSupported;
   const int slices = a.steps / a.steps_per_wave, left = slices - (W - 1) * a.walk_slices;
   if (left < 1 || left > a.walk_slices || (a.walk_slices * gps) % 4 != 0 || (left * gps) % 4 != 0) return kNotSupported;
-  const size_t lds = static_cast<size_t>(W) * 4096 + static_cast<size_t>(W) * 2 * MT * 4 * PB * 256 + static_cast<size_t>(slices) * MT * kWave * 16;
+  const size_t lds = static_cast<size_t>(W) * stage_bytes<F>() + static_cast<size_t>(W) * 2 * MT * 4 * PB * 256 + static_cast<size_t>(slices) * MT * kWave * 16;
   if (lds > kLdsMax) return kNotSupported;
   const unsigned n_tiles = static_cast<unsigned>((a.N + kTileRows - 1) / kTileRows);
   auto launch = [&](auto kernel) {
@@ -376,7 +391,7 @@ int launch_w(const GemmArgs& a, unsigned grid, hipStream_t stream) {
   // Eight wavefronts a workgroup have 256 registers each: room for four pieces (NVFP4 from 33 rows spills with six).
   if (W == 8 && MT * 4 * J / W > 4) return kNotSupported;
   if (MT * 4 * J % W != 0) return kNotSupported;  // the wavefronts share a window's pieces evenly
-  const size_t images = static_cast<size_t>(W) * 4096 + 2 * static_cast<size_t>(MT) * 4 * PB * 256;
+  const size_t images = static_cast<size_t>(W) * stage_bytes<F>() + 2 * static_cast<size_t>(MT) * 4 * PB * 256;
   const size_t with_sums = images + static_cast<size_t>(W) * a.S * MT * kWave * 16;
   const bool part = a.partial != nullptr;
   const bool rot = !part && with_sums <= kLdsMax;
@@ -422,6 +437,8 @@ bool launch_format(const GemmArgs& a, int W, int* status, hipStream_t stream) {
   if ((a.steps + spw - 1) / spw > S || static_cast<int64_t>(a.steps) * 4 * E != a.K || a.steps % 16 != 0) return false;
   if (static_cast<int64_t>(a.M) * a.xs.ld * 2 + static_cast<int64_t>(a.K) * 2 >= (int64_t{1} << 31)) return false;
   if (static_cast<int64_t>(kTileRows) * a.row_bytes >= (int64_t{1} << 31)) return false;
+  // NVFP4: a group's scales are read eight bytes at a time.
+  if (F == LX_W_NVFP4 && (reinterpret_cast<uintptr_t>(a.scale) % 8 != 0 || a.scale_row_bytes % 8 != 0)) return false;
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows;
   const unsigned grid = static_cast<unsigned>((n_tiles + W - 1) / W);
   int st;
