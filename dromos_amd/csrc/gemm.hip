@@ -1350,6 +1350,13 @@ int launch_skinny(GemmArgs a, hipStream_t stream) {
                                   : launch_skinny_x<F, 1, false, true>(a, lds, grid, threads, stream);
     }
   }
+  // No kernel with an activation image takes the call (rows too long for the image of the rows' count): the walks of
+  // single slices, whose windows fit whatever K is, before the kernel that reads its activations where they lie (NVFP4
+  // 4096 x 14336 at 1 / 8 rows in the batch-invariant mode 17.8 / 19.6 -> 16.5 / 16.7 us, 8192 x 14336 40.5 / 35.7 -> 24.0 / 24.2).
+  if (tuned < 0) {
+    int st = kOk;
+    if (launch_walk_parts<F>(a, &st, stream)) return st;
+  }
   const size_t lds = tile_lds_bytes(S, 1, MT);
   return a.xs.dtype == LX_F32 ? launch_skinny_x<F, MT, true, false>(a, lds, n_tiles, S * kWave, stream)
                               : launch_skinny_x<F, MT, false, false>(a, lds, n_tiles, S * kWave, stream);
