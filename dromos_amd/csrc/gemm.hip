@@ -1211,7 +1211,11 @@ bool try_walk(const GemmArgs& a, int* status, hipStream_t stream) {
     if (a.M <= 8 || n_tiles < 192) return false;
     if (walk_groups > 16) {
       if (n_tiles < 512 || walk_groups > 64) return false;
-      if (a.M <= (n_tiles >= 768 ? 32 + 8 : 24)) return false;  // many tiles: the windowed kernel holds on to 40 rows
+      // Many tiles: the windowed kernel holds on to 40 rows, except on the longest walks of the one-byte formats
+      // (14336 x 14336 fp8 at 16 / 32 rows: 46.0 / 58.8 -> 41.0 / 51.3 us) and on NVFP4, whose values are twice as many
+      // per byte (16384 x 14336 at 16 rows 55.5 -> 41.1 us, 14336 x 8192 at 48 rows 49.6 -> 41.2).
+      const bool long_walks = n_tiles >= 768 && (F == LX_W_NVFP4 || (F != LX_W_BF16 && walk_groups > 32));
+      if (!long_walks && a.M <= (n_tiles >= 768 ? 32 + 8 : 24)) return false;
     }
     W = n_tiles >= (walk_groups <= 16 ? 512 : 768) ? 4 : 2;
   }
@@ -1304,8 +1308,14 @@ bool walk_parts_wanted(int M, int n_tiles, int64_t K, int tuned) {
   if (tuned >= 0) return tuned == kVariantWalkParts;
   if (M <= 8) return false;
   const int mts = (M + 15) / 16;
-  if (mts >= 3) return F == LX_W_NVFP4 || K >= 8192;
-  if (F == LX_W_NVFP4 && mts == 2 && K >= 8192) return true;
+  if (F == LX_W_NVFP4) {
+    // With many tiles the whole walk of four tiles a workgroup is ahead at every row count (14336 x 4096 at 48 rows
+    // 32.8 -> 25.5 us); below that the single slices from 33 rows, from 17 rows for K >= 8192, from 9 for K >= 14336
+    // (8192 x 14336 at 16 rows 38.0 -> 29.5 us).
+    if (n_tiles >= 768) return false;
+    return mts >= 3 || (mts == 2 && K >= 8192) || K >= 14336;
+  }
+  if (mts >= 3) return K >= 8192;
   return K >= 28672 || (K >= 14336 && n_tiles <= 256);
 }
 
