@@ -26,6 +26,16 @@ namespace {
 
 constexpr int kMaxExperts = 1024;
 constexpr int kTileTokens = 64;  // activation rows a tile holds at most
+constexpr int kGroupedSplit = 4;  // wavefronts a tile at most: measured, four walking a tile in batches beat more with one batch each
+// The register budget the compiler works to, by what was measured (128 experts, 4096 x 1536, 32 and 64 tokens).
+// NVFP4's nibble decode and block scales do not fit the 128 registers a wavefront has when four share a SIMD: held
+// to them it spilled 256 (gate/up) and 78 (down) registers and ran a quarter slower than with two wavefronts a SIMD
+// and none spilled. FP8 is 2% faster with three a SIMD and no spills, INT8 4% faster with four and the few dozen
+// spills of the widest activation tiles.
+template <int F>
+constexpr int grouped_threads() {
+  return F == LX_W_NVFP4 ? kGroupedSplit * kWave : F == LX_W_FP8 ? 2 * kGroupedSplit * kWave : 4 * kGroupedSplit * kWave;
+}
 
 struct Tables {
   int* offsets;      // [E + 1] first position of each expert
@@ -152,7 +162,7 @@ struct GroupedArgs {
 };
 
 // gate/up for one (16 intermediate rows, tile of MT * 16 activation rows).
-template <int F, int MT>
+template <int F, int MT, bool WIDE>
 __device__ __forceinline__ void gate_up_tile(const GroupedArgs& a, int e, int g0, int rows, f32x4* lds) {
   const int lane = threadIdx.x & (kWave - 1);
   const int i0 = blockIdx.x * kTileRows;
@@ -166,7 +176,7 @@ __device__ __forceinline__ void gate_up_tile(const GroupedArgs& a, int e, int g0
     const int pair = a.t.order[g0 + min(mt * 16 + (lane & 15), rows - 1)];
     xrow[mt] = a.latent + static_cast<int64_t>(pair / a.top_k) * a.L;
   }
-  mfma_tile<F, 2, MT, kXGlobalBf16>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.L, lds, blockDim.x / kWave, __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), [] {}, [&](int mt, int q, f32x4(&sums)[2]) {
+  mfma_tile<F, 2, MT, kXGlobalBf16, WIDE>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.L, lds, blockDim.x / kWave, __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), [] {}, [&](int mt, int q, f32x4(&sums)[2]) {
     const int m = mt * 16 + (q & 15), i = i0 + 4 * (q >> 4);
     if (m >= rows) return;
     const int64_t stack_row = static_cast<int64_t>(e) * 2 * a.I + i;
@@ -183,21 +193,22 @@ __device__ __forceinline__ void gate_up_tile(const GroupedArgs& a, int e, int g0
   });
 }
 
-template <int F>
-__global__ void __launch_bounds__(kMaxSplit* kWave) grouped_gate_up_kernel(const GroupedArgs a) {
+// WIDE: NVFP4 block scales read eight bytes at a time (the launcher has checked that the stack allows it).
+template <int F, bool WIDE>
+__global__ void __launch_bounds__(grouped_threads<F>()) grouped_gate_up_kernel(const GroupedArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
   const int tile = blockIdx.y;
   if (tile >= *a.t.n_tiles) return;
   const int e = a.t.tile_expert[tile], g0 = a.t.tile_begin[tile], rows = a.t.tile_rows[tile];
   switch ((rows + 15) / 16) {
-    case 1: gate_up_tile<F, 1>(a, e, g0, rows, lds4); break;
-    case 2: gate_up_tile<F, 2>(a, e, g0, rows, lds4); break;
-    case 3: gate_up_tile<F, 3>(a, e, g0, rows, lds4); break;
-    default: gate_up_tile<F, 4>(a, e, g0, rows, lds4); break;
+    case 1: gate_up_tile<F, 1, WIDE>(a, e, g0, rows, lds4); break;
+    case 2: gate_up_tile<F, 2, WIDE>(a, e, g0, rows, lds4); break;
+    case 3: gate_up_tile<F, 3, WIDE>(a, e, g0, rows, lds4); break;
+    default: gate_up_tile<F, 4, WIDE>(a, e, g0, rows, lds4); break;
   }
 }
 
-template <int F, int MT>
+template <int F, int MT, bool WIDE>
 __device__ __forceinline__ void down_tile(const GroupedArgs& a, int e, int g0, int rows, f32x4* lds) {
   const int lane = threadIdx.x & (kWave - 1);
   const int l0 = blockIdx.x * kTileRows;
@@ -206,7 +217,7 @@ __device__ __forceinline__ void down_tile(const GroupedArgs& a, int e, int g0, i
   const void* xrow[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) xrow[mt] = a.down_in + static_cast<int64_t>(g0 + min(mt * 16 + (lane & 15), rows - 1)) * a.I;
-  mfma_tile<F, 1, MT, kXGlobalBf16>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.I, lds, blockDim.x / kWave, __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), [] {}, [&](int mt, int q, f32x4(&sums)[1]) {
+  mfma_tile<F, 1, MT, kXGlobalBf16, WIDE>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.I, lds, blockDim.x / kWave, __builtin_amdgcn_readfirstlane(threadIdx.x / kWave), [] {}, [&](int mt, int q, f32x4(&sums)[1]) {
     const int m = mt * 16 + (q & 15), l = l0 + 4 * (q >> 4);
     if (m >= rows) return;
     const int64_t stack_row = static_cast<int64_t>(e) * a.L + l;
@@ -217,17 +228,17 @@ __device__ __forceinline__ void down_tile(const GroupedArgs& a, int e, int g0, i
   });
 }
 
-template <int F>
-__global__ void __launch_bounds__(kMaxSplit* kWave) grouped_down_kernel(const GroupedArgs a) {
+template <int F, bool WIDE>
+__global__ void __launch_bounds__(grouped_threads<F>()) grouped_down_kernel(const GroupedArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
   const int tile = blockIdx.y;
   if (tile >= *a.t.n_tiles) return;
   const int e = a.t.tile_expert[tile], g0 = a.t.tile_begin[tile], rows = a.t.tile_rows[tile];
   switch ((rows + 15) / 16) {
-    case 1: down_tile<F, 1>(a, e, g0, rows, lds4); break;
-    case 2: down_tile<F, 2>(a, e, g0, rows, lds4); break;
-    case 3: down_tile<F, 3>(a, e, g0, rows, lds4); break;
-    default: down_tile<F, 4>(a, e, g0, rows, lds4); break;
+    case 1: down_tile<F, 1, WIDE>(a, e, g0, rows, lds4); break;
+    case 2: down_tile<F, 2, WIDE>(a, e, g0, rows, lds4); break;
+    case 3: down_tile<F, 3, WIDE>(a, e, g0, rows, lds4); break;
+    default: down_tile<F, 4, WIDE>(a, e, g0, rows, lds4); break;
   }
 }
 
@@ -286,7 +297,7 @@ int launch_stage(Kernel kernel, GroupedArgs a, int64_t K, int NT, int out_rows, 
   a.chunks = static_cast<int>(a.row_bytes / 16);
   a.steps = load_steps_for<F>(K);
   int S = split_for<F>(K, NT);
-  if (S > 4) S = 4;  // measured: four wavefronts walking a tile in batches beat more wavefronts with one batch each
+  if (S > kGroupedSplit) S = kGroupedSplit;
   a.steps_per_wave = (a.steps + S - 1) / S;
   const int64_t P = static_cast<int64_t>(a.T) * a.top_k;
   const int mt_max = static_cast<int>(((P < kTileTokens ? P : kTileTokens) + 15) / 16);
@@ -358,10 +369,14 @@ int experts_grouped(const void* latent, const int32_t* ids, const float* weights
   const int tiles = max_tiles(P, E);
   int st;
   switch (gate_up.type) {
-    case LX_W_BF16: st = launch_stage<LX_W_BF16>(grouped_gate_up_kernel<LX_W_BF16>, a, L, 2, I, tiles, s); break;
-    case LX_W_INT8: st = launch_stage<LX_W_INT8>(grouped_gate_up_kernel<LX_W_INT8>, a, L, 2, I, tiles, s); break;
-    case LX_W_FP8: st = launch_stage<LX_W_FP8>(grouped_gate_up_kernel<LX_W_FP8>, a, L, 2, I, tiles, s); break;
-    default: st = launch_stage<LX_W_NVFP4>(grouped_gate_up_kernel<LX_W_NVFP4>, a, L, 2, I, tiles, s); break;
+    case LX_W_BF16: st = launch_stage<LX_W_BF16>(grouped_gate_up_kernel<LX_W_BF16, false>, a, L, 2, I, tiles, s); break;
+    case LX_W_INT8: st = launch_stage<LX_W_INT8>(grouped_gate_up_kernel<LX_W_INT8, false>, a, L, 2, I, tiles, s); break;
+    case LX_W_FP8: st = launch_stage<LX_W_FP8>(grouped_gate_up_kernel<LX_W_FP8, false>, a, L, 2, I, tiles, s); break;
+    default:
+      st = wide_scales_fit(a.gu.scale, L / 16, static_cast<int>(row_bytes<LX_W_NVFP4>(L) / 16))
+               ? launch_stage<LX_W_NVFP4>(grouped_gate_up_kernel<LX_W_NVFP4, true>, a, L, 2, I, tiles, s)
+               : launch_stage<LX_W_NVFP4>(grouped_gate_up_kernel<LX_W_NVFP4, false>, a, L, 2, I, tiles, s);
+      break;
   }
   if (st) return st;
   if (quantised) {
@@ -374,10 +389,14 @@ int experts_grouped(const void* latent, const int32_t* ids, const float* weights
     a.xs2 = scale2;
   }
   switch (down.type) {
-    case LX_W_BF16: st = launch_stage<LX_W_BF16>(grouped_down_kernel<LX_W_BF16>, a, I, 1, L, tiles, s); break;
-    case LX_W_INT8: st = launch_stage<LX_W_INT8>(grouped_down_kernel<LX_W_INT8>, a, I, 1, L, tiles, s); break;
-    case LX_W_FP8: st = launch_stage<LX_W_FP8>(grouped_down_kernel<LX_W_FP8>, a, I, 1, L, tiles, s); break;
-    default: st = launch_stage<LX_W_NVFP4>(grouped_down_kernel<LX_W_NVFP4>, a, I, 1, L, tiles, s); break;
+    case LX_W_BF16: st = launch_stage<LX_W_BF16>(grouped_down_kernel<LX_W_BF16, false>, a, I, 1, L, tiles, s); break;
+    case LX_W_INT8: st = launch_stage<LX_W_INT8>(grouped_down_kernel<LX_W_INT8, false>, a, I, 1, L, tiles, s); break;
+    case LX_W_FP8: st = launch_stage<LX_W_FP8>(grouped_down_kernel<LX_W_FP8, false>, a, I, 1, L, tiles, s); break;
+    default:
+      st = wide_scales_fit(a.dn.scale, I / 16, static_cast<int>(row_bytes<LX_W_NVFP4>(I) / 16))
+               ? launch_stage<LX_W_NVFP4>(grouped_down_kernel<LX_W_NVFP4, true>, a, I, 1, L, tiles, s)
+               : launch_stage<LX_W_NVFP4>(grouped_down_kernel<LX_W_NVFP4, false>, a, I, 1, L, tiles, s);
+      break;
   }
   if (st) return st;
   const int64_t items = static_cast<int64_t>(T) * L;

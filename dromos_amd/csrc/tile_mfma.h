@@ -178,10 +178,11 @@ struct TileRows {
   int valid;
 };
 
-// A wavefront's private LDS: the staging image of one tile's 4 load steps (16 rows x 16 chunks, the rows 16
-// bytes apart in the banks so that both the row-wise writes and the fragment reads are conflict-free), reused
-// afterwards for the wavefront's partial sums.
-constexpr int kStagePitch = 16 * 16 + 16;
+// A wavefront's private LDS: the staging image of one tile's 4 load steps (16 rows x 16 chunks, and behind each
+// row room for its 32 bytes of NVFP4 block scales; the rows 48 bytes apart in the banks so that both the row-wise
+// writes and the fragment reads are conflict-free), reused afterwards for the wavefront's partial sums.
+constexpr int kStageRow = 16 * 16;
+constexpr int kStagePitch = kStageRow + 48;
 constexpr int kStageBytes = kTileRows * kStagePitch;
 
 template <int NT, int MT>
@@ -192,6 +193,12 @@ constexpr int wave_region_bytes() {
 inline size_t tile_lds_bytes(int S, int NT, int MT) {
   const size_t partial = static_cast<size_t>(NT) * MT * kWave * 16;
   return S * (partial > kStageBytes ? partial : static_cast<size_t>(kStageBytes));
+}
+
+// Whether the block scales of every row of a stack of NVFP4 rows can be read eight bytes (a load step's four
+// chunks) at a time: whole steps in a row, and every row's scales eight-byte aligned.
+inline bool wide_scales_fit(const void* scale, int64_t scale_row_bytes, int chunks) {
+  return chunks > 0 && chunks % 4 == 0 && scale_row_bytes % 8 == 0 && reinterpret_cast<uintptr_t>(scale) % 8 == 0;
 }
 
 // Orders this wavefront's LDS accesses as written (the hardware runs a wavefront's LDS instructions in order;
@@ -208,7 +215,8 @@ struct WeightBatch {
   static constexpr int WU = kLoadsInFlight / NT;
   static_assert(WU % 4 == 0, "weight steps are staged four at a time");
   u32x4 raw[WU / 4][NT][4];
-  uint32_t sc[WU][NT];
+  uint32_t sc[WU][NT];     // NVFP4 block scales a step at a time (rows whose scales do not come in whole, aligned groups)
+  u32x2 scq[WU / 4][NT];   // ... or a 4-step group of one row's at once: lane (g, i) holds step g's eight bytes of row i
 };
 
 // One 16-byte chunk of byte weights against the same 16 k of byte activations, added to acc.
@@ -234,8 +242,9 @@ __device__ __forceinline__ f32x4 byte_mfma(const i32x4& w, const i32x4& x, const
 // contiguous bytes of each of four rows (lane -> row 4q + lane / 16, chunk lane % 16 of a 4-step group). They pass
 // through `stage` (this wavefront's kStageBytes of LDS) to reach the lanes that feed them to the matrix
 // instruction: lane (g, i) takes chunk 4s + g of row i for step s of the group.
-template <int F, int NT>
+template <int F, int NT, bool WIDE = false>
 struct TileStream {
+  static_assert(!WIDE || F == LX_W_NVFP4, "only NVFP4 has block scales to read");
   static constexpr int E = Fmt<F>::kElems;
   static constexpr int J = E / 8;  // matrix instructions per load step
   static constexpr int WU = WeightBatch<F, NT>::WU;
@@ -244,7 +253,13 @@ struct TileStream {
   const uint8_t* stage_row[NT][4];
   u32x4* put;        // + q * 4 rows
   const u32x4* get;  // + s * 4 chunks
+  u32x2* sc_put;     // a group's block scales travel behind its rows
+  const uint8_t* sc_get;  // + s * 8 bytes
   int chunks, g, i;
+  // NVFP4 block scales are two bytes a chunk. Read a chunk at a time they are 64 two-byte loads of 16 different
+  // rows an instruction; read eight bytes a lane (WIDE: a step's four chunks) they are a quarter of the
+  // instructions and whole 32-byte runs. That needs whole steps in a row and eight-byte alignment of every row's
+  // scales: wide_scales_fit() says whether a stack of rows has both.
 
   __device__ __forceinline__ TileStream(const TileRows (&tiles)[NT], int64_t row_bytes, int64_t scale_row_bytes, int chunks_,
                                         uint8_t* stage)
@@ -260,6 +275,8 @@ struct TileStream {
     }
     put = reinterpret_cast<u32x4*>(stage + g * kStagePitch + i * 16);
     get = reinterpret_cast<const u32x4*>(stage + i * kStagePitch + g * 16);
+    sc_put = reinterpret_cast<u32x2*>(stage + i * kStagePitch + kStageRow + g * 8);
+    sc_get = stage + i * kStagePitch + kStageRow + g * 2;
   }
 
   // Asks for the batch of load steps [tb, tb + WU).
@@ -274,14 +291,20 @@ struct TileStream {
         for (int q = 0; q < 4; ++q)
           wb.raw[grp][n][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(stage_row[n][q]) + c);
     }
+    if constexpr (WIDE) {
 #pragma unroll
-    for (int u = 0; u < WU; ++u)
+      for (int grp = 0; grp < G; ++grp) {
+        const int step = min(tb + 4 * grp + g, chunks / 4 - 1);  // past the row's end: its last step's, unused
 #pragma unroll
-      for (int n = 0; n < NT; ++n) {
-        wb.sc[u][n] = 0;
-        if constexpr (F == LX_W_NVFP4)
-          wb.sc[u][n] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale[n]) + min(4 * (tb + u) + g, chunks - 1));
+        for (int n = 0; n < NT; ++n) wb.scq[grp][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(own_scale[n]) + step);
       }
+    } else if constexpr (F == LX_W_NVFP4) {
+#pragma unroll
+      for (int u = 0; u < WU; ++u)
+#pragma unroll
+        for (int n = 0; n < NT; ++n)
+          wb.sc[u][n] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale[n]) + min(4 * (tb + u) + g, chunks - 1));
+    }
   }
 
   // acc[t][mt] += the batch at tb times activation tile mt; steps from t_end on count for nothing (k_end = the
@@ -305,6 +328,7 @@ struct TileStream {
     if constexpr (XS != kXLds) load_x(0);  // in flight together with the weights
     // Four steps at a time: through the staging image into fragment order, then into the matrix instructions.
     u32x4 wv[WU][NT];
+    uint32_t scv[WU][NT];
 #pragma unroll
     for (int ub = 0; ub < WU; ub += U) {
       if (XS != kXLds && ub > 0) load_x(ub);
@@ -316,9 +340,18 @@ struct TileStream {
           for (int n = 0; n < NT; ++n) {
 #pragma unroll
             for (int q = 0; q < 4; ++q) put[q * (4 * kStagePitch / 16)] = wb.raw[grp][n][q];
+            // Row i's 32 scale bytes of the group behind image row i; lane (g, i) takes chunk 4 s + g's two of
+            // them for step s.
+            if constexpr (WIDE) *sc_put = wb.scq[grp][n];
             wave_lds_order();
 #pragma unroll
-            for (int sstep = 0; sstep < 4; ++sstep) wv[4 * grp + sstep][n] = get[sstep * 4];
+            for (int sstep = 0; sstep < 4; ++sstep) {
+              wv[4 * grp + sstep][n] = get[sstep * 4];
+              if constexpr (WIDE)
+                scv[4 * grp + sstep][n] = *reinterpret_cast<const uint16_t*>(sc_get + 8 * sstep);
+              else
+                scv[4 * grp + sstep][n] = F == LX_W_NVFP4 ? wb.sc[4 * grp + sstep][n] : 0;
+            }
             wave_lds_order();
           }
         }
@@ -328,7 +361,7 @@ struct TileStream {
         for (int j = 0; j < J; ++j) {
 #pragma unroll
           for (int n = 0; n < NT; ++n) {
-            const bf16x8 wf = weight_fragment<F>(wv[ub + u][n], wb.sc[ub + u][n], j);
+            const bf16x8 wf = weight_fragment<F>(wv[ub + u][n], scv[ub + u][n], j);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
               acc[n][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, x_operand<XS, MASK>(xf[u][j][mt], k0 + 8 * j, k_end), acc[n][mt], 0, 0, 0);
@@ -396,11 +429,11 @@ struct TileStream {
 // Steps past the slice's end (a last, partial batch) run on re-read weights against zero activations. An LDS
 // image is zero from K to the end of the row's last batch, and with it every slice but the row's last is whole
 // batches (the caller sees to both), so nothing is masked.
-template <int F, int NT, int MT, int XS, class Between>
+template <int F, int NT, int MT, int XS, bool WIDE = false, class Between>
 __device__ __forceinline__ void mfma_slice(const TileRows (&tiles)[NT], int64_t row_bytes, int64_t scale_row_bytes, int chunks,
                                            int t_begin, int t_end, const void* const (&xrow)[MT], int K, f32x4 (&acc)[NT][MT],
                                            uint8_t* stage, Between&& between) {
-  const TileStream<F, NT> ts(tiles, row_bytes, scale_row_bytes, chunks, stage);
+  const TileStream<F, NT, WIDE> ts(tiles, row_bytes, scale_row_bytes, chunks, stage);
   WeightBatch<F, NT> wb;
   if (t_begin < t_end) ts.issue(wb, t_begin);
   between();
@@ -417,7 +450,7 @@ __device__ __forceinline__ void mfma_slice(const TileRows (&tiles)[NT], int64_t 
 // epi(mt, q, sums) is called once for every (activation tile mt, lane slot q) with the NT finished sums:
 // sums[t][r] belongs to weight row 4 * (q / 16) + r of tile t and activation row mt * 16 + q % 16.
 // Every wavefront of the workgroup must make the call: it holds workgroup barriers.
-template <int F, int NT, int MT, int XS, class Between, class Epi>
+template <int F, int NT, int MT, int XS, bool WIDE = false, class Between, class Epi>
 __device__ __forceinline__ void mfma_tile(const TileRows (&tiles)[NT], int64_t row_bytes, int64_t scale_row_bytes, int chunks,
                                           int steps, int steps_per_wave, const void* const (&xrow)[MT], int K, f32x4* lds, int S,
                                           int slice, Between&& between, Epi&& epi) {
@@ -430,7 +463,7 @@ __device__ __forceinline__ void mfma_tile(const TileRows (&tiles)[NT], int64_t r
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) acc[n][mt] = f32x4{0.f, 0.f, 0.f, 0.f};
   const int t_begin = min(steps, slice * steps_per_wave), t_end = min(steps, t_begin + steps_per_wave);
-  mfma_slice<F, NT, MT, XS>(tiles, row_bytes, scale_row_bytes, chunks, t_begin, t_end, xrow, K, acc, base + slice * kRegion, between);
+  mfma_slice<F, NT, MT, XS, WIDE>(tiles, row_bytes, scale_row_bytes, chunks, t_begin, t_end, xrow, K, acc, base + slice * kRegion, between);
   if (S == 1) {
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {

@@ -44,6 +44,25 @@ def make(fmt, T, L, I, E, top_k, seed):
     return latent.cuda(), ids.cuda(), weights.cuda(), gu, dn
 
 
+def test_nvfp4_block_scales_read_either_way_give_the_same_bits(hip):
+    # Block scales are read eight bytes at a time where every row's lie eight-byte aligned and rows are whole load
+    # steps (128 values), two bytes at a time otherwise: the same stacks two bytes off, and rows of 2.25 and 1.25 steps.
+    L, I, E, top_k = 1024, 512, 16, 4
+    latent, ids, weights, gu, dn = make("nvfp4", 40, L, I, E, top_k, 5)
+    want = ops.experts_grouped(hip, latent, ids, weights, gu, dn, I, E, top_k)
+
+    def shifted(w):
+        flat = torch.zeros(w.scale.numel() * w.scale.element_size() + 8, dtype=torch.uint8, device="cuda")
+        view = flat[2 : 2 + w.scale.numel() * w.scale.element_size()].view(w.scale.dtype).view(w.scale.shape)
+        view.copy_(w.scale)
+        assert view.data_ptr() % 8 == 2
+        return Weight(w.fmt, w.data, view, w.glob, w.expert_global)
+
+    got = ops.experts_grouped(hip, latent, ids, weights, shifted(gu), shifted(dn), I, E, top_k)
+    assert torch.equal(got, want)
+    checks.grouped_case(hip, "nvfp4", 23, 288, 160, 8, 2, seed=9)
+
+
 @pytest.mark.parametrize("fmt", FMT)
 def test_rows_do_not_depend_on_the_batch(hip, fmt):
     L, I, E, top_k = 1024, 512, 32, 4
