@@ -27,15 +27,17 @@ namespace {
 constexpr int kMaxExperts = 1024;
 constexpr int kTileTokens = 64;  // activation rows a tile holds at most
 constexpr int kGroupedSplit = 4;  // wavefronts a tile at most: measured, four walking a tile in batches beat more with one batch each
-// The register budget the compiler works to, by what was measured (128 experts, 4096 x 1536, 32 and 64 tokens).
-// NVFP4's nibble decode and block scales do not fit the 128 registers a wavefront has when four share a SIMD: held
-// to them it spilled 256 (gate/up) and 78 (down) registers and ran a quarter slower than with two wavefronts a SIMD
-// and none spilled. FP8 is 2% faster with three a SIMD and no spills, INT8 4% faster with four and the few dozen
-// spills of the widest activation tiles.
+// Wavefronts a SIMD the stage kernels are compiled for at least (512 registers a SIMD lane: 128 each at four, 168 at three), by
+// what was measured (128 experts, 4096 x 1536, 32 and 64 tokens). NVFP4's nibble decode and block scales do not fit
+// 128 registers: held to them it spilled 256 (gate/up) and 78 (down) and ran 470 us; with all it asks for (220, two
+// wavefronts a SIMD) 390; at three a SIMD, a few dozen spilled in the wide activation tiles, 331. FP8 is 2% faster
+// with three and no spills, INT8 4% faster with four and the few dozen spills of the widest activation tiles.
 template <int F>
-constexpr int grouped_threads() {
-  return F == LX_W_NVFP4 ? kGroupedSplit * kWave : F == LX_W_FP8 ? 2 * kGroupedSplit * kWave : 4 * kGroupedSplit * kWave;
+constexpr int grouped_waves() {
+  return F == LX_W_NVFP4 || F == LX_W_FP8 ? 3 : 4;
 }
+#define DRO_GROUPED_KERNEL(F) \
+  __global__ void __launch_bounds__(kGroupedSplit* kWave) __attribute__((amdgpu_waves_per_eu(grouped_waves<F>())))
 
 struct Tables {
   int* offsets;      // [E + 1] first position of each expert
@@ -195,7 +197,7 @@ __device__ __forceinline__ void gate_up_tile(const GroupedArgs& a, int e, int g0
 
 // WIDE: NVFP4 block scales read eight bytes at a time (the launcher has checked that the stack allows it).
 template <int F, bool WIDE>
-__global__ void __launch_bounds__(grouped_threads<F>()) grouped_gate_up_kernel(const GroupedArgs a) {
+DRO_GROUPED_KERNEL(F) grouped_gate_up_kernel(const GroupedArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
   const int tile = blockIdx.y;
   if (tile >= *a.t.n_tiles) return;
@@ -229,7 +231,7 @@ __device__ __forceinline__ void down_tile(const GroupedArgs& a, int e, int g0, i
 }
 
 template <int F, bool WIDE>
-__global__ void __launch_bounds__(grouped_threads<F>()) grouped_down_kernel(const GroupedArgs a) {
+DRO_GROUPED_KERNEL(F) grouped_down_kernel(const GroupedArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
   const int tile = blockIdx.y;
   if (tile >= *a.t.n_tiles) return;
