@@ -30,8 +30,13 @@ namespace {
 // x_pitch = that + 8 elements apart (16 bytes off a multiple of the banks' span, so the 16 rows of a fragment read
 // fall into different banks). A workgroup then holds `tiles_per_wg` tiles of S wavefronts each, which share the
 // image. Otherwise (any M up to 64) the fragments are read from global memory and a workgroup is one tile.
-template <int F, int MT, bool XF32, bool XL>
-__global__ void __launch_bounds__(kMaxSplit* kWave) skinny_kernel(const GemmArgs a) {
+// LEAN (NVFP4, whose nibble decode does not fit the 128 registers a wavefront has in a workgroup of sixteen: 90 to 256
+// registers spilled with two to four activation tiles): the same kernel compiled for the workgroups of at most LEAN = 4
+// or 8 wavefronts that most shapes ask for (at 4, three wavefronts a SIMD, what measured best in the grouped experts,
+// which are this code), with the block scales read eight bytes at a time (the launcher checks that they can be).
+template <int F, int MT, bool XF32, bool XL, int LEAN = 0>
+__global__ void __launch_bounds__((LEAN ? LEAN : kMaxSplit) * kWave) __attribute__((amdgpu_waves_per_eu(LEAN == 4 ? 3 : 1)))
+skinny_kernel(const GemmArgs a) {
   extern __shared__ __align__(16) f32x4 lds4[];
   static_assert(!XL || MT == 1, "only one activation tile is staged in LDS");
   constexpr int kRegion = wave_region_bytes<1, MT>();
@@ -111,8 +116,8 @@ __global__ void __launch_bounds__(kMaxSplit* kWave) skinny_kernel(const GemmArgs
     }
   };
   constexpr int XS = XL ? kXLds : XF32 ? kXGlobalF32 : kXGlobalBf16;
-  mfma_tile<F, 1, MT, XS>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.K,
-                          reinterpret_cast<f32x4*>(lds_bytes + tile_in_wg * S * kRegion), S, slice, between,
+  mfma_tile<F, 1, MT, XS, LEAN != 0>(tiles, a.row_bytes, a.scale_row_bytes, a.chunks, a.steps, a.steps_per_wave, xrow, a.K,
+                                     reinterpret_cast<f32x4*>(lds_bytes + tile_in_wg * S * kRegion), S, slice, between,
                           [&](int mt, int q, f32x4(&sums)[1]) {
     const int m = mt * 16 + (q & 15), nq = n0 + 4 * (q >> 4);  // q % 64 == lane: rf and bs are this slot's
     if (m < a.M && tile_live) {
@@ -1171,9 +1176,9 @@ __global__ void __launch_bounds__(256) gemm_plain_kernel(const GemmArgs a, int w
   }
 }
 
-template <int F, int MT, bool XF32, bool XL>
+template <int F, int MT, bool XF32, bool XL, int LEAN = 0>
 int launch_skinny_x(const GemmArgs& a, size_t lds, unsigned grid, unsigned threads, hipStream_t stream) {
-  auto kernel = skinny_kernel<F, MT, XF32, XL>;
+  auto kernel = skinny_kernel<F, MT, XF32, XL, LEAN>;
   if (lds > 48 * 1024) {
     static thread_local bool raised = false;
     if (!raised) {
@@ -1368,6 +1373,15 @@ int launch_skinny(GemmArgs a, hipStream_t stream) {
     if (launch_walk_parts<F>(a, &st, stream)) return st;
   }
   const size_t lds = tile_lds_bytes(S, 1, MT);
+  if constexpr (F == LX_W_NVFP4) {
+    if (S <= 8 && wide_scales_fit(a.scale, a.scale_row_bytes, a.chunks)) {
+      if (S <= 4)
+        return a.xs.dtype == LX_F32 ? launch_skinny_x<F, MT, true, false, 4>(a, lds, n_tiles, S * kWave, stream)
+                                    : launch_skinny_x<F, MT, false, false, 4>(a, lds, n_tiles, S * kWave, stream);
+      return a.xs.dtype == LX_F32 ? launch_skinny_x<F, MT, true, false, 8>(a, lds, n_tiles, S * kWave, stream)
+                                  : launch_skinny_x<F, MT, false, false, 8>(a, lds, n_tiles, S * kWave, stream);
+    }
+  }
   return a.xs.dtype == LX_F32 ? launch_skinny_x<F, MT, true, false>(a, lds, n_tiles, S * kWave, stream)
                               : launch_skinny_x<F, MT, false, false>(a, lds, n_tiles, S * kWave, stream);
 }

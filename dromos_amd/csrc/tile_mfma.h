@@ -298,12 +298,15 @@ struct TileStream {
 #pragma unroll
         for (int n = 0; n < NT; ++n) wb.scq[grp][n] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(own_scale[n]) + step);
       }
-    } else if constexpr (F == LX_W_NVFP4) {
+    } else {
 #pragma unroll
       for (int u = 0; u < WU; ++u)
 #pragma unroll
-        for (int n = 0; n < NT; ++n)
-          wb.sc[u][n] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale[n]) + min(4 * (tb + u) + g, chunks - 1));
+        for (int n = 0; n < NT; ++n) {
+          wb.sc[u][n] = 0;
+          if constexpr (F == LX_W_NVFP4)
+            wb.sc[u][n] = __builtin_nontemporal_load(reinterpret_cast<const uint16_t*>(own_scale[n]) + min(4 * (tb + u) + g, chunks - 1));
+        }
     }
   }
 
@@ -347,10 +350,7 @@ struct TileStream {
 #pragma unroll
             for (int sstep = 0; sstep < 4; ++sstep) {
               wv[4 * grp + sstep][n] = get[sstep * 4];
-              if constexpr (WIDE)
-                scv[4 * grp + sstep][n] = *reinterpret_cast<const uint16_t*>(sc_get + 8 * sstep);
-              else
-                scv[4 * grp + sstep][n] = F == LX_W_NVFP4 ? wb.sc[4 * grp + sstep][n] : 0;
+              if constexpr (WIDE) scv[4 * grp + sstep][n] = *reinterpret_cast<const uint16_t*>(sc_get + 8 * sstep);
             }
             wave_lds_order();
           }
@@ -361,7 +361,7 @@ struct TileStream {
         for (int j = 0; j < J; ++j) {
 #pragma unroll
           for (int n = 0; n < NT; ++n) {
-            const bf16x8 wf = weight_fragment<F>(wv[ub + u][n], scv[ub + u][n], j);
+            const bf16x8 wf = weight_fragment<F>(wv[ub + u][n], WIDE ? scv[ub + u][n] : wb.sc[ub + u][n], j);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt)
               acc[n][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf, x_operand<XS, MASK>(xf[u][j][mt], k0 + 8 * j, k_end), acc[n][mt], 0, 0, 0);

@@ -57,7 +57,9 @@ def test_gemm_w_k_boundaries(hip, fmt, K):
     gemm_case(hip, fmt, 12, 21, K, seed=K)
 
 
-@pytest.mark.parametrize("N,K", [(10304, 2048), (2048, 4096), (256, 6400), (8, 2048), (1, 512)])
+# The last two: rows that are not whole walks (K = 11 and 61 NVFP4 load steps) on matrices with the tiles for few,
+# long slices: the tile kernel that reads its activations where they lie, in workgroups of at most 4 and 8 wavefronts.
+@pytest.mark.parametrize("N,K", [(10304, 2048), (2048, 4096), (256, 6400), (8, 2048), (1, 512), (11008, 1408), (4096, 7808)])
 @pytest.mark.parametrize("fmt", FMT)
 def test_gemm_w_decode_shapes(hip, fmt, N, K):
     gemm_case(hip, fmt, 32, N, K, seed=N % 89)
@@ -98,7 +100,7 @@ def test_other_maths_and_arguments(hip):
 
 
 @pytest.mark.parametrize("fmt", FMT)
-@pytest.mark.parametrize("N,K", [(1024, 2048), (300, 4096), (2048, 1024)])
+@pytest.mark.parametrize("N,K", [(1024, 2048), (300, 4096), (2048, 1024), (11008, 1408), (4096, 7808)])
 def test_skinny_rows_do_not_depend_on_the_batch(hip, fmt, N, K):
     # engine/cuda/kernels.h:466-471: M = 1, 2, 8, 16, 32, 64 and across chunks of 64.
     w = random_weight(FORMATS[fmt], N, K, N + K).to("cuda")
