@@ -1212,7 +1212,7 @@ bool try_walk(const GemmArgs& a, int* status, hipStream_t stream) {
     // (bf16, K >= 8192) win once the batch is large, where the tile kernels' activation reads grow with every row tile:
     // 8192 x 8192 fp8 at 32 / 64 rows 28.4 -> 24.6 / 50.4 -> 39.4 us, bf16 40.6 -> 36.7 / 58.8 -> 43.4 us, 14336 x 4096 bf16
     // at 64 rows 39.3 -> 35.3 us, 14336 x 8192 fp8 at 48 rows 47.5 -> 41.6 us. Few tiles (4096 rows) stay with the tile kernels.
-    const int walk_groups = a.steps >> 2;
+    const int walk_groups = (a.steps + 3) >> 2;
     if (a.M <= 8 || n_tiles < 192) return false;
     if (walk_groups > 16) {
       if (n_tiles < 512 || walk_groups > 64) return false;
@@ -1246,9 +1246,9 @@ bool launch_walk_parts(GemmArgs a, int* status, hipStream_t stream) {
   if (spw < 8 || spw % 8 != 0) return false;
   const int slices = (a.steps + spw - 1) / spw, gps = spw >> 2;
   if (slices < 2 || slices > a.S) return false;
-  // A walk is groups in fours: two slices to a workgroup where one is not (then the row must be whole slices).
+  // A walk is groups in fours: two slices to a workgroup where one is not (the launcher then wants whole slices in pairs,
+  // or rows for its kernels that fill a walk up).
   const int per_wg = gps % 4 == 0 ? 1 : 2;
-  if (per_wg == 2 && (a.steps % spw != 0 || slices % 2 != 0)) return false;
   const int n_tiles = (a.N + kTileRows - 1) / kTileRows, mts = (a.M + 15) / 16;
   void* const partial = slab_scratch(stream, sizeof(float) * 4 * kWave * mts * n_tiles * slices);
   if (!partial) return false;

@@ -56,9 +56,14 @@ template <int F>
 constexpr int stage_bytes() {
   return F == LX_W_NVFP4 ? 4096 + 16 * kScalePitch : 4096;
 }
-template <int F, int MT, int W, int MODE>
+// RAGGED (kPlain and kPart): rows that are not whole walks, that is, whose load steps are not a multiple of 16 or whose
+// last step is cut short by K. A walk still runs in fours of groups: past the row's end the loads are clamped to the row's
+// last 16 bytes (weights, block scales and activations alike) and the activation pieces from K on are zeroed on their way
+// into the image, so the groups and chunks that are not there add zeros to the row's last slice.
+template <int F, int MT, int W, int MODE, bool RAGGED = false>
 __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   constexpr bool ROT = MODE == kRot, PART = MODE == kPart, SPLIT = MODE == kSplit;
+  static_assert(!RAGGED || MODE == kPlain || MODE == kPart, "rows that are not whole walks: from the row's start, or single slices");
   extern __shared__ __align__(16) f32x4 lds4[];
   constexpr int E = Fmt<F>::kElems, J = E / 8;
   constexpr int PB = 4 * J;          // 16-byte pieces of an image row under one load step
@@ -77,14 +82,15 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   uint8_t* const stage = lds + wave * kStage;
   uint8_t* const img = lds + W * kStage + (SPLIT ? wave * 2 * kImage : 0);  // + buffer * kImage
   const int gps = a.steps_per_wave >> 2;  // groups of four load steps in a slice (the row's last slice may be shorter)
-  const int row_groups = a.steps >> 2;    // and in a row
+  const int row_groups = RAGGED ? (a.steps + 3) >> 2 : a.steps >> 2;  // and in a row
   const int slices = (row_groups + gps - 1) / gps;  // the slices that hold steps (a.S may count empty ones behind them: their sums are zero)
   const int first_slice = ROT ? blockIdx.x % slices : PART ? blockIdx.y * a.walk_slices : SPLIT ? wave * a.walk_slices : 0, rot = first_slice * gps;
-  const int groups = PART || SPLIT ? min(a.walk_slices * gps, row_groups - rot) : row_groups, last = groups - 1;  // the groups this wavefront walks
+  const int real_groups = PART || SPLIT ? min(a.walk_slices * gps, row_groups - rot) : row_groups;
+  const int groups = RAGGED ? (real_groups + 3) & ~3 : real_groups, last = groups - 1;  // the groups this wavefront walks
   // The l-th group this wavefront takes (l past the end repeats the last one).
   auto group_of = [&](int l) {
     const int gq = min(l, last) + rot;
-    return !PART && !SPLIT && gq >= row_groups ? gq - row_groups : gq;
+    return ROT && gq >= row_groups ? gq - row_groups : gq;  // kRot goes round; RAGGED: groups past the row's end hold nothing
   };
 
   // Staging: item idx = (tile of rows * 4 + step of the window) * J + quad of pieces; wavefront tw takes
@@ -99,26 +105,46 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   const uint32_t ld_bytes = static_cast<uint32_t>(a.xs.ld) * 2u;
   uint32_t x_off[Q];  // byte offset of this lane's piece of item `it` within window 0
   uint32_t x_lds[J == 2 ? Q : 1];  // J == 2: where it goes in an image
+  // RAGGED: the window offset up to which the piece lies inside the row (beyond: the row's last piece, and zeros).
+  uint32_t x_lim[RAGGED ? Q : 1];
+  const uint32_t k_bytes = static_cast<uint32_t>(a.K) * 2u;
 #pragma unroll
   for (int it = 0; it < Q; ++it) {
     const int idx = tw + it * WS;
+    uint32_t k_off;
     if constexpr (J == 2) {
       const int h = idx & 1, u = (idx >> 1) & 3, mt = idx >> 3;
       const int row = 8 * h + (i >> 1), piece = 2 * g + (i & 1);
-      x_off[it] = static_cast<uint32_t>(min(16 * mt + row, a.M - 1)) * ld_bytes + static_cast<uint32_t>(u * 4 * E + piece * 8) * 2u;
+      k_off = static_cast<uint32_t>(u * 4 * E + piece * 8) * 2u;
+      x_off[it] = static_cast<uint32_t>(min(16 * mt + row, a.M - 1)) * ld_bytes + k_off;
       x_lds[it] = static_cast<uint32_t>(((mt * 4 + u) * PB + piece) * 256 + ((row + 8 * (piece & 1)) & 15) * 16);
     } else {
       const int pq = idx & (J - 1), u = (idx / J) & 3, mt = idx / (4 * J);
-      x_off[it] = static_cast<uint32_t>(min(16 * mt + r, a.M - 1)) * ld_bytes + static_cast<uint32_t>(u * 4 * E + pq * 32 + e3 * 8) * 2u;
+      k_off = static_cast<uint32_t>(u * 4 * E + pq * 32 + e3 * 8) * 2u;
+      x_off[it] = static_cast<uint32_t>(min(16 * mt + r, a.M - 1)) * ld_bytes + k_off;
     }
+    if constexpr (RAGGED) x_lim[it] = k_bytes - 16u - k_off;  // the launcher sees to K >= a window
   }
   u32x4 xr[2][Q];  // two windows on their way
   auto stage_load = [&](auto set, int gamma) {
-    const char* const src = xbase + static_cast<uint32_t>(group_of(gamma)) * (16u * E * 2u);  // a window is 16 E values of k
+    const uint32_t at_k = static_cast<uint32_t>(group_of(gamma)) * (16u * E * 2u);  // a window is 16 E values of k
+    const char* const src = xbase + at_k;
 #pragma unroll
-    for (int it = 0; it < Q; ++it) xr[decltype(set)::value][it] = *reinterpret_cast<const u32x4*>(src + x_off[it]);
+    for (int it = 0; it < Q; ++it) {
+      if constexpr (RAGGED) xr[decltype(set)::value][it] = *reinterpret_cast<const u32x4*>(xbase + (x_off[it] + min(at_k, x_lim[it])));
+      else xr[decltype(set)::value][it] = *reinterpret_cast<const u32x4*>(src + x_off[it]);
+    }
   };
   auto stage_store = [&](auto set, int gamma) {
+    if constexpr (RAGGED) {
+      // A window that reaches past K (no load is asked for in here: the wait counts stay what they are).
+      const uint32_t at_k = static_cast<uint32_t>(group_of(gamma)) * (16u * E * 2u);
+      if (at_k + 16u * E * 2u > k_bytes) {
+#pragma unroll
+        for (int it = 0; it < Q; ++it)
+          if (at_k > x_lim[it]) xr[decltype(set)::value][it] = u32x4{0u, 0u, 0u, 0u};
+      }
+    }
     if constexpr (J == 2) {
       uint8_t* const dst = img + (gamma & 1) * kImage;
 #pragma unroll
@@ -135,7 +161,7 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   const uint8_t* const own_scale = a.scale + (static_cast<int64_t>(n0) + min(i, valid - 1)) * a.scale_row_bytes;  // NVFP4 only
   uint32_t row_off[4];
 #pragma unroll
-  for (int q = 0; q < 4; ++q) row_off[q] = static_cast<uint32_t>(min(4 * q + g, valid - 1)) * static_cast<uint32_t>(a.row_bytes) + i * 16u;
+  for (int q = 0; q < 4; ++q) row_off[q] = static_cast<uint32_t>(min(4 * q + g, valid - 1)) * static_cast<uint32_t>(a.row_bytes) + (RAGGED ? 0u : i * 16u);
   u32x4 raw[4][4];
   // NVFP4: a group's block scales of the lane's row i, the eight bytes under piece group g (one load a group and lane,
   // 32 contiguous bytes a row; a lane's fragments need bytes 8 u + 2 g, 8 u + 2 g + 1 of the row's 32 for step u, which
@@ -144,10 +170,14 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
   auto issue_group = [&](auto slot, int gamma) {
     constexpr int SL = decltype(slot)::value;
     const int gq = group_of(gamma);
-    const uint32_t c = static_cast<uint32_t>(gq) * 256u;  // a group is 256 bytes of a row
+    // A group is 256 bytes of a row (RAGGED: the lane's chunk, or the row's last one).
+    const uint32_t c = RAGGED ? min(static_cast<uint32_t>(gq) * 256u + i * 16u, static_cast<uint32_t>(a.row_bytes) - 16u) : static_cast<uint32_t>(gq) * 256u;
 #pragma unroll
     for (int q = 0; q < 4; ++q) raw[SL][q] = __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(tile_w + (row_off[q] + c)));
-    if constexpr (F == LX_W_NVFP4) sc[SL] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(own_scale + 32 * gq + 8 * g));
+    if constexpr (F == LX_W_NVFP4) {
+      const uint32_t sc_at = RAGGED ? min(32u * gq + 8u * g, static_cast<uint32_t>(a.scale_row_bytes) - 8u) : 32u * gq + 8u * g;
+      sc[SL] = __builtin_nontemporal_load(reinterpret_cast<const u32x2*>(own_scale + sc_at));
+    }
   };
   // Row 4 q + g, chunk i goes into the wavefront's image; row i, chunk 4 s + g comes out.
   uint32_t put_at[4], get_at[4];
@@ -278,8 +308,10 @@ __global__ void __launch_bounds__(W* kWave) walk_kernel(const GemmArgs a) {
         } else total[mt] = slice == 0 ? acc[mt] : total[mt] + acc[mt];
         acc[mt] = f32x4{0.f, 0.f, 0.f, 0.f};
       }
-      if (at == row_groups) at = 0, slice = 0, slice_end = min(gps, row_groups);  // round to the row's start
-      else ++slice, slice_end = min(slice_end + gps, row_groups);
+      if (at == row_groups) {
+        if constexpr (RAGGED) slice_end = -1;  // what follows holds nothing: no slice ends again
+        else at = 0, slice = 0, slice_end = min(gps, row_groups);  // round to the row's start
+      } else ++slice, slice_end = min(slice_end + gps, row_groups);
     }
   };
   for (int gamma = 0; gamma < groups - 4; gamma += 4) {
@@ -378,11 +410,14 @@ int launch_split(const GemmArgs& a, hipStream_t stream) {
   }
 }
 
+// ragged: rows that are not whole walks (the RAGGED kernels: from the row's start with the sums in registers, or single
+// slices; no split over a workgroup's wavefronts).
 template <int F, int W>
-int launch_w(const GemmArgs& a, unsigned grid, hipStream_t stream) {
+int launch_w(const GemmArgs& a, unsigned grid, bool ragged, hipStream_t stream) {
   constexpr int J = Fmt<F>::kElems / 8, PB = 4 * J;
   const int MT = (a.M + 15) / 16;
   if (a.walk_split) {
+    if (ragged) return kNotSupported;
     if constexpr (W == 2 || W == 4) return launch_split<F, W>(a, stream);
     else return kNotSupported;
   }
@@ -394,15 +429,17 @@ int launch_w(const GemmArgs& a, unsigned grid, hipStream_t stream) {
   const size_t images = static_cast<size_t>(W) * stage_bytes<F>() + 2 * static_cast<size_t>(MT) * 4 * PB * 256;
   const size_t with_sums = images + static_cast<size_t>(W) * a.S * MT * kWave * 16;
   const bool part = a.partial != nullptr;
-  const bool rot = !part && with_sums <= kLdsMax;
+  const bool rot = !part && !ragged && with_sums <= kLdsMax;
   const size_t lds = rot ? with_sums : images;
   if (lds > kLdsMax) return kNotSupported;
   unsigned parts = 1;
   if (part) {
     // Whole slices to a workgroup, their groups in fours.
     const int gps = a.steps_per_wave >> 2, slices = (a.steps + a.steps_per_wave - 1) / a.steps_per_wave;
-    const bool ragged = a.steps % a.steps_per_wave != 0;
-    if (a.walk_slices < 1 || (a.walk_slices * gps) % 4 != 0 || (ragged ? gps % 4 != 0 : slices % a.walk_slices != 0)) return kNotSupported;
+    // (A short last slice is whole fours of groups when every slice is; the RAGGED kernels fill the last workgroup's walk up.)
+    const bool short_last = a.steps % a.steps_per_wave != 0;
+    if (a.walk_slices < 1 || (a.walk_slices * gps) % 4 != 0) return kNotSupported;
+    if (!ragged && (short_last ? gps % 4 != 0 : slices % a.walk_slices != 0)) return kNotSupported;
     parts = static_cast<unsigned>((slices + a.walk_slices - 1) / a.walk_slices);
   }
   auto launch = [&](auto kernel) {
@@ -413,11 +450,14 @@ int launch_w(const GemmArgs& a, unsigned grid, hipStream_t stream) {
   auto with_mt = [&](auto mt_tag) {
     constexpr int M16 = decltype(mt_tag)::value;
     if constexpr (M16 * 4 * J % W != 0) return static_cast<int>(kNotSupported);
-    else if constexpr (W == 8) return part ? launch(walk_kernel<F, M16, W, kPart>) : static_cast<int>(kNotSupported);
-    else if (part) {
-      if constexpr (W == 4) return launch(walk_kernel<F, M16, W, kPart>);
+    else if constexpr (W == 8) {
+      if (!part) return static_cast<int>(kNotSupported);
+      return ragged ? launch(walk_kernel<F, M16, W, kPart, true>) : launch(walk_kernel<F, M16, W, kPart>);
+    } else if (part) {
+      if constexpr (W == 4) return ragged ? launch(walk_kernel<F, M16, W, kPart, true>) : launch(walk_kernel<F, M16, W, kPart>);
       else return static_cast<int>(kNotSupported);
-    } else return rot ? launch(walk_kernel<F, M16, W, kRot>) : launch(walk_kernel<F, M16, W, kPlain>);
+    } else if (ragged) return launch(walk_kernel<F, M16, W, kPlain, true>);
+    else return rot ? launch(walk_kernel<F, M16, W, kRot>) : launch(walk_kernel<F, M16, W, kPlain>);
   };
   switch (MT) {
     case 1: return with_mt(Tag<1>{});
@@ -433,8 +473,12 @@ bool launch_format(const GemmArgs& a, int W, int* status, hipStream_t stream) {
   const int S = a.S, spw = a.steps_per_wave;
   if (a.M < 1 || a.M > 64 || S < 1 || spw % 8 != 0) return false;
   // Slices of whole batches, the row's last one as long as the row reaches (S may count empty ones behind it: a zero
-  // added last changes no sum), and groups in fours.
-  if ((a.steps + spw - 1) / spw > S || static_cast<int64_t>(a.steps) * 4 * E != a.K || a.steps % 16 != 0) return false;
+  // added last changes no sum). Rows that are not groups in fours of whole steps take the RAGGED kernels: at least one
+  // walk of four groups long, and NVFP4 in whole steps (a step's block scales are read as one).
+  if ((a.steps + spw - 1) / spw > S) return false;
+  const bool whole_steps = static_cast<int64_t>(a.steps) * 4 * E == a.K;
+  const bool ragged = !whole_steps || a.steps % 16 != 0;
+  if (ragged && (a.steps < 16 || (F == LX_W_NVFP4 && !whole_steps) || a.K % E != 0)) return false;
   if (static_cast<int64_t>(a.M) * a.xs.ld * 2 + static_cast<int64_t>(a.K) * 2 >= (int64_t{1} << 31)) return false;
   if (static_cast<int64_t>(kTileRows) * a.row_bytes >= (int64_t{1} << 31)) return false;
   // NVFP4: a group's scales are read eight bytes at a time.
@@ -443,10 +487,10 @@ bool launch_format(const GemmArgs& a, int W, int* status, hipStream_t stream) {
   const unsigned grid = static_cast<unsigned>((n_tiles + W - 1) / W);
   int st;
   switch (W) {
-    case 8: st = launch_w<F, 8>(a, grid, stream); break;
-    case 4: st = launch_w<F, 4>(a, grid, stream); break;
-    case 2: st = launch_w<F, 2>(a, grid, stream); break;
-    case 1: st = launch_w<F, 1>(a, grid, stream); break;
+    case 8: st = launch_w<F, 8>(a, grid, ragged, stream); break;
+    case 4: st = launch_w<F, 4>(a, grid, ragged, stream); break;
+    case 2: st = launch_w<F, 2>(a, grid, ragged, stream); break;
+    case 1: st = launch_w<F, 1>(a, grid, ragged, stream); break;
     default: return false;
   }
   if (st == kNotSupported) return false;

@@ -62,6 +62,32 @@ def test_every_variant_gives_the_same_bits(hip, fmt, M):
             assert torch.equal(out.view(torch.int32), outs[0].view(torch.int32)), f"variant {variant} changes bits at {fmt} {N}x{K} M={M}"
 
 
+# Rows that are not whole walks: load steps that are not a multiple of 16 (11 and 21.5 groups of four), a last step cut
+# short by K (bf16 43.25 steps, one-byte formats 22.25), an activation matrix whose last row ends where the allocation ends.
+RAGGED = {"bf16": [(150, 1408), (2048, 1384)], "int8": [(150, 1408), (2048, 5504), (300, 1424)],
+          "fp8": [(150, 1408), (2048, 5504), (300, 1424)], "nvfp4": [(150, 2688), (2048, 5504)]}
+
+
+@pytest.mark.parametrize("M", [9, 16, 33, 64])
+@pytest.mark.parametrize("fmt", FMT)
+def test_rows_that_are_not_whole_walks(hip, fmt, M):
+    for N, K in RAGGED[fmt]:
+        g = torch.Generator().manual_seed(M + N)
+        w = random_weight(FORMATS[fmt], N, K, N + K)
+        x = torch.randn(M, K, generator=g).to(torch.bfloat16)
+        bias = torch.randn(N, generator=g)
+        want = ops.gemv_reference(x, w.dense(), bias, 1.0, 0.0, None)
+        wd, xd, bd = w.to("cuda"), x.cuda(), bias.cuda()
+        outs = {}
+        for variant in (0, 1, 2, 3, 6, 7, None):
+            force(hip, fmt, M, N, K, variant)
+            y = torch.full((M, N), float("nan"), device="cuda")
+            outs[variant] = ops.gemm_w(hip, xd, wd, MATH_BF16, bias=bd, y=y).clone()
+        checks.check_product(outs[0].cpu(), want)
+        for variant, out in outs.items():
+            assert torch.equal(out.view(torch.int32), outs[0].view(torch.int32)), f"variant {variant} changes bits at {fmt} {N}x{K} M={M}"
+
+
 @pytest.mark.parametrize("fmt", FMT)
 def test_walk_rows_do_not_depend_on_the_batch(hip, fmt):
     N, K = SHAPES[fmt][1]
