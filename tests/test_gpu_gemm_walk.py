@@ -14,7 +14,7 @@ from dromos_amd.formats import random_weight
 
 pytestmark = pytest.mark.gpu
 FMT = checks.FMT_NAMES
-# K whose rows are whole slices of whole four-group walks in the format (the shapes the kernel takes), N with a ragged last tile
+# K whose rows are whole slices of whole four-group walks in the format (what the kernel takes without its clamps), N with a ragged last tile
 SHAPES = {"bf16": [(150, 512), (4096, 1024)], "int8": [(150, 1024), (4096, 2048)], "fp8": [(150, 1024), (4096, 4096)], "nvfp4": [(150, 2048), (4096, 4096)]}
 
 
@@ -62,8 +62,8 @@ def test_every_variant_gives_the_same_bits(hip, fmt, M):
             assert torch.equal(out.view(torch.int32), outs[0].view(torch.int32)), f"variant {variant} changes bits at {fmt} {N}x{K} M={M}"
 
 
-# Rows that are not whole walks: load steps that are not a multiple of 16 (11 and 21.5 groups of four), a last step cut
-# short by K (bf16 43.25 steps, one-byte formats 22.25), an activation matrix whose last row ends where the allocation ends.
+# Rows that are not whole walks: load steps that are not a multiple of 16 (11 and 21.5 groups of four) and a last step
+# cut short by K (bf16 43.25 steps, one-byte formats 22.25).
 RAGGED = {"bf16": [(150, 1408), (2048, 1384)], "int8": [(150, 1408), (2048, 5504), (300, 1424)],
           "fp8": [(150, 1408), (2048, 5504), (300, 1424)], "nvfp4": [(150, 2688), (2048, 5504)]}
 
