@@ -1320,8 +1320,15 @@ bool walk_parts_wanted(int M, int n_tiles, int64_t K, int tuned) {
     if (n_tiles >= 768) return false;
     return mts >= 3 || (mts == 2 && K >= 8192) || K >= 14336;
   }
-  if (mts >= 3) return K >= 8192;
-  return K >= 28672 || (K >= 14336 && n_tiles <= 256);
+  // Rows of 5120 .. 7168 values (bf16 from 6144) on at most 384 tiles, where neither the whole walks nor the tile kernels
+  // fill the device: 5120 x 5120 fp8 at 32 / 48 / 64 rows 19.2 / 23.8 / 27.1 -> 13 / 15 / 17 us, 6144 x 7168 23.3 / 32.6 / 39.0
+  // -> 17.5 / 20 / 23, 4096 x 6144 at 48 / 64 rows 20.3 / 23.3 -> 15 / 16.5, bf16 6144 x 6144 24.0 / 29.6 / 33.0 -> 21 / 26 / 27
+  // (at worst a tie: 6144 x 5120, and 6144 x 6144 one-byte at 32 rows 5 % behind); at 17 .. 32 rows 4096-row matrices
+  // stay with the split walk and the slab kernel, which tie.
+  const int64_t mid_k = F == LX_W_BF16 ? 6144 : 5120;
+  if (mts >= 3) return K >= 8192 || (K >= mid_k && n_tiles <= 384);
+  if (K >= 28672 || (K >= 14336 && n_tiles <= 256)) return true;
+  return K >= mid_k && K < 8192 && n_tiles > 256 && n_tiles <= 384;
 }
 
 template <int F, int MT>
