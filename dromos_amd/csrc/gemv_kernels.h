@@ -307,6 +307,10 @@ int launch_stream(GemvArgs a, const Shape& shape, hipStream_t stream) {
 template <int F, int MT, bool XB>
 int launch_rows(const GemvArgs& a, const Shape& shape, hipStream_t stream) {
   if constexpr (MT == 1) {
+    // Rows of five or six steps (K = 5120, 6144 of one-byte weights) are asked for whole, like those of seven below: as
+    // batches of two steps they would be three round trips, as a batch of eight a third of the loads would be repeats.
+    if (a.split == 1 && a.steps == 5) return launch_stream<F, MT, 1, 5, XB>(a, shape, stream);
+    if (a.split == 1 && a.steps == 6) return launch_stream<F, MT, 1, 6, XB>(a, shape, stream);
     switch (shape.depth) {
       case 8:
         // Rows of exactly seven steps (K = 14336 in NVFP4) are asked for whole, without an eighth, repeated load.
