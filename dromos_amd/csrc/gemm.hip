@@ -1316,9 +1316,10 @@ bool walk_parts_wanted(int M, int n_tiles, int64_t K, int tuned) {
   if (F == LX_W_NVFP4) {
     // With many tiles the whole walk of four tiles a workgroup is ahead at every row count (14336 x 4096 at 48 rows
     // 32.8 -> 25.5 us); below that the single slices from 33 rows, from 17 rows for K >= 8192, from 9 for K >= 14336
-    // (8192 x 14336 at 16 rows 38.0 -> 29.5 us).
+    // (8192 x 14336 at 16 rows 38.0 -> 29.5 us); K >= 11008 since the walks take rows that are not whole walks (at 16 rows
+    // 9216 x 11008 39.7 -> 30 us, 11008 x 11008 40.5 -> 32, 5120 x 13824 33.4 -> 27; a tie on 4096 and 8192 x 11008).
     if (n_tiles >= 768) return false;
-    return mts >= 3 || (mts == 2 && K >= 8192) || K >= 14336;
+    return mts >= 3 || (mts == 2 && K >= 8192) || K >= 11008;
   }
   // Rows of 5120 .. 7168 values (bf16 from 6144) on at most 384 tiles, where neither the whole walks nor the tile kernels
   // fill the device: 5120 x 5120 fp8 at 32 / 48 / 64 rows 19.2 / 23.8 / 27.1 -> 13 / 15 / 17 us, 6144 x 7168 23.3 / 32.6 / 39.0
