@@ -1222,7 +1222,11 @@ bool try_walk(const GemmArgs& a, int* status, hipStream_t stream) {
       const bool long_walks = n_tiles >= 768 && (F == LX_W_NVFP4 || (F != LX_W_BF16 && walk_groups > 32));
       if (!long_walks && a.M <= (n_tiles >= 768 ? 32 + 8 : 24)) return false;
     }
-    W = n_tiles >= (walk_groups <= 16 ? 512 : 768) ? 4 : 2;
+    // (Rows that are not whole walks start every workgroup at the row's start, and four tiles a workgroup are ahead from
+    // 576 tiles: at 32 rows fp8 9216 x 11008 40.2 -> 32.6 us, 11008 x 11008 41.1 -> 34.4, 11008 x 13824 49.9 -> 40.2; on the
+    // 512 tiles of 8192 x 11008 two are: 28.1 against 31.9.)
+    const bool whole_walks = a.steps % 16 == 0 && static_cast<int64_t>(a.steps) * 4 * Fmt<F>::kElems == a.K;
+    W = n_tiles >= (walk_groups <= 16 ? 512 : whole_walks ? 768 : 576) ? 4 : 2;
   }
   auto launch = [&](int w) {
     if constexpr (F == LX_W_BF16) return launch_walk_bf16(a, w, status, stream);
