@@ -64,8 +64,9 @@ def test_every_variant_gives_the_same_bits(hip, fmt, M):
 
 # Rows that are not whole walks: load steps that are not a multiple of 16 (11 and 21.5 groups of four) and a last step
 # cut short by K (bf16 43.25 steps, one-byte formats 22.25).
-RAGGED = {"bf16": [(150, 1408), (2048, 1384)], "int8": [(150, 1408), (2048, 5504), (300, 1424)],
-          "fp8": [(150, 1408), (2048, 5504), (300, 1424)], "nvfp4": [(150, 2688), (2048, 5504)]}
+# The last of each: a quarter of a step (NVFP4: one step) past 16, so that three of the walk's last four groups hold nothing.
+RAGGED = {"bf16": [(150, 1408), (2048, 1384), (300, 520)], "int8": [(150, 1408), (2048, 5504), (300, 1424), (300, 1040)],
+          "fp8": [(150, 1408), (2048, 5504), (300, 1424), (300, 1040)], "nvfp4": [(150, 2688), (2048, 5504), (300, 2176)]}
 
 
 @pytest.mark.parametrize("M", [9, 16, 33, 64])
