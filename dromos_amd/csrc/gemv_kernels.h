@@ -311,6 +311,16 @@ int launch_rows(const GemvArgs& a, const Shape& shape, hipStream_t stream) {
     // batches of two steps they would be three round trips, as a batch of eight a third of the loads would be repeats.
     if (a.split == 1 && a.steps == 5) return launch_stream<F, MT, 1, 5, XB>(a, shape, stream);
     if (a.split == 1 && a.steps == 6) return launch_stream<F, MT, 1, 6, XB>(a, shape, stream);
+    // Rows of 9 .. 14 steps in two even batches of one row (they were 4 + 4 + x of two rows, or 8 + x): 4096 rows of 9216 ..
+    // 14336 one-byte values 8.7 .. 11.6 -> 8.2 .. 11.3 us, bf16 11008 x 4608 .. 7168 18.4 .. 25.0 -> 16.3 .. 24.4 (one-byte
+    // 11008 x 9216 / 10240 lose 4 - 6 %).
+    if (a.split == 1 && a.steps >= 9 && a.steps <= 14) {
+      switch ((a.steps + 1) / 2) {
+        case 5: return launch_stream<F, MT, 1, 5, XB>(a, shape, stream);
+        case 6: return launch_stream<F, MT, 1, 6, XB>(a, shape, stream);
+        default: return launch_stream<F, MT, 1, 7, XB>(a, shape, stream);
+      }
+    }
     switch (shape.depth) {
       case 8:
         // Rows of exactly seven steps (K = 14336 in NVFP4) are asked for whole, without an eighth, repeated load.

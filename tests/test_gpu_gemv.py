@@ -17,10 +17,11 @@ from dromos_amd.formats import Weight, master_weight, quantize_with, random_weig
 
 pytestmark = pytest.mark.gpu
 FMT = checks.FMT_NAMES
-# The last six: rows of exactly five and six load steps in one format or another (bf16 2560 / 3072, one-byte 5120 / 6144,
-# NVFP4 10240 / 12288), which a single activation row asks for whole.
+# From (1024, 2560) on: rows of exactly five and six load steps in one format or another (bf16 2560 / 3072, one-byte 5120 /
+# 6144, NVFP4 10240 / 12288), which a single activation row asks for whole, and rows of 9 .. 14 steps (two even batches:
+# one-byte 10240 / 11008 / 12288, bf16 5120 / 6144, NVFP4 18432).
 SHAPES = [(10304, 2048), (2048, 4096), (3072, 2048), (1024, 512), (256, 2048), (256, 6400), (8, 2048),
-          (1024, 2560), (1024, 3072), (1024, 5120), (1024, 6144), (1024, 10240), (1024, 12288)]
+          (1024, 2560), (1024, 3072), (1024, 5120), (1024, 6144), (1024, 10240), (1024, 12288), (1024, 18432), (1024, 11008)]
 
 
 @pytest.mark.parametrize("K", [48, 528, 2048])
