@@ -1325,8 +1325,10 @@ bool walk_parts_wanted(int M, int n_tiles, int64_t K, int tuned) {
     // 32.8 -> 25.5 us); below that the single slices from 33 rows, from 17 rows for K >= 8192, from 9 for K >= 14336
     // (8192 x 14336 at 16 rows 38.0 -> 29.5 us); K >= 11008 since the walks take rows that are not whole walks (at 16 rows
     // 9216 x 11008 39.7 -> 30 us, 11008 x 11008 40.5 -> 32, 5120 x 13824 33.4 -> 27; a tie on 4096 and 8192 x 11008).
+    // With four tiles a workgroup up to 16 rows they are also ahead there on 257 .. 512 tiles from K = 5120 (at 16 rows
+    // 5120 x 5120 16.4 -> 11.9 us, 6144 x 7168 20.4 -> 15.8, 8192 x 8192 21.6 -> 17.7; on 576 tiles and more the whole walk is).
     if (n_tiles >= 768) return false;
-    return mts >= 3 || (mts == 2 && K >= 8192) || K >= 11008;
+    return mts >= 3 || (mts == 2 && K >= 8192) || K >= 11008 || (mts == 1 && K >= 5120 && n_tiles > 256 && n_tiles <= 512);
   }
   // Rows of 5120 .. 7168 values (bf16 from 6144) on at most 384 tiles, where neither the whole walks nor the tile kernels
   // fill the device: 5120 x 5120 fp8 at 32 / 48 / 64 rows 19.2 / 23.8 / 27.1 -> 13 / 15 / 17 us, 6144 x 7168 23.3 / 32.6 / 39.0
@@ -1336,6 +1338,8 @@ bool walk_parts_wanted(int M, int n_tiles, int64_t K, int tuned) {
   const int64_t mid_k = F == LX_W_BF16 ? 6144 : 5120;
   if (mts >= 3) return K >= 8192 || (K >= mid_k && n_tiles <= 384);
   if (K >= 28672 || (K >= 14336 && n_tiles <= 256)) return true;
+  // (Up to 16 rows of one-byte weights also K >= 13824 on at most 512 tiles: 8192 x 14336 fp8 27.6 -> 24.5 us, 5120 x 13824 25.1 -> 20.7.)
+  if (mts == 1 && F != LX_W_BF16 && K >= 13824 && n_tiles <= 512) return true;
   return K >= mid_k && K < 8192 && n_tiles > 256 && n_tiles <= 384;
 }
 
