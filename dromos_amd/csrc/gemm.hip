@@ -1220,7 +1220,11 @@ bool try_walk(const GemmArgs& a, int* status, hipStream_t stream) {
       // (14336 x 14336 fp8 at 16 / 32 rows: 46.0 / 58.8 -> 41.0 / 51.3 us) and on NVFP4, whose values are twice as many
       // per byte (16384 x 14336 at 16 rows 55.5 -> 41.1 us, 14336 x 8192 at 48 rows 49.6 -> 41.2).
       const bool long_walks = n_tiles >= 768 && (F == LX_W_NVFP4 || (F != LX_W_BF16 && walk_groups > 32));
-      if (!long_walks && a.M <= (n_tiles >= 768 ? 32 + 8 : 24)) return false;
+      // Below 768 tiles from 25 rows; the one-byte formats and NVFP4 from 17 rows on walks of more than 32 groups or fewer than
+      // 576 tiles (at 17 .. 24 rows fp8 8192 x 14336 38.7 -> 32.4 us, 9216 x 11008 39.6 -> 31.3, 8192 x 8192 24.4 -> 21.2; with 32
+      // groups on 576 .. 688 tiles the windowed kernel stays 4 - 7 % ahead).
+      const int walk_from = n_tiles >= 768 ? 32 + 8 : F != LX_W_BF16 && (walk_groups > 32 || n_tiles < 576) ? 16 : 24;
+      if (!long_walks && a.M <= walk_from) return false;
     }
     // (Rows that are not whole walks start every workgroup at the row's start, and four tiles a workgroup are ahead from
     // 576 tiles: at 32 rows fp8 9216 x 11008 40.2 -> 32.6 us, 11008 x 11008 41.1 -> 34.4, 11008 x 13824 49.9 -> 40.2; on the
@@ -1326,9 +1330,10 @@ bool walk_parts_wanted(int M, int n_tiles, int64_t K, int tuned) {
     // (8192 x 14336 at 16 rows 38.0 -> 29.5 us); K >= 11008 since the walks take rows that are not whole walks (at 16 rows
     // 9216 x 11008 39.7 -> 30 us, 11008 x 11008 40.5 -> 32, 5120 x 13824 33.4 -> 27; a tie on 4096 and 8192 x 11008).
     // With four tiles a workgroup up to 16 rows they are also ahead there on 257 .. 512 tiles from K = 5120 (at 16 rows
-    // 5120 x 5120 16.4 -> 11.9 us, 6144 x 7168 20.4 -> 15.8, 8192 x 8192 21.6 -> 17.7; on 576 tiles and more the whole walk is).
+    // 5120 x 5120 16.4 -> 11.9 us, 6144 x 7168 20.4 -> 15.8, 8192 x 8192 21.6 -> 17.7; at 24 / 32 rows 6144 x 7168 25.3 -> 21; on 576
+    // tiles and more the whole walk is).
     if (n_tiles >= 768) return false;
-    return mts >= 3 || (mts == 2 && K >= 8192) || K >= 11008 || (mts == 1 && K >= 5120 && n_tiles > 256 && n_tiles <= 512);
+    return mts >= 3 || (mts == 2 && K >= 8192) || K >= 11008 || (K >= 5120 && n_tiles > 256 && n_tiles <= 512);
   }
   // Rows of 5120 .. 7168 values (bf16 from 6144) on at most 384 tiles, where neither the whole walks nor the tile kernels
   // fill the device: 5120 x 5120 fp8 at 32 / 48 / 64 rows 19.2 / 23.8 / 27.1 -> 13 / 15 / 17 us, 6144 x 7168 23.3 / 32.6 / 39.0
